@@ -1,0 +1,14 @@
+from .spec import PartSpec, LayerSpec, ScheduleEntry, ModelSpec, default_schedule
+from .registry import (Architecture, register_architecture, unregister_architecture,
+                       registered_architectures, architecture_of, architecture_of_config,
+                       read_config_json, config_from_dict, config_from_folder, spec_of)
+from .mistral import MistralConfig, PRESETS, preset, build_spec as build_mistral_spec, ARCHITECTURE as MISTRAL
+
+register_architecture(MISTRAL, MistralConfig, build_mistral_spec, model_type="mistral", replace=True)
+
+__all__ = [
+    "PartSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "default_schedule",
+    "Architecture", "register_architecture", "unregister_architecture", "registered_architectures",
+    "architecture_of", "architecture_of_config", "read_config_json", "config_from_dict",
+    "config_from_folder", "spec_of", "MistralConfig", "PRESETS", "preset",
+]

@@ -1,0 +1,90 @@
+"""The architecture-neutral description of a model: which parts, in which order.
+
+A configuration class (one per architecture, read from that architecture's own
+config.json keys) is turned into a `ModelSpec` by its architecture's builder.  The
+spec is plain data: part kinds are strings looked up in the part registries, sizes
+and constants are parameters, and the order in which layers run is a list.  Nothing
+below the spec knows which architecture it came from.
+
+The reference drives every architecture from one flat `ModelConfig` with a per-layer
+`LayerConfig{layer_type, ffn_type}` list (crates/braidinfer-runtime/src/config.rs:75-115,
+:9-37); the `(mixer kind, feed-forward kind)` pair per layer is kept, the flat struct
+is not.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A part by the name it is registered under, and its parameters."""
+
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+    def __hash__(self):
+        return hash((self.kind, tuple(sorted((k, repr(v)) for k, v in self.params.items()))))
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer: a mixer and a feed-forward, each behind its norm, arranged by `block`.
+
+    `mixer` or `feed_forward` may be None (a layer with only the other half, as the
+    reference's `LayerType::Ffn` / `FfnType::None`, config.rs:26-37).  `prefix` is the
+    tensor-name prefix of the layer's weights, e.g. ``model.layers.3.``.
+    """
+
+    prefix: str
+    mixer: Optional[PartSpec]
+    feed_forward: Optional[PartSpec]
+    mixer_norm: Optional[PartSpec]
+    ffn_norm: Optional[PartSpec]
+    block: str = "prenorm_residual"
+    # tensor-name pieces under `prefix` (the names of the architecture's checkpoints)
+    mixer_name: str = "self_attn."
+    feed_forward_name: str = "mlp."
+    mixer_norm_name: str = "input_layernorm."
+    ffn_norm_name: str = "post_attention_layernorm."
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    """One position of the run order.
+
+    `layer` indexes `ModelSpec.layers`; a layer may appear more than once (its weights
+    are then shared).  `cache` names the cache unit the mixer works on: entries with
+    the same `cache` see the same keys and values.  An entry with `writes_cache=False`
+    only reads what another entry wrote earlier in the same step.
+    """
+
+    layer: int
+    cache: Optional[int] = None
+    writes_cache: bool = True
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    architecture: str
+    hidden_size: int
+    vocab_size: int
+    embedding: PartSpec
+    layers: List[LayerSpec]
+    schedule: List[ScheduleEntry]
+    final_norm: PartSpec
+    lm_head: PartSpec
+    # position encodings by name; mixers refer to them by that name
+    positions: Dict[str, PartSpec]
+    max_position_embeddings: int
+    stop_token_ids: List[int] = field(default_factory=list)
+    bos_token_id: Optional[int] = None
+    embedding_prefix: str = "model.embed_tokens."
+    final_norm_prefix: str = "model.norm."
+    lm_head_prefix: str = "lm_head."
+
+
+def default_schedule(n_layers: int) -> List[ScheduleEntry]:
+    """Every layer once, in order, each with a cache unit of its own."""
+    return [ScheduleEntry(layer=i, cache=i) for i in range(n_layers)]

@@ -1,0 +1,229 @@
+// Row-wise and element-wise kernels of a decoder step: embedding gather, RMSNorm,
+// rotary tables, rotation + paged key/value write, SiLU*mul, residual add, row gather.
+// Activations are `T` (float in the 32-bit path, bf16 in the serving path); the
+// residual stream and all statistics are float in both.
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding ------
+// out[t, :] = float(table[token[t], :])            reference: op_embedding,
+// kernels/megakernel_ops.hip:1757-1768 (one instruction per token there; one launch
+// for all packed tokens here).  A token id outside the table writes zeros; the host
+// rejects such ids before the launch.
+template <typename W>
+__global__ void embedding_kernel(const W* __restrict__ table, const int* __restrict__ tokens,
+                                 float* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x;
+    const int tok = tokens[t];
+    float* o = out + (size_t)t * H;
+    if (tok < 0 || tok >= V) {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = 0.f;
+        return;
+    }
+    const W* r = table + (size_t)tok * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<W>(r[i]);
+}
+
+extern "C" int br_embedding(const void* table, int table_is_bf16, const int* tokens, float* out,
+                            int T, int H, int V, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (H <= 0 || V <= 0) return BR_BAD_ARG;
+    int threads = H >= 1024 ? 256 : 64;
+    if (table_is_bf16)
+        embedding_kernel<bf16><<<T, threads, 0, s>>>((const bf16*)table, tokens, out, H, V);
+    else
+        embedding_kernel<float><<<T, threads, 0, s>>>((const float*)table, tokens, out, H, V);
+    return br_check_launch();
+}
+
+// -------------------------------------------------------------------- RMSNorm ------
+// y = x * rsqrt(mean(x^2) + eps) * w, statistics in float       reference:
+// op_rmsnorm_wx, kernels/megakernel_ops.hip:862-904.  `rows` (optional) gathers:
+// y[i] = norm(x[rows[i]]).  One block per row; the sum of squares is reduced by a
+// fixed tree so a row's result does not depend on its neighbours.
+template <typename T>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               T* __restrict__ y, const int* __restrict__ rows, int H, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[r] : r) * H;
+    T* yr = y + (size_t)r * H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) { float v = xr[i]; ss += v * v; }
+    const float tot = block_sum(ss, scratch);
+    const float inv = rsqrtf(tot / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) yr[i] = from_f32<T>(xr[i] * inv * w[i]);
+}
+
+extern "C" int br_rmsnorm(const float* x, const float* w, void* y, int y_is_bf16, const int* rows,
+                          int R, int H, float eps, hipStream_t s) {
+    if (R <= 0) return BR_OK;
+    if (H <= 0) return BR_BAD_ARG;
+    int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
+    if (y_is_bf16)
+        rmsnorm_kernel<bf16><<<R, threads, 0, s>>>(x, w, (bf16*)y, rows, H, eps);
+    else
+        rmsnorm_kernel<float><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps);
+    return br_check_launch();
+}
+
+// --------------------------------------------------------------- rotary tables -----
+// cos/sin[t, p] of theta = float(pos[t]) * inv_freq[p]         reference: op_mrope,
+// kernels/megakernel_ops.hip:2019-2024 (cosf/sinf per element there; once per step
+// here, shared by all layers).
+__global__ void rope_table_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq,
+                                  float* __restrict__ cs, float* __restrict__ sn, int T, int P) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= T * P) return;
+    const int t = i / P, p = i - t * P;
+    const float th = (float)pos[t] * inv_freq[p];
+    cs[i] = cosf(th);
+    sn[i] = sinf(th);
+}
+
+extern "C" int br_rope_table(const int* pos, const float* inv_freq, float* cs, float* sn, int T, int P,
+                             hipStream_t s) {
+    if (T <= 0 || P <= 0) return BR_OK;
+    int n = T * P;
+    rope_table_kernel<<<(n + 255) / 256, 256, 0, s>>>(pos, inv_freq, cs, sn, T, P);
+    return br_check_launch();
+}
+
+// ------------------------------------------------- rotation + paged K/V write ------
+// For token t with query/key/value rows in `qkv` ([T, (nq + 2 nkv) * hd], q heads
+// first, then k heads, then v heads): rotate the first `rd` elements of every q and k
+// head by the token's angle (reference: op_mrope, megakernel_ops.hip:2025-2030; pair
+// (2p, 2p+1) when adjacent, (p, p + rd/2) when half), write q back in place, and store
+// the rotated k and the untouched v in the token's cache page (reference:
+// op_kv_write_paged_batch.hip:58-73 for the page/offset arithmetic; keys are stored
+// after rotation, once).  Cache layout per unit: [page][K|V][kv_head][token_in_page][hd].
+// A token whose sequence has slot < 0 is padding: q is still rotated, nothing is stored.
+// grid = (T, nq + 2 nkv), block = 64.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ cs,
+                                     const float* __restrict__ sn, const int* __restrict__ pos,
+                                     const int* __restrict__ seq_of_token, const int* __restrict__ slots,
+                                     const int* __restrict__ block_table, int table_stride,
+                                     T* __restrict__ cache, int nq, int nkv, int hd, int rd, int adjacent,
+                                     int page, int write_cache) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int width = (nq + 2 * nkv) * hd;
+    T* src = qkv + (size_t)t * width + (size_t)h * hd;
+    const bool is_q = h < nq, is_k = !is_q && h < nq + nkv;
+    T* dst = nullptr;
+    if (!is_q) {
+        if (!write_cache) return;
+        const int slot = slots[seq_of_token[t]];
+        if (slot < 0) return;
+        const int p = pos[t];
+        const int pg = block_table[(size_t)slot * table_stride + p / page];
+        const int kvh = is_k ? h - nq : h - nq - nkv;
+        dst = cache + ((((size_t)pg * 2 + (is_k ? 0 : 1)) * nkv + kvh) * page + (p % page)) * hd;
+    }
+    if (is_q || is_k) {
+        const int P = rd / 2;
+        const float* c = cs ? cs + (size_t)t * P : nullptr;
+        const float* s = sn ? sn + (size_t)t * P : nullptr;
+        T* o = is_q ? src : dst;
+        for (int p = threadIdx.x; p < P; p += blockDim.x) {
+            const int i0 = adjacent ? 2 * p : p, i1 = adjacent ? 2 * p + 1 : p + P;
+            const float a = to_f32<T>(src[i0]), b = to_f32<T>(src[i1]);
+            const float co = c ? c[p] : 1.f, si = s ? s[p] : 0.f;
+            o[i0] = from_f32<T>(a * co - b * si);
+            o[i1] = from_f32<T>(a * si + b * co);
+        }
+        if (is_k) for (int i = rd + threadIdx.x; i < hd; i += blockDim.x) o[i] = src[i];
+    } else {
+        for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+    }
+}
+
+extern "C" int br_rope_kv_write(void* qkv, int is_bf16, const float* cs, const float* sn, const int* pos,
+                                const int* seq_of_token, const int* slots, const int* block_table,
+                                int table_stride, void* cache, int T, int nq, int nkv, int hd, int rd,
+                                int adjacent, int page, int write_cache, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (nq <= 0 || nkv <= 0 || hd <= 0 || rd < 0 || rd > hd || (rd & 1) || page <= 0) return BR_BAD_ARG;
+    dim3 grid(T, nq + 2 * nkv);
+    if (is_bf16)
+        rope_kv_write_kernel<bf16><<<grid, 64, 0, s>>>((bf16*)qkv, cs, sn, pos, seq_of_token, slots,
+                                                       block_table, table_stride, (bf16*)cache, nq, nkv,
+                                                       hd, rd, adjacent, page, write_cache);
+    else
+        rope_kv_write_kernel<float><<<grid, 64, 0, s>>>((float*)qkv, cs, sn, pos, seq_of_token, slots,
+                                                        block_table, table_stride, (float*)cache, nq, nkv,
+                                                        hd, rd, adjacent, page, write_cache);
+    return br_check_launch();
+}
+
+// ------------------------------------------------------------------ SiLU * mul -----
+// a[t, i] = silu(g[t, i]) * u[t, i], silu(x) = x / (1 + exp(-x)), from the fused
+// gate/up output gu[t, 0:I] = g, gu[t, I:2I] = u       reference: op_silu_mul,
+// kernels/megakernel_ops.hip:374-407.
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ a, int I, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    size_t t = i / I, c = i - t * I;
+    float g = to_f32<T>(gu[t * 2 * I + c]), u = to_f32<T>(gu[t * 2 * I + I + c]);
+    a[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int br_silu_mul(const void* gu, void* a, int is_bf16, int T, int I, hipStream_t s) {
+    if (T <= 0 || I <= 0) return BR_OK;
+    size_t n = (size_t)T * I;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (is_bf16) silu_mul_kernel<bf16><<<blocks, 256, 0, s>>>((const bf16*)gu, (bf16*)a, I, n);
+    else silu_mul_kernel<float><<<blocks, 256, 0, s>>>((const float*)gu, (float*)a, I, n);
+    return br_check_launch();
+}
+
+// ---------------------------------------------------------------- residual add -----
+// x[i] += float(y[i])                 reference: op_residual_add, megakernel_ops.hip:1185-1212
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ y, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += to_f32<T>(y[i]);
+}
+
+extern "C" int br_residual_add(float* x, const void* y, int y_is_bf16, size_t n, hipStream_t s) {
+    if (n == 0) return BR_OK;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (y_is_bf16) residual_add_kernel<bf16><<<blocks, 256, 0, s>>>(x, (const bf16*)y, n);
+    else residual_add_kernel<float><<<blocks, 256, 0, s>>>(x, (const float*)y, n);
+    return br_check_launch();
+}
+
+// ------------------------------------------------------------------ row gather -----
+// out[i, :] = x[rows[i], :] (float)   reference: D2dCopy of the last row,
+// megakernel/megakernel_compile.rs:522-527.
+__global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                   float* __restrict__ out, int H) {
+    const float* xr = x + (size_t)rows[blockIdx.x] * H;
+    float* o = out + (size_t)blockIdx.x * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = xr[i];
+}
+
+extern "C" int br_gather_rows(const float* x, const int* rows, float* out, int R, int H, hipStream_t s) {
+    if (R <= 0 || H <= 0) return BR_OK;
+    gather_rows_kernel<<<R, 128, 0, s>>>(x, rows, out, H);
+    return br_check_launch();
+}
+
+// --------------------------------------------------------------- dtype convert -----
+// float -> bf16 (round to nearest even) and bf16 -> float, for activations that meet a
+// weight kept in the other precision.
+__global__ void f32_to_bf16_kernel(const float* __restrict__ a, bf16* __restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) b[i] = (bf16)a[i];
+}
+__global__ void bf16_to_f32_kernel(const bf16* __restrict__ a, float* __restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) b[i] = (float)a[i];
+}
+extern "C" int br_convert(const void* a, void* b, int to_bf16, size_t n, hipStream_t s) {
+    if (n == 0) return BR_OK;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (to_bf16) f32_to_bf16_kernel<<<blocks, 256, 0, s>>>((const float*)a, (bf16*)b, n);
+    else bf16_to_f32_kernel<<<blocks, 256, 0, s>>>((const bf16*)a, (float*)b, n);
+    return br_check_launch();
+}

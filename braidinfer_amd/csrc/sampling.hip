@@ -1,0 +1,252 @@
+// Sampling over rows of float logits [B, V]: argmax, and the reference's sampler
+// (crates/braidinfer-runtime/src/sampling.rs:49-171) in its order: logit bias,
+// repetition penalty, temperature, top-k, min-p, top-p, softmax, inverse CDF with a
+// uniform number the host supplies.  One block per row; every reduction and scan has a
+// fixed order, so a row samples the same token alone or inside any batch.
+#include "common.h"
+
+#define SBLOCK 256
+
+// order-preserving map float -> uint32 (larger float = larger key; -0 < +0 is harmless)
+__device__ __forceinline__ uint32_t f2key(float f) {
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key2f(uint32_t k) {
+    uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return __uint_as_float(u);
+}
+
+// ---------------------------------------------------------------------- argmax -----
+// out[b] = index of the largest logit of row b; the lowest index wins ties (the
+// reference's GPU kernel keeps the first maximum within a thread's stripe,
+// kernels/argmax.hip:21-27; its host argmax keeps the last, generate.rs:493-500; one
+// rule is fixed here).  NaN never wins.
+__device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int oi) {
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+
+__global__ __launch_bounds__(SBLOCK) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+    __shared__ float sv[SBLOCK / 64];
+    __shared__ int si[SBLOCK / 64];
+    const float* r = logits + (size_t)blockIdx.x * V;
+    float bv = -INFINITY; int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += SBLOCK) argmax_combine(bv, bi, r[i], i);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(bv, o, 64); int oi = __shfl_xor(bi, o, 64);
+        argmax_combine(bv, bi, ov, oi);
+    }
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < SBLOCK / 64; ++w) argmax_combine(bv, bi, sv[w], si[w]);
+        out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+    }
+}
+
+extern "C" int br_argmax(const float* logits, int* out, int B, int V, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0) return BR_BAD_ARG;
+    argmax_kernel<<<B, SBLOCK, 0, s>>>(logits, out, V);
+    return br_check_launch();
+}
+
+// --------------------------------------------------- bias, penalty, temperature ----
+// work[b, :] = logits[b, :]; then per row, in the reference's order (sampling.rs:57-87):
+// bias entries (token, delta) are added; every history token's logit is divided by the
+// penalty when positive, multiplied otherwise, once per occurrence (`count` times for a
+// unique token); everything is divided by the temperature when it is not 0.
+// Sparse lists are ragged: entries of row b are [off[b], off[b+1]).
+__global__ __launch_bounds__(SBLOCK) void sample_prepare_kernel(
+    const float* __restrict__ logits, float* __restrict__ work, int V,
+    const int* __restrict__ bias_off, const int* __restrict__ bias_tok, const float* __restrict__ bias_val,
+    const int* __restrict__ hist_off, const int* __restrict__ hist_tok, const int* __restrict__ hist_cnt,
+    const float* __restrict__ penalty, const float* __restrict__ temperature) {
+    const int b = blockIdx.x;
+    const float* r = logits + (size_t)b * V;
+    float* w = work + (size_t)b * V;
+    for (int i = threadIdx.x; i < V; i += SBLOCK) w[i] = r[i];
+    __syncthreads();
+    if (bias_off) {
+        // entries of one row may repeat a token: one thread applies them in order
+        if (threadIdx.x == 0)
+            for (int e = bias_off[b]; e < bias_off[b + 1]; ++e) {
+                int tk = bias_tok[e];
+                if (tk >= 0 && tk < V) w[tk] += bias_val[e];
+            }
+        __syncthreads();
+    }
+    const float pen = penalty ? penalty[b] : 1.f;
+    if (hist_off && pen != 1.f) {
+        for (int e = hist_off[b] + threadIdx.x; e < hist_off[b + 1]; e += SBLOCK) {
+            int tk = hist_tok[e];
+            if (tk < 0 || tk >= V) continue;
+            float v = w[tk];
+            for (int c = 0; c < hist_cnt[e]; ++c) v = (v > 0.f) ? v / pen : v * pen;
+            w[tk] = v;
+        }
+        __syncthreads();
+    }
+    const float temp = temperature[b];
+    if (temp != 0.f)
+        for (int i = threadIdx.x; i < V; i += SBLOCK) w[i] = w[i] / temp;
+}
+
+extern "C" int br_sample_prepare(const float* logits, float* work, int B, int V, const int* bias_off,
+                                 const int* bias_tok, const float* bias_val, const int* hist_off,
+                                 const int* hist_tok, const int* hist_cnt, const float* penalty,
+                                 const float* temperature, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0) return BR_BAD_ARG;
+    sample_prepare_kernel<<<B, SBLOCK, 0, s>>>(logits, work, V, bias_off, bias_tok, bias_val, hist_off,
+                                               hist_tok, hist_cnt, penalty, temperature);
+    return br_check_launch();
+}
+
+// ------------------------------------------------- top-k / min-p / top-p filter ----
+// Masks entries of work[b, :] to -inf as sampling.rs:89-151 does.  The row is sorted
+// once, descending by value with the lower index first among equals, as 64-bit keys
+// (value key << 32 | ~index) by a bitonic network in `keys` ([B, n2], n2 = V rounded up
+// to a power of two).  top-k keeps the first k of that order; min-p keeps values with
+// exp(v - max) >= min_p; top-p keeps the shortest prefix of the survivors whose
+// probabilities (softmax over the survivors) sum to >= top_p, accumulated in order.
+#define FBLOCK 1024
+__global__ __launch_bounds__(FBLOCK) void sample_filter_kernel(
+    float* __restrict__ work, unsigned long long* __restrict__ keys, int V, int n2,
+    const int* __restrict__ top_k, const float* __restrict__ min_p, const float* __restrict__ top_p,
+    const float* __restrict__ temperature) {
+    __shared__ float red[16];
+    __shared__ int keep_s;
+    const int b = blockIdx.x;
+    const int k = top_k[b]; const float mp = min_p[b], tp = top_p[b];
+    const bool use_k = k > 0 && k < V, use_mp = mp > 0.f, use_tp = tp < 1.f;
+    if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
+    float* w = work + (size_t)b * V;
+    unsigned long long* ks = keys + (size_t)b * n2;
+    for (int i = threadIdx.x; i < n2; i += FBLOCK)
+        ks[i] = i < V ? (((unsigned long long)f2key(w[i]) << 32) | (uint32_t)(~(uint32_t)i)) : 0ull;
+    __syncthreads();
+    // bitonic sort, descending
+    for (int size = 2; size <= n2; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int i = threadIdx.x; i < n2 / 2; i += FBLOCK) {
+                const int lo = 2 * i - (i & (stride - 1)), hi = lo + stride;
+                const bool desc = (lo & size) == 0;
+                unsigned long long a = ks[lo], c = ks[hi];
+                if ((a < c) == desc) { ks[lo] = c; ks[hi] = a; }
+            }
+            __syncthreads();
+        }
+    }
+    // survivors are a prefix [0, keep) of the sorted order
+    int keep = V;
+    if (use_k) keep = k;
+    const float vmax = key2f((uint32_t)(ks[0] >> 32));
+    if (use_mp) {
+        // values are descending: count entries of the prefix with exp(v - max) >= min_p
+        float cnt = 0.f;
+        for (int i = threadIdx.x; i < keep; i += FBLOCK) {
+            float v = key2f((uint32_t)(ks[i] >> 32));
+            if (!(v > -INFINITY && expf(v - vmax) < mp)) cnt += 1.f;
+        }
+        keep = (int)(block_sum(cnt, red) + 0.5f);
+    }
+    if (use_tp) {
+        float part = 0.f;
+        for (int i = threadIdx.x; i < keep; i += FBLOCK) {
+            float v = key2f((uint32_t)(ks[i] >> 32));
+            if (v > -INFINITY) part += expf(v - vmax);
+        }
+        const float sum = block_sum(part, red);
+        if (threadIdx.x == 0) {
+            float cum = 0.f; int cut = keep;
+            for (int i = 0; i < keep; ++i) {
+                float v = key2f((uint32_t)(ks[i] >> 32));
+                if (!(v > -INFINITY)) { cut = i; break; }
+                cum += expf(v - vmax) / sum;
+                if (cum >= tp) { cut = i + 1; break; }
+            }
+            keep_s = cut;
+        }
+        __syncthreads();
+        keep = keep_s;
+    }
+    for (int i = keep + threadIdx.x; i < V; i += FBLOCK) w[~(uint32_t)(ks[i] & 0xffffffffu)] = -INFINITY;
+}
+
+extern "C" int br_sample_filter(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
+                                const float* min_p, const float* top_p, const float* temperature,
+                                hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0 || n2 < V || (n2 & (n2 - 1))) return BR_BAD_ARG;
+    sample_filter_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature);
+    return br_check_launch();
+}
+
+// ----------------------------------------------------------- softmax + draw --------
+// out[b] = first index i with u <= sum_{j<=i} softmax(work[b])_j  (sampling.rs:153-170);
+// argmax of the row when temperature is 0 (:81-84) or when rounding leaves u above the
+// last partial sum (:170).  Sums run over indices in ascending order, SBLOCK at a time.
+__global__ __launch_bounds__(SBLOCK) void sample_draw_kernel(const float* __restrict__ work, int* __restrict__ out,
+                                                             int V, const float* __restrict__ temperature,
+                                                             const float* __restrict__ u) {
+    __shared__ float red[16];
+    __shared__ float wsum[SBLOCK / 64];
+    __shared__ int found;
+    __shared__ float sv[SBLOCK / 64];
+    __shared__ int si[SBLOCK / 64];
+    const int b = blockIdx.x;
+    const float* w = work + (size_t)b * V;
+    // argmax (lowest index wins)
+    float bv = -INFINITY; int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += SBLOCK) argmax_combine(bv, bi, w[i], i);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(bv, o, 64); int oi = __shfl_xor(bi, o, 64);
+        argmax_combine(bv, bi, ov, oi);
+    }
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    if (threadIdx.x == 0) found = 0x7fffffff;
+    __syncthreads();
+    for (int ww = 0; ww < SBLOCK / 64; ++ww) argmax_combine(bv, bi, sv[ww], si[ww]);
+    if (bi == 0x7fffffff) bi = 0;
+    if (temperature[b] == 0.f) { if (threadIdx.x == 0) out[b] = bi; return; }
+    const float vmax = bv;
+    float part = 0.f;
+    for (int i = threadIdx.x; i < V; i += SBLOCK) part += expf(w[i] - vmax);
+    const float sum = block_sum(part, red);
+    const float target = u[b];
+    float base = 0.f;   // cumulative probability before this chunk
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int i0 = 0; i0 < V; i0 += SBLOCK) {
+        const int i = i0 + threadIdx.x;
+        const float p = i < V ? expf(w[i] - vmax) / sum : 0.f;
+        // inclusive scan inside the wave, then across the waves
+        float sc = p;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+        __syncthreads();
+        if (lane == 63) wsum[wv] = sc;
+        __syncthreads();
+        float before = base;
+        for (int x = 0; x < wv; ++x) before += wsum[x];
+        const float cum = before + sc;
+        // the first index with u <= cum: every later index satisfies it too, take the minimum
+        if (i < V && target <= cum) atomicMin(&found, i);
+        float tot = base;
+        for (int x = 0; x < SBLOCK / 64; ++x) tot += wsum[x];
+        base = tot;
+        __syncthreads();
+        if (found != 0x7fffffff) break;
+    }
+    if (threadIdx.x == 0) out[b] = found != 0x7fffffff ? found : bi;
+}
+
+extern "C" int br_sample_draw(const float* work, int* out, int B, int V, const float* temperature,
+                              const float* u, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0) return BR_BAD_ARG;
+    sample_draw_kernel<<<B, SBLOCK, 0, s>>>(work, out, V, temperature, u);
+    return br_check_launch();
+}

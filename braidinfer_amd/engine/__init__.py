@@ -1,0 +1,5 @@
+from .step import StepBatch, Workspace, pack_step
+from .model import DecoderModel, Layer
+from .engine import Engine, StepEntry, parse_dtype
+
+__all__ = ["StepBatch", "Workspace", "pack_step", "DecoderModel", "Layer", "Engine", "StepEntry", "parse_dtype"]

@@ -1,0 +1,146 @@
+"""The engine: a loaded model, its cache, and the one step function.
+
+reference: `Model::prefill(&[u32]) -> logits of the last token` and
+`Model::decode_step(token, position) -> logits` for the one sequence a `Model` holds
+(crates/braidinfer-runtime/src/model/state.rs:39-206, model/mod.rs:279-286).  Here one
+`step` serves a batch: every entry brings the next tokens of its sequence, and logits
+come back for the places asked for.
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..cache import SequenceCache
+from ..config import config_from_folder, spec_of
+from ..errors import BraidError, CacheError, ConfigError, KernelError, StepError
+from ..parts import Runtime
+from ..weights import load_tensors, random_tensors, write_model_folder
+from .model import DecoderModel
+from .step import StepBatch, Workspace, pack_step
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    if dtype not in _DTYPES:
+        raise ConfigError(f"dtype {dtype!r} is not supported; use 'bfloat16' or 'float32'")
+    return _DTYPES[dtype]
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one sequence, and the places among them whose logits are wanted."""
+
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+def _require_gpu(device: torch.device) -> None:
+    if device.type != "cuda":
+        raise KernelError(f"the engine runs on a GPU only (asked for {device}); there is no CPU path")
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU is visible to this process; the engine has no CPU path")
+
+
+class Engine:
+    def __init__(self, config, model: DecoderModel, rt: Runtime, max_tokens: int,
+                 max_seq_len: Optional[int] = None, n_slots: Optional[int] = None):
+        self.config = config
+        self.model = model
+        self.spec = model.spec
+        self.rt = rt
+        self.device = rt.device
+        self.ws = Workspace(rt.device)
+        self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens=max_tokens,
+                                   max_seq_len=max_seq_len, n_slots=n_slots, dtype=rt.dtype, device=rt.device)
+        self.vocab_size = self.spec.vocab_size
+
+    # ---- construction ------------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
+                    max_seq_len: Optional[int] = None, n_slots: Optional[int] = None) -> "Engine":
+        device = torch.device(device)
+        _require_gpu(device)
+        config = config_from_folder(folder)
+        model = DecoderModel(spec_of(config))
+        rt = Runtime(device=device, dtype=parse_dtype(dtype))
+        tensors = load_tensors(folder, model.weight_specs(), device, rt.dtype,
+                               allow_unexpected=model.optional_names())
+        model.load(tensors, rt)
+        return cls(config, model, rt, max_tokens, max_seq_len, n_slots)
+
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
+               max_seq_len: Optional[int] = None, n_slots: Optional[int] = None, std: float = 0.02,
+               num_layers: Optional[int] = None) -> "Engine":
+        """Seeded random weights made on the device (no folder): bf16 N(0, std) matrices,
+        norm weights 1, as the random-weights folder mode makes them."""
+        device = torch.device(device)
+        _require_gpu(device)
+        model = DecoderModel(spec_of(config))
+        rt = Runtime(device=device, dtype=parse_dtype(dtype))
+        tensors = {}
+        for name, t in random_tensors(model.weight_specs(), seed, device, torch.bfloat16, std):
+            kind_vec = t.dim() == 1
+            tensors[name] = t.to(torch.float32) if (kind_vec or rt.dtype == torch.float32) else t
+        model.load(tensors, rt)
+        return cls(config, model, rt, max_tokens, max_seq_len, n_slots)
+
+    @staticmethod
+    def write_random_folder(folder: str, config, seed: int = 0, std: float = 0.02,
+                            vector_jitter: float = 0.0) -> str:
+        """Random-weights mode: a model folder (config.json, model.safetensors)."""
+        model = DecoderModel(spec_of(config))
+        return write_model_folder(folder, config, model.weight_specs(), seed, std, vector_jitter)
+
+    # ---- slots -----------------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ---- the step function -------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the given tokens of each entry's sequence as one batch, from the cache
+        earlier steps left; return float32 logits `[number of wanted places, vocab]` on the
+        device, in the order of the entries and of each entry's `want`.
+
+        Nothing is changed if the step cannot be run (bad entry, no room in the cache)."""
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        slots = [e.slot for e in entries]
+        token_lists = [list(e.tokens) for e in entries]
+        V = self.vocab_size
+        rows: List[int] = []
+        base = 0
+        for e, tl in zip(entries, token_lists):
+            if not tl:
+                raise StepError(f"slot {e.slot}: an entry brings no tokens")
+            for t in tl:
+                if not isinstance(t, int) or isinstance(t, bool) or not 0 <= t < V:
+                    raise StepError(f"slot {e.slot}: token {t!r} is outside the vocabulary of {V}")
+            for w in e.want:
+                if not isinstance(w, int) or not 0 <= w < len(tl):
+                    raise StepError(f"slot {e.slot}: wanted place {w!r} is outside its {len(tl)} tokens")
+                rows.append(base + w)
+            base += len(tl)
+        new = [len(tl) for tl in token_lists]
+        self.cache.reserve(slots, new)          # all or nothing
+        starts = [self.cache.lengths[s] for s in slots]
+        step = pack_step(slots, token_lists, starts, self.device, self.ws)
+        n_want = len(rows)
+        want_rows = (torch.tensor(rows, dtype=torch.int32).to(self.device) if n_want
+                     else torch.empty(0, dtype=torch.int32, device=self.device))
+        logits = self.model.forward(step, self.cache, want_rows, n_want)
+        self.cache.commit(slots, new)
+        return logits

@@ -1,0 +1,157 @@
+"""A decoder built from a `ModelSpec`: parts by kind, layers by list, run order by list.
+
+The model is the same code for every architecture; what differs is the spec its
+architecture's builder returns.  reference: `Model` owns weights, activations, cache
+and the compiled program (crates/braidinfer-runtime/src/model/mod.rs:23-119); the
+per-layer order is megakernel/megakernel_compile.rs:115-236, the tail (last-row gather,
+final norm, lm_head) :238-262 and :521-551.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import kernels as K
+from ..cache import CacheNeed, SequenceCache, StateNeed
+from ..config import ModelSpec, spec_of
+from ..errors import ConfigError, StepError
+from ..parts import MixerContext, Runtime, block_arrangement, build_part
+from ..weights import TensorSpec
+from .step import StepBatch
+
+
+class Layer:
+    """The parts of one layer; built from a `LayerSpec`."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.mixer = build_part("mixer", spec.mixer) if spec.mixer else None
+        self.feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward else None
+        self.mixer_norm = build_part("norm", spec.mixer_norm) if (spec.mixer and spec.mixer_norm) else None
+        self.ffn_norm = build_part("norm", spec.ffn_norm) if (spec.feed_forward and spec.ffn_norm) else None
+        self.run = block_arrangement(spec.block)
+        self.rt: Optional[Runtime] = None
+
+    def named_parts(self):
+        s = self.spec
+        for part, name in ((self.mixer_norm, s.mixer_norm_name), (self.mixer, s.mixer_name),
+                           (self.ffn_norm, s.ffn_norm_name), (self.feed_forward, s.feed_forward_name)):
+            if part is not None:
+                yield part, s.prefix + name
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = build_part("embedding", spec.embedding)
+        self.layers: List[Layer] = [Layer(ls) for ls in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm)
+        self.lm_head = build_part("lm_head", spec.lm_head)
+        self.positions = {name: build_part("position", ps) for name, ps in spec.positions.items()}
+        self.schedule = list(spec.schedule)
+        for e in self.schedule:
+            if not 0 <= e.layer < len(self.layers):
+                raise ConfigError(f"schedule names layer {e.layer}, the model has {len(self.layers)}")
+        written = set()
+        for e in self.schedule:
+            if e.cache is not None and self.layers[e.layer].mixer is not None:
+                if e.writes_cache:
+                    written.add(e.cache)
+                elif e.cache not in written:
+                    raise ConfigError(f"schedule entry reads cache {e.cache} before any entry writes it")
+        self.rt: Optional[Runtime] = None
+
+    # ---- weights -------------------------------------------------------------------
+    def _named_parts(self):
+        s = self.spec
+        yield self.embedding, s.embedding_prefix
+        for layer in self.layers:
+            yield from layer.named_parts()
+        yield self.final_norm, s.final_norm_prefix
+        yield self.lm_head, s.lm_head_prefix
+        for name, p in self.positions.items():
+            yield p, f"position.{name}."
+
+    def weight_specs(self) -> List[TensorSpec]:
+        out: List[TensorSpec] = []
+        for part, prefix in self._named_parts():
+            out.extend(part.weight_specs(prefix))
+        names = [s.name for s in out]
+        if len(set(names)) != len(names):
+            dup = sorted({n for n in names if names.count(n) > 1})
+            raise ConfigError(f"two parts declare the same tensor: {dup}")
+        return out
+
+    def optional_names(self) -> List[str]:
+        out: List[str] = []
+        for part, prefix in self._named_parts():
+            f = getattr(part, "optional_names", None)
+            if f:
+                out.extend(f(prefix))
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        for part, prefix in self._named_parts():
+            part.load(tensors, prefix, rt)
+        for layer in self.layers:
+            layer.rt = rt
+
+    # ---- what the cache must hold ----------------------------------------------------
+    def cache_needs(self) -> Dict[int, CacheNeed]:
+        needs: Dict[int, CacheNeed] = {}
+        for e in self.schedule:
+            m = self.layers[e.layer].mixer
+            if m is None or e.cache is None:
+                continue
+            n = m.cache_need()
+            if n is None:
+                continue
+            if e.cache in needs and needs[e.cache] != n:
+                raise ConfigError(f"cache unit {e.cache} is shared by mixers with different needs: "
+                                  f"{needs[e.cache]} and {n}")
+            needs[e.cache] = n
+        return needs
+
+    def state_needs(self) -> Dict[object, StateNeed]:
+        out: Dict[object, StateNeed] = {}
+        for i, e in enumerate(self.schedule):
+            m = self.layers[e.layer].mixer
+            if m is None:
+                continue
+            n = m.state_need()
+            if n is not None:
+                out[("entry", i)] = n
+        return out
+
+    # ---- one step ----------------------------------------------------------------------
+    def forward(self, step: StepBatch, cache: SequenceCache, want_rows: torch.Tensor, n_want: int) -> torch.Tensor:
+        """Run the step's tokens through every scheduled layer; return float32 logits
+        `[n_want, vocab]` of the rows `want_rows` (indices into the packed tokens)."""
+        rt = self.rt
+        T, H = step.n_tokens, self.spec.hidden_size
+        ws = step.ws
+        x = ws.get("residual", (T, H), torch.float32)
+        self.embedding.forward(step.tokens, x)
+        step.position_data = {}
+        for name, enc in self.positions.items():
+            step.position_data[name] = enc.prepare(step)
+            enc.add_to_embedding(x, step)
+        for i, e in enumerate(self.schedule):
+            layer = self.layers[e.layer]
+            ctx = MixerContext(unit=e.cache, writes_cache=e.writes_cache)
+            if layer.mixer is not None:
+                if e.cache is not None and e.cache in cache.group_of_unit:
+                    g = cache.unit_group(e.cache)
+                    ctx.storage, ctx.block_table, ctx.page_tokens = g.storage[e.cache], g.table_dev, g.page_tokens
+                ctx.state = cache.state(("entry", i))
+            layer.run(layer, x, step, ctx)
+        logits = ws.get("logits", (max(n_want, 1), self.spec.vocab_size), torch.float32)[:n_want]
+        if n_want == 0:
+            return logits
+        hn = ws.get("final_h", (n_want, H), rt.dtype)
+        self.final_norm.forward(x, hn, rows=want_rows)
+        self.lm_head.forward(hn, logits, ws)
+        return logits

@@ -1,0 +1,98 @@
+"""What one step hands to the parts: the packed tokens of a batch and where they sit.
+
+A step runs the tokens it is given, as one batch: `n_i >= 1` new tokens for each of B
+sequences, packed one after another.  All arrays are int32 on the device; the same
+numbers are kept as Python lists for host-side decisions.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+
+class Workspace:
+    """Named scratch buffers that grow and are reused from step to step."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._bufs: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:n].view(tuple(int(s) for s in shape))
+
+    def clear(self) -> None:
+        self._bufs.clear()
+
+
+@dataclass
+class StepBatch:
+    n_tokens: int                    # T: tokens in this step (padding included)
+    n_seqs: int                      # B: sequences (padding included)
+    tokens: torch.Tensor             # [T] token ids
+    positions: torch.Tensor          # [T] position of each token in its sequence
+    seq_of_token: torch.Tensor       # [T] index into the batch
+    cu_seqlens: torch.Tensor         # [B + 1] offsets of the sequences' tokens
+    slots: torch.Tensor              # [B] cache slot of each sequence, -1 = padding
+    ctx_lens: torch.Tensor           # [B] length of each sequence after this step
+    # the same on the host
+    host_slots: List[int] = field(default_factory=list)
+    host_new: List[int] = field(default_factory=list)       # n_i
+    host_start: List[int] = field(default_factory=list)     # length before the step
+    is_decode: bool = False          # every sequence brings exactly one token
+    max_new: int = 0
+    max_ctx: int = 0
+    ws: Optional[Workspace] = None
+    position_data: Dict[str, Any] = field(default_factory=dict)
+    extras: Dict[str, Any] = field(default_factory=dict)     # per-step scratch of parts (keyed by them)
+
+
+def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts: Sequence[int],
+              device, ws: Workspace, pad_seqs: int = 0) -> StepBatch:
+    """Build the device arrays of a step in one host-to-device copy.  `pad_seqs` extra
+    sequences of one dummy token (slot -1, position 0) may follow the real ones."""
+    B = len(slots) + pad_seqs
+    new = [len(t) for t in token_lists] + [1] * pad_seqs
+    T = sum(new)
+    flat: List[int] = []
+    # layout of the one int32 staging array: tokens | positions | seq_of_token | cu | slots | ctx
+    toks: List[int] = []
+    pos: List[int] = []
+    sot: List[int] = []
+    cu = [0]
+    ctx: List[int] = []
+    all_slots = list(slots) + [-1] * pad_seqs
+    all_starts = list(starts) + [0] * pad_seqs
+    for b in range(B):
+        tl = token_lists[b] if b < len(token_lists) else [0]
+        st = all_starts[b]
+        toks.extend(tl)
+        pos.extend(range(st, st + len(tl)))
+        sot.extend([b] * len(tl))
+        cu.append(cu[-1] + len(tl))
+        ctx.append(st + len(tl) if all_slots[b] >= 0 else 0)
+    flat = toks + pos + sot + cu + all_slots + ctx
+    host = torch.tensor(flat, dtype=torch.int32)
+    dev = host.to(device)
+    o = 0
+    def take(n):
+        nonlocal o
+        v = dev[o:o + n]
+        o += n
+        return v
+    tokens, positions, seq_of_token = take(T), take(T), take(T)
+    cu_seqlens, slots_d, ctx_d = take(B + 1), take(B), take(B)
+    return StepBatch(
+        n_tokens=T, n_seqs=B, tokens=tokens, positions=positions, seq_of_token=seq_of_token,
+        cu_seqlens=cu_seqlens, slots=slots_d, ctx_lens=ctx_d, host_slots=all_slots, host_new=new,
+        host_start=all_starts, is_decode=all(n == 1 for n in new), max_new=max(new) if new else 0,
+        max_ctx=max(ctx) if ctx else 0, ws=ws)

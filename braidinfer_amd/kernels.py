@@ -1,0 +1,256 @@
+"""Python launchers of the HIP kernels: argument checks on the host, then one C call.
+
+Every function takes torch tensors that live on the GPU, checks what the kernel and its
+grid assume (device, dtype, contiguity, shapes) and launches on torch's current stream.
+There is no fallback: a missing library or a size a kernel does not take raises
+`KernelError`.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_void_p, c_int, c_float, c_size_t
+from typing import Optional
+
+import torch
+
+from .errors import KernelError
+from .csrc import build as _build
+
+_P = c_void_p
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _req(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(name: str, *tensors) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError(f"{name}: tensor on {t.device}; kernels run on the GPU only")
+        if not t.is_contiguous():
+            raise KernelError(f"{name}: tensor of shape {tuple(t.shape)} is not contiguous")
+
+
+def _is_bf16(t: torch.Tensor, name: str) -> int:
+    if t.dtype == torch.bfloat16:
+        return 1
+    if t.dtype == torch.float32:
+        return 0
+    raise KernelError(f"{name}: dtype {t.dtype} is not supported (float32 or bfloat16)")
+
+
+def _check(rc: int, name: str) -> None:
+    if rc == 0:
+        return
+    raise KernelError(f"{name}: " + {1: "arguments outside what the kernel takes",
+                                     2: "launch failed"}.get(rc, f"error {rc}"))
+
+
+_sigs_done = set()
+
+
+def _fn(module: str, name: str, argtypes):
+    lib = _build.load(module)
+    f = getattr(lib, name)
+    if (module, name) not in _sigs_done:
+        f.argtypes = argtypes
+        f.restype = c_int
+        _sigs_done.add((module, name))
+    return f
+
+
+# ------------------------------------------------------------------ elementwise -----
+def embedding(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("embedding", table, tokens, out)
+    T = tokens.numel()
+    V, H = table.shape
+    _req(tokens.dtype == torch.int32, "embedding: tokens must be int32")
+    _req(out.dtype == torch.float32 and out.shape == (T, H), "embedding: out must be float32 [T, H]")
+    f = _fn("elementwise", "br_embedding", [_P, c_int, _P, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(table), _is_bf16(table, "embedding"), _ptr(tokens), _ptr(out), T, H, V, _stream()), "embedding")
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float,
+            rows: Optional[torch.Tensor] = None) -> None:
+    _dev("rmsnorm", x, w, out, rows)
+    H = x.shape[-1]
+    R = out.shape[0]
+    _req(x.dtype == torch.float32 and w.dtype == torch.float32, "rmsnorm: x and w must be float32")
+    _req(w.numel() == H and out.shape[-1] == H, "rmsnorm: widths of x, w and out differ")
+    if rows is None:
+        _req(x.shape[0] == R, "rmsnorm: out has other rows than x")
+    else:
+        _req(rows.dtype == torch.int32 and rows.numel() == R, "rmsnorm: rows must be int32 [R]")
+    f = _fn("elementwise", "br_rmsnorm", [_P, _P, _P, c_int, _P, c_int, c_int, c_float, _P])
+    _check(f(_ptr(x), _ptr(w), _ptr(out), _is_bf16(out, "rmsnorm"), _ptr(rows), R, H, float(eps), _stream()),
+           "rmsnorm")
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    _dev("rope_table", positions, inv_freq, cos, sin)
+    T, P = positions.numel(), inv_freq.numel()
+    _req(positions.dtype == torch.int32 and inv_freq.dtype == torch.float32, "rope_table: dtypes")
+    _req(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.numel() >= T * P
+         and sin.numel() >= T * P, "rope_table: tables must be float32 [T, P]")
+    f = _fn("elementwise", "br_rope_table", [_P, _P, _P, _P, c_int, c_int, _P])
+    _check(f(_ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), T, P, _stream()), "rope_table")
+
+
+def rope_kv_write(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                  positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
+                  block_table: torch.Tensor, cache: Optional[torch.Tensor], nq: int, nkv: int, hd: int,
+                  rotary_dim: int, adjacent: bool, page: int, write_cache: bool) -> None:
+    _dev("rope_kv_write", qkv, cos, sin, positions, seq_of_token, slots, block_table, cache)
+    T = qkv.shape[0]
+    _req(qkv.shape[1] == (nq + 2 * nkv) * hd, "rope_kv_write: qkv width is not (nq + 2 nkv) * head_dim")
+    _req(positions.numel() >= T and seq_of_token.numel() >= T, "rope_kv_write: positions shorter than tokens")
+    _req(block_table.dim() == 2 and block_table.dtype == torch.int32, "rope_kv_write: block table int32 [slots, pages]")
+    if cos is not None:
+        _req(cos.numel() >= T * (rotary_dim // 2) and sin is not None, "rope_kv_write: rotary tables too short")
+    if write_cache:
+        _req(cache is not None and cache.dtype == qkv.dtype, "rope_kv_write: cache dtype differs from activations")
+        _req(cache.shape[1:] == (2, nkv, page, hd), "rope_kv_write: cache unit must be [pages, 2, nkv, page, hd]")
+    f = _fn("elementwise", "br_rope_kv_write",
+            [_P, c_int, _P, _P, _P, _P, _P, _P, c_int, _P] + [c_int] * 8 + [_P])
+    _check(f(_ptr(qkv), _is_bf16(qkv, "rope_kv_write"), _ptr(cos), _ptr(sin), _ptr(positions),
+             _ptr(seq_of_token), _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(cache), T, nq, nkv,
+             hd, rotary_dim, int(adjacent), page, int(write_cache), _stream()), "rope_kv_write")
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("silu_mul", gu, out)
+    T, I2 = gu.shape
+    _req(I2 % 2 == 0 and out.shape == (T, I2 // 2) and out.dtype == gu.dtype, "silu_mul: out must be [T, I] of gu's dtype")
+    f = _fn("elementwise", "br_silu_mul", [_P, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(gu), _ptr(out), _is_bf16(gu, "silu_mul"), T, I2 // 2, _stream()), "silu_mul")
+
+
+def residual_add(x: torch.Tensor, y: torch.Tensor) -> None:
+    _dev("residual_add", x, y)
+    _req(x.dtype == torch.float32 and x.numel() == y.numel(), "residual_add: x float32, same size as y")
+    f = _fn("elementwise", "br_residual_add", [_P, _P, c_int, c_size_t, _P])
+    _check(f(_ptr(x), _ptr(y), _is_bf16(y, "residual_add"), x.numel(), _stream()), "residual_add")
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("gather_rows", x, rows, out)
+    _req(x.dtype == torch.float32 and out.dtype == torch.float32 and rows.dtype == torch.int32, "gather_rows: dtypes")
+    _req(out.shape == (rows.numel(), x.shape[1]), "gather_rows: out must be [R, H]")
+    f = _fn("elementwise", "br_gather_rows", [_P, _P, _P, c_int, c_int, _P])
+    _check(f(_ptr(x), _ptr(rows), _ptr(out), rows.numel(), x.shape[1], _stream()), "gather_rows")
+
+
+def convert(a: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("convert", a, out)
+    _req(a.numel() == out.numel(), "convert: sizes differ")
+    if a.dtype == torch.float32 and out.dtype == torch.bfloat16:
+        to_bf16 = 1
+    elif a.dtype == torch.bfloat16 and out.dtype == torch.float32:
+        to_bf16 = 0
+    else:
+        raise KernelError(f"convert: {a.dtype} -> {out.dtype} is not supported")
+    f = _fn("elementwise", "br_convert", [_P, _P, c_int, c_size_t, _P])
+    _check(f(_ptr(a), _ptr(out), to_bf16, a.numel(), _stream()), "convert")
+
+
+# ------------------------------------------------------------------------ GEMM ------
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out[M, N] (+)= a[M, K] @ w[N, K]^T.
+
+    float32 a and w: the true 32-bit kernel (out float32).  bfloat16 a and w: the
+    matrix-core kernels with float accumulation; out is bfloat16, or float32 (and may
+    then accumulate, which is how a projection adds into the residual stream).
+    Rows of `a` and `out` may be strided (a view of a wider buffer); w is contiguous.
+    """
+    name = "gemm"
+    for t in (a, w, out):
+        if not t.is_cuda:
+            raise KernelError(f"{name}: tensor on {t.device}; kernels run on the GPU only")
+    _req(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: 2-D tensors")
+    M, K = a.shape
+    N = w.shape[0]
+    _req(w.shape[1] == K and out.shape == (M, N), f"gemm: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)}")
+    _req(w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1, "gemm: rows must be dense")
+    lda, ldc = (a.stride(0) if M > 1 else K), (out.stride(0) if M > 1 else N)
+    if a.dtype == torch.float32 and w.dtype == torch.float32:
+        _req(out.dtype == torch.float32, "gemm: float32 inputs give a float32 output")
+        f = _fn("gemm_f32", "br_gemm_f32", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P])
+        _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, int(accumulate), _stream()), name)
+    elif a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        if out.dtype == torch.bfloat16:
+            _req(not accumulate, "gemm: accumulation needs a float32 output")
+            mode = 0
+        elif out.dtype == torch.float32:
+            mode = 2 if accumulate else 1
+        else:
+            raise KernelError(f"gemm: output dtype {out.dtype}")
+        f = _fn("gemm_bf16", "br_gemm_bf16", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P])
+        _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, mode, _stream()), name)
+    else:
+        raise KernelError(f"gemm: a is {a.dtype} and w is {w.dtype}; both float32 or both bfloat16")
+
+
+# ------------------------------------------------------------------- attention -----
+def attention_simple(q: torch.Tensor, q_stride: int, out: torch.Tensor, positions: torch.Tensor,
+                     seq_of_token: torch.Tensor, slots: torch.Tensor, block_table: torch.Tensor,
+                     cache: torch.Tensor, T: int, nq: int, nkv: int, hd: int, page: int,
+                     window: Optional[int], scale: float) -> None:
+    _dev("attention_simple", out, positions, seq_of_token, slots, block_table, cache)
+    _req(q.is_cuda and q.dtype == cache.dtype == out.dtype, "attention_simple: q, cache and out share a dtype")
+    _req(out.shape == (T, nq * hd), "attention_simple: out must be [T, nq * hd]")
+    _req(cache.shape[1:] == (2, nkv, page, hd), "attention_simple: cache unit must be [pages, 2, nkv, page, hd]")
+    _req(nq % nkv == 0, "attention_simple: heads must be a multiple of kv heads")
+    _req(hd <= 512, f"attention_simple: head_dim {hd} above 512 is not supported")
+    f = _fn("attention_simple", "br_attn_simple",
+            [_P, c_size_t, _P, c_int, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, _P])
+    _check(f(_ptr(q), q_stride, _ptr(out), _is_bf16(q, "attention_simple"), _ptr(positions), _ptr(seq_of_token),
+             _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(cache), T, nq, nkv, hd, page,
+             int(window or 0), float(scale), _stream()), "attention_simple")
+
+
+# -------------------------------------------------------------------- sampling -----
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("argmax", logits, out)
+    B, V = logits.shape
+    _req(logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= B, "argmax: float32 in, int32 out")
+    f = _fn("sampling", "br_argmax", [_P, _P, c_int, c_int, _P])
+    _check(f(_ptr(logits), _ptr(out), B, V, _stream()), "argmax")
+
+
+def sample_prepare(logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature):
+    _dev("sample_prepare", logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature)
+    B, V = logits.shape
+    _req(logits.dtype == torch.float32 and work.dtype == torch.float32 and work.shape == logits.shape, "sample_prepare: float32 [B, V]")
+    f = _fn("sampling", "br_sample_prepare", [_P, _P, c_int, c_int] + [_P] * 9)
+    _check(f(_ptr(logits), _ptr(work), B, V, _ptr(bias_off), _ptr(bias_tok), _ptr(bias_val), _ptr(hist_off),
+             _ptr(hist_tok), _ptr(hist_cnt), _ptr(penalty), _ptr(temperature), _stream()), "sample_prepare")
+
+
+def sample_filter(work, keys, top_k, min_p, top_p, temperature):
+    _dev("sample_filter", work, keys, top_k, min_p, top_p, temperature)
+    B, V = work.shape
+    n2 = keys.shape[1]
+    _req(keys.dtype == torch.int64 and keys.shape[0] == B and n2 >= V and n2 & (n2 - 1) == 0,
+         "sample_filter: keys must be int64 [B, power of two >= V]")
+    f = _fn("sampling", "br_sample_filter", [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P])
+    _check(f(_ptr(work), _ptr(keys), B, V, n2, _ptr(top_k), _ptr(min_p), _ptr(top_p), _ptr(temperature), _stream()),
+           "sample_filter")
+
+
+def sample_draw(work, out, temperature, u):
+    _dev("sample_draw", work, out, temperature, u)
+    B, V = work.shape
+    _req(out.dtype == torch.int32 and u.dtype == torch.float32 and temperature.dtype == torch.float32, "sample_draw: dtypes")
+    f = _fn("sampling", "br_sample_draw", [_P, _P, c_int, c_int, _P, _P, _P])
+    _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(u), _stream()), "sample_draw")

@@ -1,0 +1,80 @@
+"""Grouped-query attention over the paged cache.
+
+Per token: q, k, v = W n (no bias; reference compile_attention.rs:82-85 and
+model_load.rs:635-670); q and k rotated by the position encoding; k (rotated) and v
+stored in the token's page; scores (q . k_j) * scale over the keys the token may see,
+softmax in float, weighted sum of v (reference: op_attn_paged,
+kernels/megakernel_ops.hip:2150-2343: kv head = q head / (nq / nkv) :2192, scale
+rsqrt(head_dim) :2194, causality by loop bound); x += W_o o (compile_attention.rs:333-376).
+A window W limits a query at position i to keys i-W < j <= i (absent in the reference,
+config.rs:416).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import kernels as K
+from ..cache import CacheNeed
+from ..errors import ConfigError
+from ..weights import TensorSpec
+from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
+from .linear import fuse_rows, linear
+
+
+class GQAAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 window: Optional[int] = None, position: Optional[str] = "rope", scale: Optional[float] = None):
+        if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
+            raise ConfigError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if head_dim <= 0 or head_dim % 2:
+            raise ConfigError(f"attention: head_dim {head_dim} must be positive and even")
+        self.H, self.nq, self.nkv, self.hd = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.window = None if window is None else int(window)
+        self.position = position
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        self.w_qkv = self.w_o = None
+
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        return [
+            TensorSpec(prefix + "q_proj.weight", (self.nq * self.hd, self.H)),
+            TensorSpec(prefix + "k_proj.weight", (self.nkv * self.hd, self.H)),
+            TensorSpec(prefix + "v_proj.weight", (self.nkv * self.hd, self.H)),
+            TensorSpec(prefix + "o_proj.weight", (self.H, self.nq * self.hd)),
+        ]
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+        self.w_qkv = fuse_rows([tensors[prefix + n + "_proj.weight"] for n in ("q", "k", "v")])
+        self.w_o = tensors[prefix + "o_proj.weight"].contiguous()
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(kv_heads=self.nkv, head_dim=self.hd, window=self.window)
+
+    def forward(self, h, x, step, ctx: MixerContext) -> None:
+        T = step.n_tokens
+        nq, nkv, hd = self.nq, self.nkv, self.hd
+        dt = self.rt.dtype
+        qkv = step.ws.get("attn_qkv", (T, (nq + 2 * nkv) * hd), dt)
+        linear(h, self.w_qkv, qkv, step.ws)
+        tables = step.position_data.get(self.position) if self.position else None
+        if tables is not None and not isinstance(tables, RotaryTables):
+            tables = None
+        K.rope_kv_write(qkv, tables.cos if tables else None, tables.sin if tables else None,
+                        step.positions, step.seq_of_token, step.slots, ctx.block_table, ctx.storage,
+                        nq, nkv, hd, tables.rotary_dim if tables else 0, tables.adjacent if tables else False,
+                        ctx.page_tokens, ctx.writes_cache)
+        o = step.ws.get("attn_out", (T, nq * hd), dt)
+        self.attend(qkv, o, step, ctx)
+        linear(o, self.w_o, x, step.ws, accumulate=True)
+
+    def attend(self, qkv, o, step, ctx: MixerContext) -> None:
+        T = step.n_tokens
+        K.attention_simple(qkv, qkv.stride(0), o, step.positions, step.seq_of_token, step.slots,
+                           ctx.block_table, ctx.storage, T, self.nq, self.nkv, self.hd, ctx.page_tokens,
+                           self.window, self.scale)
+
+
+register_part("mixer", "gqa_attention", GQAAttention, replace=True)

@@ -1,0 +1,151 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+A part is built from the parameters of its `PartSpec` alone; it never sees the model's
+configuration or name.  Kinds:
+
+* `Norm`             x[T, H] float32 -> activations [T, H] in the compute dtype
+* `PositionEncoding` per step: `prepare(step)`; offers rotary tables and/or an addition
+                     to the embeddings
+* `Mixer`            adds its output to the residual stream; declares what it keeps per
+                     sequence: a `CacheNeed` (growing keys/values) and/or a `StateNeed`
+                     (fixed size)
+* `FeedForward`      adds its output to the residual stream
+* block arrangements functions that run one layer's parts in order
+
+Tensors: the residual stream `x` is float32 `[T, hidden]` in both precisions; `h` is the
+normed input in the compute dtype (`runtime.dtype`).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional
+
+import torch
+
+from ..cache import CacheNeed, StateNeed
+from ..errors import ConfigError
+from ..weights import TensorSpec
+
+
+@dataclass
+class Runtime:
+    """Where and in which precision a model runs."""
+
+    device: torch.device
+    dtype: torch.dtype            # torch.float32 (true 32-bit path) or torch.bfloat16
+
+    @property
+    def is_bf16(self) -> bool:
+        return self.dtype == torch.bfloat16
+
+
+class Part:
+    """Base of every part: declares tensors by name, receives them once loaded."""
+
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        return []
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, step) -> Any:
+        """Called once per step before the layers; the result is kept in
+        `step.position_data[name]` for the mixers."""
+        return None
+
+    def add_to_embedding(self, x: torch.Tensor, step) -> None:
+        """Encodings that act on the embeddings override this."""
+
+
+@dataclass
+class RotaryTables:
+    """cos/sin [T, rotary_dim/2] float32 for the step's tokens."""
+
+    cos: torch.Tensor
+    sin: torch.Tensor
+    rotary_dim: int
+    adjacent: bool
+
+
+class Mixer(Part):
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, step, ctx: "MixerContext") -> None:
+        """Add the mixer's output for the step's tokens to `x` in place."""
+        raise NotImplementedError
+
+
+@dataclass
+class MixerContext:
+    """What one schedule entry hands its mixer: its cache unit and state, if it asked."""
+
+    unit: Optional[int] = None
+    storage: Optional[torch.Tensor] = None        # [pages, 2, kv_heads, page_tokens, head_dim]
+    block_table: Optional[torch.Tensor] = None    # int32 [slots, pages per sequence], device
+    page_tokens: int = 0
+    writes_cache: bool = True
+    state: Optional[torch.Tensor] = None          # [slots, *StateNeed.shape]
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, x: torch.Tensor, step) -> None:
+        """Add the feed-forward's output for the step's tokens to `x` in place."""
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class OutputHead(Part):
+    def forward(self, h: torch.Tensor, out: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+# ------------------------------------------------------------------ registries ------
+_REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "embedding": {}, "lm_head": {}, "block": {},
+}
+
+
+def register_part(category: str, kind: str, factory: Callable[..., Any], replace: bool = False) -> None:
+    """`factory(**params)` builds the part (for "block": the arrangement function)."""
+    if category not in _REGISTRIES:
+        raise ConfigError(f"unknown part category {category!r}; known: {sorted(_REGISTRIES)}")
+    if kind in _REGISTRIES[category] and not replace:
+        raise ConfigError(f"{category} {kind!r} is already registered")
+    _REGISTRIES[category][kind] = factory
+
+
+def unregister_part(category: str, kind: str) -> None:
+    _REGISTRIES[category].pop(kind, None)
+
+
+def build_part(category: str, spec) -> Any:
+    reg = _REGISTRIES[category]
+    if spec.kind not in reg:
+        raise ConfigError(f"unknown {category} {spec.kind!r}; registered: {sorted(reg)}")
+    return reg[spec.kind](**spec.params)
+
+
+def block_arrangement(kind: str):
+    reg = _REGISTRIES["block"]
+    if kind not in reg:
+        raise ConfigError(f"unknown block arrangement {kind!r}; registered: {sorted(reg)}")
+    return reg[kind]()
+
+
+def registered_parts(category: str) -> List[str]:
+    return sorted(_REGISTRIES[category])

@@ -1,0 +1,43 @@
+"""SwiGLU feed-forward: x += W_d (silu(W_g n) * (W_u n)), silu(g) = g / (1 + exp(-g))
+(reference: op_ffn_gate_up_wx and op_ffn_down_res, kernels/megakernel_ops.hip:1474-1553,
+:1559-1602; the activation is fixed to SiLU there, :1538-1544)."""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from .. import kernels as K
+from ..weights import TensorSpec
+from .base import FeedForward, Runtime, register_part
+from .linear import fuse_rows, linear
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.H, self.I = int(hidden_size), int(intermediate_size)
+        self.w_gu = self.w_d = None
+
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        return [
+            TensorSpec(prefix + "gate_proj.weight", (self.I, self.H)),
+            TensorSpec(prefix + "up_proj.weight", (self.I, self.H)),
+            TensorSpec(prefix + "down_proj.weight", (self.H, self.I)),
+        ]
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+        self.w_gu = fuse_rows([tensors[prefix + "gate_proj.weight"], tensors[prefix + "up_proj.weight"]])
+        self.w_d = tensors[prefix + "down_proj.weight"].contiguous()
+
+    def forward(self, h, x, step) -> None:
+        T = step.n_tokens
+        dt = self.rt.dtype
+        gu = step.ws.get("ffn_gu", (T, 2 * self.I), dt)
+        linear(h, self.w_gu, gu, step.ws)
+        a = step.ws.get("ffn_act", (T, self.I), dt)
+        K.silu_mul(gu, a)
+        linear(a, self.w_d, x, step.ws, accumulate=True)
+
+
+register_part("feed_forward", "swiglu", SwiGLU, replace=True)

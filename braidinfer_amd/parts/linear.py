@@ -1,0 +1,45 @@
+"""A projection y = a W^T through the hand-written matrix kernels, for any meeting of
+precisions: bf16 weights take bf16 activations (matrix cores, float accumulation); a
+weight stored in 32-bit stays so and is multiplied in 32-bit, with the activations
+widened for it.  reference: op_linear_proj, kernels/megakernel_ops.hip:166-276 (bf16
+weight, f32 activation, f32 accumulate, no bias)."""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels as K
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, ws, accumulate: bool = False) -> None:
+    """out (+)= a @ w^T.  `accumulate` needs a float32 `out`."""
+    if a.dtype == w.dtype:
+        if a.dtype == torch.float32 or out.dtype == torch.float32 or not accumulate:
+            if a.dtype == torch.float32 and out.dtype != torch.float32:
+                tmp = ws.get("linear_out32", out.shape, torch.float32)
+                K.gemm(a, w, tmp)
+                K.convert(tmp, out)
+                return
+            K.gemm(a, w, out, accumulate)
+            return
+    if w.dtype == torch.float32 and a.dtype == torch.bfloat16:
+        a32 = ws.get("linear_in32", a.shape, torch.float32)
+        if a.is_contiguous():
+            K.convert(a, a32)
+        else:
+            a32.copy_(a)
+        linear(a32, w, out, ws, accumulate)
+        return
+    if w.dtype == torch.bfloat16 and a.dtype == torch.float32:
+        a16 = ws.get("linear_in16", a.shape, torch.bfloat16)
+        K.convert(a.contiguous(), a16)
+        linear(a16, w, out, ws, accumulate)
+        return
+    raise TypeError(f"linear: activations {a.dtype}, weight {w.dtype}")
+
+
+def fuse_rows(mats):
+    """Stack weight matrices along the output dimension so that one product serves all
+    (the reference keeps q/k/v and gate/up separate: three and two launches,
+    megakernel/compile_attention.rs:82-85).  Mixed precisions widen to float32."""
+    dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+    return torch.cat([m.to(dt) for m in mats], dim=0).contiguous()

@@ -1,0 +1,264 @@
+"""The plain implementation: a slow, whole-sequence Mistral forward in NumPy float32,
+written from the reference's formulas, one function per part, no cache, no batching.
+It shares no code with `braidinfer_amd` (it does not import it); tests compare the
+engine with it.
+
+Every function cites where the reference computes the same thing
+(paths under crates/braidinfer-runtime/src/ or kernels/ of mcelrath/braidinfer).
+Where the reference has nothing (sliding window) or deviates from the checkpoint
+format (rotary pairing), the function's docstring says which convention is fixed.
+"""
+import json
+import math
+import os
+import struct
+
+import numpy as np
+
+F = np.float32
+
+
+# ---------------------------------------------------------------- reading a folder ----
+def bf16_bytes_to_f32(raw):
+    """bf16 -> f32 by shifting 16 bits (kernels/bf16_utils.h:7-12)."""
+    u16 = np.frombuffer(raw, dtype="<u2").astype(np.uint32)
+    return (u16 << 16).view(np.float32)
+
+
+def read_folder(folder):
+    """config.json as a dict and every tensor of model.safetensors as float32 arrays
+    (container layout: braidinfer-core/src/safetensors.rs:71-80)."""
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    with open(os.path.join(folder, "model.safetensors"), "rb") as f:
+        (hlen,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(hlen))
+        data = f.read()
+    tensors = {}
+    for name, e in header.items():
+        if name == "__metadata__":
+            continue
+        b, en = e["data_offsets"]
+        raw = data[b:en]
+        if e["dtype"] == "BF16":
+            a = bf16_bytes_to_f32(raw)
+        elif e["dtype"] == "F32":
+            a = np.frombuffer(raw, dtype="<f4")
+        else:
+            raise ValueError(f"dtype {e['dtype']} of {name}")
+        tensors[name] = a.reshape(e["shape"]).astype(F)
+    return cfg, tensors
+
+
+def sizes(cfg):
+    """Keys and defaults as config.rs:208-277 reads them, except tie_word_embeddings
+    (false when absent) and sliding_window (read; config.rs never parses it)."""
+    nq = cfg["num_attention_heads"]
+    return dict(
+        L=cfg["num_hidden_layers"], H=cfg["hidden_size"], nq=nq,
+        nkv=cfg.get("num_key_value_heads", nq), hd=cfg.get("head_dim") or cfg["hidden_size"] // nq,
+        I=cfg["intermediate_size"], V=cfg["vocab_size"], theta=float(cfg.get("rope_theta", 10000.0)),
+        eps=float(cfg.get("rms_norm_eps", 1e-5)), window=cfg.get("sliding_window"),
+        tied=bool(cfg.get("tie_word_embeddings", False)), pairing=cfg.get("rope_pairing", "half"),
+        layer_types=cfg.get("layer_types"))
+
+
+# ------------------------------------------------------------------------ the parts ----
+def embedding(table, tokens):
+    """x[t] = table[token[t]], no scaling (kernels/megakernel_ops.hip:1757-1768)."""
+    return table[np.asarray(tokens, dtype=np.int64)].astype(F)
+
+
+def rms_norm(x, w, eps):
+    """y = x * rsqrt(mean(x^2) + eps) * w; eps inside the root, plain w
+    (kernels/megakernel_ops.hip:862-904)."""
+    x = x.astype(F)
+    ms = (x * x).sum(axis=-1, keepdims=True, dtype=F) / F(x.shape[-1])
+    return (x * (F(1.0) / np.sqrt(ms + F(eps))) * w.astype(F)).astype(F)
+
+
+def linear(x, W):
+    """y = x W^T, W stored [out, in], no bias (kernels/megakernel_ops.hip:166-276)."""
+    return (x.astype(F) @ W.astype(F).T).astype(F)
+
+
+def rope_inv_freq(rotary_dim, theta):
+    """inv_freq[p] = 1 / theta^(2p / rotary_dim) in f32 (weights.rs:743-751)."""
+    p = np.arange(rotary_dim // 2, dtype=F)
+    expo = (F(2.0) * p / F(rotary_dim)).astype(F)
+    return (F(1.0) / np.power(F(theta), expo, dtype=F)).astype(F)
+
+
+def rope(x, positions, inv_freq, pairing):
+    """Rotate pairs of each head by theta = f32(pos) * inv_freq[p]:
+    a' = a cos - b sin, b' = a sin + b cos (kernels/megakernel_ops.hip:2019-2030).
+    pairing "adjacent": (2p, 2p+1), as that kernel does; "half": (p, p + rd/2), the
+    layout of MistralForCausalLM checkpoints (the convention the engine defaults to).
+    x: [T, heads, hd]; only the first rd = 2 len(inv_freq) elements are rotated."""
+    T, nh, hd = x.shape
+    P = inv_freq.shape[0]
+    th = (np.asarray(positions, dtype=F)[:, None] * inv_freq[None, :]).astype(F)   # [T, P]
+    c, s = np.cos(th).astype(F)[:, None, :], np.sin(th).astype(F)[:, None, :]
+    out = x.astype(F).copy()
+    if pairing == "adjacent":
+        a, b = x[..., 0:2 * P:2], x[..., 1:2 * P:2]
+        out[..., 0:2 * P:2] = a * c - b * s
+        out[..., 1:2 * P:2] = a * s + b * c
+    else:
+        a, b = x[..., :P], x[..., P:2 * P]
+        out[..., :P] = a * c - b * s
+        out[..., P:2 * P] = a * s + b * c
+    return out.astype(F)
+
+
+def attention(q, k, v, nq, nkv, window=None, scale=None):
+    """softmax over the keys a query may see of (q . k_j) * rsqrt(hd), times v
+    (kernels/megakernel_ops.hip:2192-2194 kv head = q head / (nq/nkv) and the scale,
+    :2310-2342 the softmax; causality is the loop bound j <= i, compile_attention.rs:285).
+    Window W (ours; the reference has none): query i sees keys j with i - W < j <= i.
+    q: [T, nq, hd], k, v: [T, nkv, hd] -> [T, nq, hd]."""
+    T, _, hd = q.shape
+    scale = F(1.0 / math.sqrt(hd)) if scale is None else F(scale)
+    out = np.zeros((T, nq, hd), dtype=F)
+    g = nq // nkv
+    i = np.arange(T)[:, None]
+    j = np.arange(T)[None, :]
+    allowed = j <= i
+    if window is not None:
+        allowed &= j > i - window
+    for h in range(nq):
+        kh = h // g
+        s = (q[:, h, :].astype(F) @ k[:, kh, :].astype(F).T) * scale          # [T, T]
+        s = np.where(allowed, s, F(-np.inf))
+        m = s.max(axis=-1, keepdims=True)
+        e = np.exp(s - m, dtype=F)
+        p = e / e.sum(axis=-1, keepdims=True, dtype=F)
+        out[:, h, :] = p.astype(F) @ v[:, kh, :].astype(F)
+    return out
+
+
+def silu(x):
+    """silu(g) = g / (1 + exp(-g)) (kernels/megakernel_ops.hip:374-407)."""
+    x = x.astype(F)
+    return (x / (F(1.0) + np.exp(-x, dtype=F))).astype(F)
+
+
+def swiglu(n, Wg, Wu, Wd):
+    """W_d (silu(W_g n) * (W_u n)) (kernels/megakernel_ops.hip:1538-1544, :1559-1602)."""
+    return linear(silu(linear(n, Wg)) * linear(n, Wu), Wd)
+
+
+def attention_block(x, positions, w, prefix, sz, window):
+    """x + W_o attn(rope(W_q n), rope(W_k n), W_v n), n = norm(x)
+    (megakernel/compile_attention.rs:78-376)."""
+    T = x.shape[0]
+    n = rms_norm(x, w[prefix + "input_layernorm.weight"], sz["eps"])
+    q = linear(n, w[prefix + "self_attn.q_proj.weight"]).reshape(T, sz["nq"], sz["hd"])
+    k = linear(n, w[prefix + "self_attn.k_proj.weight"]).reshape(T, sz["nkv"], sz["hd"])
+    v = linear(n, w[prefix + "self_attn.v_proj.weight"]).reshape(T, sz["nkv"], sz["hd"])
+    inv = rope_inv_freq(sz["hd"], sz["theta"])
+    q, k = rope(q, positions, inv, sz["pairing"]), rope(k, positions, inv, sz["pairing"])
+    o = attention(q, k, v, sz["nq"], sz["nkv"], window).reshape(T, sz["nq"] * sz["hd"])
+    return (x + linear(o, w[prefix + "self_attn.o_proj.weight"])).astype(F)
+
+
+def ffn_block(x, w, prefix, sz):
+    """x + swiglu(norm(x)) (megakernel/compile_layers.rs:373-386)."""
+    n = rms_norm(x, w[prefix + "post_attention_layernorm.weight"], sz["eps"])
+    return (x + swiglu(n, w[prefix + "mlp.gate_proj.weight"], w[prefix + "mlp.up_proj.weight"],
+                       w[prefix + "mlp.down_proj.weight"])).astype(F)
+
+
+def layer_window(sz, i):
+    if sz["window"] is None:
+        return None
+    if sz["layer_types"] is None:
+        return sz["window"]
+    return sz["window"] if sz["layer_types"][i] == "sliding_attention" else None
+
+
+def forward(cfg, w, tokens, positions=None):
+    """Logits [T, V] of one whole sequence (layer loop megakernel/megakernel_compile.rs:115-236;
+    final norm and lm_head :238-262)."""
+    sz = sizes(cfg)
+    T = len(tokens)
+    positions = np.arange(T) if positions is None else np.asarray(positions)
+    x = embedding(w["model.embed_tokens.weight"], tokens)
+    for i in range(sz["L"]):
+        p = f"model.layers.{i}."
+        x = attention_block(x, positions, w, p, sz, layer_window(sz, i))
+        x = ffn_block(x, w, p, sz)
+    n = rms_norm(x, w["model.norm.weight"], sz["eps"])
+    head = w["model.embed_tokens.weight"] if sz["tied"] else w["lm_head.weight"]
+    return linear(n, head)
+
+
+# ------------------------------------------------------------------------- sampling ----
+def argmax_lowest(v):
+    """Index of the maximum; the lowest index wins ties (the engine's stated rule; the
+    reference's host argmax keeps the last, generate.rs:493-500)."""
+    return int(np.argmax(np.asarray(v)))
+
+
+def sample(logits, u, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, repetition_penalty=1.0,
+           history=(), logit_bias=None):
+    """The reference's sampler in its order (sampling.rs:49-171), with the uniform draw
+    `u` given.  Sorting is stable by (value descending, index ascending)."""
+    l = np.array(logits, dtype=F)
+    n = l.shape[0]
+    if logit_bias:
+        for tok, d in logit_bias:
+            if 0 <= tok < n:
+                l[tok] = F(l[tok] + F(d))
+    if repetition_penalty != 1.0:
+        for tok in history:
+            if 0 <= tok < n:
+                l[tok] = F(l[tok] / F(repetition_penalty)) if l[tok] > 0 else F(l[tok] * F(repetition_penalty))
+    if temperature == 0.0:
+        return argmax_lowest(l)
+    l = (l / F(temperature)).astype(F)
+    order = sorted(range(n), key=lambda i: (-l[i], i))
+    if 0 < top_k < n:
+        for i in order[top_k:]:
+            l[i] = -np.inf
+    if min_p > 0.0:
+        mx = l.max()
+        for i in range(n):
+            if l[i] > -np.inf and np.exp(F(l[i] - mx), dtype=F) < F(min_p):
+                l[i] = -np.inf
+    if top_p < 1.0:
+        idx = [i for i in order if l[i] > -np.inf]
+        mx = l[idx[0]]
+        pr = np.array([np.exp(F(l[i] - mx), dtype=F) for i in idx], dtype=F)
+        pr = pr / pr.sum(dtype=F)
+        cum, cut = F(0), len(idx)
+        for r, p in enumerate(pr):
+            cum = F(cum + p)
+            if cum >= F(top_p):
+                cut = r + 1
+                break
+        for i in idx[cut:]:
+            l[i] = -np.inf
+    mx = l.max()
+    pr = np.exp((l - mx).astype(F), dtype=F)
+    pr = pr / pr.sum(dtype=F)
+    cum = F(0)
+    for i in range(n):
+        cum = F(cum + pr[i])
+        if F(u) <= cum:
+            return i
+    return argmax_lowest(pr)
+
+
+def greedy_generate(cfg, w, prompt, max_new_tokens, stop_ids=()):
+    """The reference's loop (generate.rs:314-439): argmax of the prompt's last logits,
+    then one token at a time; a stop token ends the sequence and is not emitted."""
+    toks = list(prompt)
+    out = []
+    for _ in range(max_new_tokens):
+        nxt = argmax_lowest(forward(cfg, w, toks)[-1])
+        if nxt in stop_ids:
+            break
+        out.append(nxt)
+        toks.append(nxt)
+    return out
