@@ -11,11 +11,13 @@ from .config import (MistralConfig, preset, PRESETS, config_from_folder, config_
                      register_architecture, registered_architectures, PartSpec, LayerSpec, ScheduleEntry,
                      ModelSpec)
 from .parts import register_part
-from .engine import Engine, StepEntry, DecoderModel
+from .engine import Engine, StepEntry, DecoderModel, generate, GenerationResult, GenerationStats
+from .sampling import SamplingParams, Sampler
 
 __version__ = "0.1.0"
 
 __all__ = ["BraidError", "ConfigError", "WeightError", "CacheError", "KernelError", "StepError",
            "MistralConfig", "preset", "PRESETS", "config_from_folder", "config_from_dict", "spec_of",
            "register_architecture", "registered_architectures", "PartSpec", "LayerSpec", "ScheduleEntry",
-           "ModelSpec", "register_part", "Engine", "StepEntry", "DecoderModel"]
+           "ModelSpec", "register_part", "Engine", "StepEntry", "DecoderModel", "generate", "GenerationResult",
+           "GenerationStats", "SamplingParams", "Sampler"]

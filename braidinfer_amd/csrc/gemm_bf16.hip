@@ -1,0 +1,288 @@
+// bf16 matrix products on the gfx950 matrix cores: C[M,N] (+)= A[M,K] * W[N,K]^T with
+// bf16 inputs, float accumulation, and a bf16 or float output.  W is a weight matrix as
+// checkpoints store it ([out, in], row-major), so both operands are read along k.
+//
+// Two kernels:
+//  * gemm_tile: LDS-staged tiles for many rows (prompts): 4 waves, each a TM x TN grid of
+//    v_mfma_f32_32x32x16_bf16 blocks; global loads of the next k-tile are issued before the
+//    current one is multiplied and written to the other LDS buffer after it.
+//  * gemm_skinny: M <= 64 rows (decode): pure weight streaming.  A workgroup owns 16*RB
+//    weight rows; its 4 waves take interleaved 128-element k-chunks, every lane reading
+//    64 contiguous bytes of one weight row per chunk straight into v_mfma_f32_16x16x32_bf16
+//    operands (the k-permutation inside a chunk is the same for both operands, so the dot
+//    product is unchanged); the waves' partial sums are added in wave order in LDS.
+//
+// reference: op_linear_proj (GEMV per output row, kernels/megakernel_ops.hip:166-276) for
+// what is computed; wmma_gemm_bf16 (kernels/wmma_gemm_bf16.hip:27-82, one wave32 per 16x16
+// tile without LDS, used only by its tests) for the matrix-core form on RDNA3.
+#include "common.h"
+
+// output modes
+#define OUT_BF16 0
+#define OUT_F32 1
+#define OUT_F32_ACC 2
+
+template <int MODE>
+__device__ __forceinline__ void store_out(void* C, size_t idx, float v) {
+    if (MODE == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
+    else if (MODE == OUT_F32) ((float*)C)[idx] = v;
+    else ((float*)C)[idx] += v;
+}
+
+__device__ __forceinline__ bf16x8 zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+    return z;
+}
+
+// 8 consecutive bf16 of row `row` at k; zeros outside [0,rows) x [0,K).
+template <bool ALIGNED>
+__device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, size_t ld, int row, int rows, int k, int K) {
+    if (row >= rows || k >= K) return zero8();
+    const bf16* p = base + (size_t)row * ld + k;
+    if (ALIGNED) {
+        if (k + 8 <= K) return *(const bf16x8*)p;
+    }
+    bf16x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (k + i < K) ? p[i] : (bf16)0.f;
+    return v;
+}
+
+// ------------------------------------------------------------------ gemm_tile -------
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MODE, bool ALIGNED>
+__global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                        void* __restrict__ C, int M, int N, int K,
+                                                        size_t lda, size_t ldc, int tiles_m, int tiles_n) {
+    static_assert(WAVES_M * WAVES_N == 4, "4 waves");
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;      // per-wave tile
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int LDS_LD = BK + 8;                           // padded row, in bf16
+    constexpr int A_CHUNKS = BM * BK / 8 / 256, B_CHUNKS = BN * BK / 8 / 256;
+    constexpr int CPR = BK / 8;                              // 16-byte chunks per tile row
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    bf16* As = (bf16*)smem;                                  // [2][BM][LDS_LD]
+    bf16* Bs = As + 2 * BM * LDS_LD;                         // [2][BN][LDS_LD]
+
+    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of
+    // tiles (n-major, m inner) so that the workgroups sharing an L2 share weight tiles.
+    const int total = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = total / 8, xcd = pid % 8, idx = pid / 8;
+        if (pid < per * 8) pid = xcd * per + idx;
+    }
+    const int tile_n = pid / tiles_m, tile_m = pid - tile_n * tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
+    const int lrow = lane & 31, lk = (lane >> 5) * 8;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    bf16x8 ra[A_CHUNKS], rb[B_CHUNKS];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; ++c) {
+            const int id = tid + c * 256, r = id / CPR, kc = (id % CPR) * 8;
+            ra[c] = load8<ALIGNED>(A, lda, m0 + r, M, k0 + kc, K);
+        }
+#pragma unroll
+        for (int c = 0; c < B_CHUNKS; ++c) {
+            const int id = tid + c * 256, r = id / CPR, kc = (id % CPR) * 8;
+            rb[c] = load8<ALIGNED>(W, (size_t)K, n0 + r, N, k0 + kc, K);
+        }
+    };
+    auto sstore = [&](int buf) {
+        bf16* a = As + buf * BM * LDS_LD;
+        bf16* b = Bs + buf * BN * LDS_LD;
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; ++c) {
+            const int id = tid + c * 256, r = id / CPR, kc = (id % CPR) * 8;
+            *(bf16x8*)(a + r * LDS_LD + kc) = ra[c];
+        }
+#pragma unroll
+        for (int c = 0; c < B_CHUNKS; ++c) {
+            const int id = tid + c * 256, r = id / CPR, kc = (id % CPR) * 8;
+            *(bf16x8*)(b + r * LDS_LD + kc) = rb[c];
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+    gload(0);
+    sstore(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+        const bf16* a = As + buf * BM * LDS_LD + (wm + lrow) * LDS_LD + lk;
+        const bf16* b = Bs + buf * BN * LDS_LD + (wn + lrow) * LDS_LD + lk;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            bf16x8 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = *(const bf16x8*)(a + i * 32 * LDS_LD + kk);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = *(const bf16x8*)(b + j * 32 * LDS_LD + kk);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) sstore(buf ^ 1);
+        __syncthreads();
+    }
+
+    // acc[i][j][r]: row = 8 (r / 4) + 4 (lane / 32) + r % 4, column = lane % 32 of the block
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn + j * 32 + (lane & 31);
+            if (n >= N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < M) store_out<MODE>(C, (size_t)m * ldc + n, acc[i][j][r]);
+            }
+        }
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                       int mode, bool aligned, hipStream_t s) {
+    const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    const long long total = (long long)tm * tn;
+    if (total > 0x7fffffffLL) return BR_BAD_ARG;
+    const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
+#define BR_LAUNCH_TILE(MODE, AL)                                                                        \
+    do {                                                                                                \
+        auto kern = gemm_tile_kernel<BM, BN, BK, WAVES_M, WAVES_N, MODE, AL>;                           \
+        if (lds > 48 * 1024) {                                                                          \
+            static bool set = false;                                                                    \
+            if (!set) {                                                                                 \
+                if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                        (int)lds) != hipSuccess) return BR_LAUNCH_FAILED;               \
+                set = true;                                                                             \
+            }                                                                                           \
+        }                                                                                               \
+        kern<<<(unsigned)total, 256, lds, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);                     \
+    } while (0)
+    if (aligned) {
+        if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16, true);
+        else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32, true);
+        else BR_LAUNCH_TILE(OUT_F32_ACC, true);
+    } else {
+        if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16, false);
+        else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32, false);
+        else BR_LAUNCH_TILE(OUT_F32_ACC, false);
+    }
+#undef BR_LAUNCH_TILE
+    return br_check_launch();
+}
+
+// ----------------------------------------------------------------- gemm_skinny ------
+// grid = ceil(N / (16 RB)); block = 256 (4 waves).  Needs K % 8 == 0 and 16-byte aligned rows.
+template <int MB, int RB, int MODE>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                          void* __restrict__ C, int M, int N, int K,
+                                                          size_t lda, size_t ldc) {
+    constexpr int ROWS = 16 * RB, COLS = 16 * MB;
+    __shared__ float red[4][ROWS][COLS + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+
+    f32x4 acc[RB][MB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+    const int nchunks = (K + 127) / 128;
+    for (int c = wave; c < nchunks; c += 4) {
+        const int kb = c * 128 + g * 32;
+        bf16x8 fw[RB][4], fx[MB][4];
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) fw[i][s] = load8<true>(W, (size_t)K, n0 + i * 16 + r16, N, kb + s * 8, K);
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) fx[j][s] = load8<true>(A, lda, j * 16 + r16, M, kb + s * 8, K);
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+                for (int j = 0; j < MB; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i][s], fx[j][s], acc[i][j], 0, 0, 0);
+    }
+    // acc[i][j][r]: weight row = 16 i + 4 (lane / 16) + r, batch row = 16 j + lane % 16
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * g + r][j * 16 + r16] = acc[i][j][r];
+    __syncthreads();
+    for (int e = tid; e < ROWS * COLS; e += 256) {
+        const int m = e / ROWS, nl = e - m * ROWS;   // consecutive threads: consecutive weight rows
+        const int n = n0 + nl;
+        if (m < M && n < N) {
+            const float v = ((red[0][nl][m] + red[1][nl][m]) + red[2][nl][m]) + red[3][nl][m];
+            store_out<MODE>(C, (size_t)m * ldc + n, v);
+        }
+    }
+}
+
+template <int MB, int RB>
+static int launch_skinny(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                         int mode, hipStream_t s) {
+    const unsigned grid = (unsigned)((N + 16 * RB - 1) / (16 * RB));
+    if (mode == OUT_BF16) gemm_skinny_kernel<MB, RB, OUT_BF16><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else if (mode == OUT_F32) gemm_skinny_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else gemm_skinny_kernel<MB, RB, OUT_F32_ACC><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    return br_check_launch();
+}
+
+// kernel: 0 = choose, 1 = tile 128x128, 2 = tile 256x128, 3 = skinny (tests force one)
+extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
+                               size_t ldc, int mode, int kernel, hipStream_t s) {
+    if (M <= 0 || N <= 0) return BR_OK;
+    if (K <= 0 || lda < (size_t)K || ldc < (size_t)N || mode < 0 || mode > 2) return BR_BAD_ARG;
+    const bf16* A = (const bf16*)A_;
+    const bf16* W = (const bf16*)W_;
+    const bool aligned = (K % 8 == 0) && (lda % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
+    if (kernel == 3 && (!aligned || M > 64)) return BR_BAD_ARG;
+    if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : ((M >= 1024 && N >= 1024) ? 2 : 1);
+    if (kernel == 3) {
+        // rows per workgroup: keep at least ~2 workgroups per CU when N allows it
+        const bool wide = N >= 16384;
+        if (M <= 16) return wide ? launch_skinny<1, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                 : launch_skinny<1, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
+        if (M <= 32) return wide ? launch_skinny<2, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                 : launch_skinny<2, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
+        return wide ? launch_skinny<4, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
+                    : launch_skinny<4, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
+    }
+    if (kernel == 2) return launch_tile<256, 128, 32, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, aligned, s);
+    return launch_tile<128, 128, 64, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, aligned, s);
+}
+
+extern "C" int br_gemm_bf16(const void* A, const void* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                            int mode, hipStream_t s) {
+    return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, s);
+}

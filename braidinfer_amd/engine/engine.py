@@ -86,9 +86,11 @@ class Engine:
         model = DecoderModel(spec_of(config))
         rt = Runtime(device=device, dtype=parse_dtype(dtype))
         tensors = {}
-        for name, t in random_tensors(model.weight_specs(), seed, device, torch.bfloat16, std):
-            kind_vec = t.dim() == 1
-            tensors[name] = t.to(torch.float32) if (kind_vec or rt.dtype == torch.float32) else t
+        specs = model.weight_specs()
+        kinds = {sp.name: sp.kind for sp in specs}
+        for name, t in random_tensors(specs, seed, device, torch.bfloat16, std):
+            widen = kinds[name] == "vector" or rt.dtype == torch.float32
+            tensors[name] = t.to(torch.float32) if (widen and kinds[name] != "int") else t
         model.load(tensors, rt)
         return cls(config, model, rt, max_tokens, max_seq_len, n_slots)
 
@@ -144,3 +146,24 @@ class Engine:
         logits = self.model.forward(step, self.cache, want_rows, n_want)
         self.cache.commit(slots, new)
         return logits
+
+    # ---- generation (the Python entry point) -----------------------------------------------
+    def generate(self, prompts, max_new_tokens: int = 64, temperature: float = 0.0, seed=None,
+                 stop_token_ids=None, top_k: int = 0, top_p: float = 1.0, min_p: float = 0.0,
+                 repetition_penalty: float = 1.0, logit_bias=None, include_stop: bool = False,
+                 max_batch=None, return_stats: bool = False):
+        """Token ids in, generated token ids out: `prompts` is one list of ids or a list of
+        such lists.  Sampling options carry the reference's names (sampling.rs:7-19);
+        temperature 0 is greedy.  Returns the new tokens of each prompt (and the
+        throughput statistics with `return_stats`)."""
+        from ..sampling import SamplingParams
+        from .generate import generate as _generate
+        single = bool(prompts) and isinstance(prompts[0], int)
+        plist = [list(prompts)] if single else [list(p) for p in prompts]
+        params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p,
+                                repetition_penalty=repetition_penalty, seed=seed, min_p=min_p,
+                                logit_bias=logit_bias)
+        results, stats = _generate(self, plist, params, max_new_tokens, stop_token_ids, include_stop, max_batch)
+        toks = [r.tokens for r in results]
+        out = toks[0] if single else toks
+        return (out, stats) if return_stats else out

@@ -165,13 +165,15 @@ def convert(a: torch.Tensor, out: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------------ GEMM ------
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, kernel: int = 0) -> None:
     """out[M, N] (+)= a[M, K] @ w[N, K]^T.
 
     float32 a and w: the true 32-bit kernel (out float32).  bfloat16 a and w: the
     matrix-core kernels with float accumulation; out is bfloat16, or float32 (and may
     then accumulate, which is how a projection adds into the residual stream).
     Rows of `a` and `out` may be strided (a view of a wider buffer); w is contiguous.
+    `kernel` forces one bf16 kernel (1: 128x128 tiles, 2: 256x128 tiles, 3: skinny, for
+    M <= 64); 0 chooses by shape.
     """
     name = "gemm"
     for t in (a, w, out):
@@ -195,8 +197,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             mode = 2 if accumulate else 1
         else:
             raise KernelError(f"gemm: output dtype {out.dtype}")
-        f = _fn("gemm_bf16", "br_gemm_bf16", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P])
-        _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, mode, _stream()), name)
+        f = _fn("gemm_bf16", "br_gemm_bf16_ex", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P])
+        _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, mode, kernel, _stream()), name)
     else:
         raise KernelError(f"gemm: a is {a.dtype} and w is {w.dtype}; both float32 or both bfloat16")
 

@@ -1,0 +1,163 @@
+"""The generation loop's decisions, with a stand-in engine that needs no GPU: batches,
+stop tokens, budgets, sequences that end earlier, slots given back."""
+import pytest
+import torch
+
+from braidinfer_amd.engine import generate, plan_batches
+from braidinfer_amd.errors import CacheError, StepError
+from braidinfer_amd.sampling import SamplingParams, uniform
+
+
+class FakeCache:
+    def __init__(self, n_pages, page_tokens=64, max_seq_len=None, n_slots=None):
+        self.n_pages, self.page_tokens = n_pages, page_tokens
+        self.max_seq_len = max_seq_len or n_pages * page_tokens
+        self.n_slots = n_slots or n_pages
+
+
+class FakeSpec:
+    stop_token_ids = [0]
+    vocab_size = 50
+
+
+class FakeEngine:
+    """Next token = (last token + 1) % V: every sequence counts upwards."""
+
+    def __init__(self, n_pages=32, **kw):
+        self.cache = FakeCache(n_pages, **kw)
+        self.spec = FakeSpec()
+        self.vocab_size = 50
+        self.device = "cpu"
+        self.live = {}
+        self.next_slot = 0
+        self.steps = []            # (slots, number of tokens each) per step
+        self.max_live = 0
+
+    def alloc_slot(self):
+        s = self.next_slot
+        self.next_slot += 1
+        self.live[s] = 0
+        self.max_live = max(self.max_live, len(self.live))
+        return s
+
+    def free_slot(self, s):
+        assert s in self.live, "slot freed twice"
+        del self.live[s]
+
+    def length(self, s):
+        return self.live[s]
+
+    def step(self, entries):
+        self.steps.append(([e.slot for e in entries], [len(e.tokens) for e in entries]))
+        rows = []
+        for e in entries:
+            assert e.slot in self.live
+            self.live[e.slot] += len(e.tokens)
+            for w in e.want:
+                row = torch.zeros(50)
+                row[(e.tokens[w] + 1) % 50] = 1.0
+                rows.append(row)
+        return torch.stack(rows)
+
+
+class ArgmaxSampler:
+    def sample(self, logits, params, histories, us):
+        return [int(r.argmax()) for r in logits]
+
+
+def run(engine, prompts, **kw):
+    return generate(engine, prompts, sampler=ArgmaxSampler(), **kw)
+
+
+def test_counts_upwards_until_the_budget():
+    e = FakeEngine()
+    res, stats = run(e, [[5, 6, 7]], max_new_tokens=4, stop_token_ids=[])
+    assert res[0].tokens == [8, 9, 10, 11] and res[0].finish_reason == "length" and res[0].prompt_tokens == 3
+    assert e.steps[0] == ([0], [3]) and all(s == ([0], [1]) for s in e.steps[1:])
+    assert len(e.steps) == 4            # the prompt step gives the first token; no step after the last
+    assert stats.prefill_tokens == 3 and stats.decode_tokens == 3 and not e.live
+
+
+def test_stop_token_ends_without_being_emitted():
+    e = FakeEngine()
+    res, _ = run(e, [[46]], max_new_tokens=10)             # model's stop token is 0
+    assert res[0].tokens == [47, 48, 49] and res[0].finish_reason == "stop"
+    res, _ = run(e, [[46]], max_new_tokens=10, include_stop=True)
+    assert res[0].tokens == [47, 48, 49, 0]
+    res, _ = run(e, [[49]], max_new_tokens=10)             # the very first token stops
+    assert res[0].tokens == [] and res[0].finish_reason == "stop"
+
+
+def test_shorter_sequences_leave_the_batch_and_give_their_slot_back():
+    e = FakeEngine()
+    res, _ = run(e, [[40], [47], [10, 11]], max_new_tokens=5, stop_token_ids=[0])
+    assert res[0].tokens == [41, 42, 43, 44, 45] and res[1].tokens == [48, 49] and res[2].tokens == [12, 13, 14, 15, 16]
+    sizes = [len(s[0]) for s in e.steps]
+    assert sizes == [3, 3, 3, 2, 2]     # request 1 stops on its third token and leaves before the fourth step
+    assert e.steps[0][1] == [1, 1, 2] and not e.live
+
+
+def test_batches_run_one_after_another_when_the_cache_is_small():
+    e = FakeEngine(n_pages=2)            # two pages: two short requests at a time
+    res, stats = run(e, [[1], [2], [3], [4], [5]], max_new_tokens=3, stop_token_ids=[])
+    assert [r.tokens for r in res] == [[2, 3, 4], [3, 4, 5], [4, 5, 6], [5, 6, 7], [6, 7, 8]]
+    assert stats.batches == 3 and e.max_live == 2 and not e.live
+
+
+def test_empty_prompt_and_zero_budget():
+    e = FakeEngine()
+    res, _ = run(e, [[], [3]], max_new_tokens=2, stop_token_ids=[])
+    assert res[0].tokens == [] and res[0].finish_reason == "empty" and res[1].tokens == [4, 5]
+    res, _ = run(e, [[3]], max_new_tokens=0)
+    assert res[0].tokens == [] and e.live == {}
+
+
+def test_context_limit_is_a_reason():
+    e = FakeEngine(n_pages=4, max_seq_len=6)
+    res, _ = run(e, [[1, 2, 3, 4]], max_new_tokens=10, stop_token_ids=[])
+    # the cache takes 6 tokens: prompt 4, then tokens 5 and 6 are fed; the third new token is the last
+    assert res[0].finish_reason == "context" and res[0].tokens == [5, 6, 7]
+
+
+def test_slots_are_returned_when_a_step_fails():
+    e = FakeEngine()
+    def boom(entries):
+        raise StepError("no")
+    e.step = boom
+    with pytest.raises(StepError):
+        run(e, [[1], [2]], max_new_tokens=2)
+    assert not e.live
+
+
+def test_plan_batches():
+    assert plan_batches([5, 9, 12], 8, 64 * 3, 4096) == [[0, 1, 2]]
+    assert plan_batches([5, 9, 12], 8, 64 * 2, 4096) == [[0, 1], [2]]
+    assert plan_batches([60, 60], 8, 64 * 3, 4096) == [[0], [1]]          # 68 tokens need two pages each
+    assert plan_batches([1, 1, 1, 1], 1, 64 * 8, 4096, max_batch=3) == [[0, 1, 2], [3]]
+    assert plan_batches([1, 1, 1], 1, 64 * 8, 4096, n_slots=2) == [[0, 1], [2]]
+    assert plan_batches([100], 1000, 64 * 2, 128) == [[0]]                # growth is capped by the longest sequence
+    with pytest.raises(CacheError, match="longest"):
+        plan_batches([200], 8, 64 * 8, 128)
+    with pytest.raises(CacheError, match="cache holds"):
+        plan_batches([200], 8, 64 * 2, 4096)
+
+
+def test_one_parameter_set_per_request_or_one_for_all():
+    e = FakeEngine()
+    with pytest.raises(StepError):
+        run(e, [[1], [2]], params=[SamplingParams.greedy()])
+    with pytest.raises(ValueError):
+        run(e, [[1]], params=SamplingParams(top_p=0.0))
+
+
+def test_sampling_defaults_are_the_references():
+    d, g = SamplingParams(), SamplingParams.greedy()
+    assert (d.temperature, d.top_k, d.top_p, d.repetition_penalty, d.seed, d.min_p, d.logit_bias) == (1.0, 50, 1.0, 1.0, None, 0.0, None)
+    assert (g.temperature, g.top_k) == (0.0, 0) and g.is_plain_greedy
+
+
+def test_uniform_numbers_depend_only_on_seed_sequence_and_draw():
+    a = [uniform(7, 3, i) for i in range(1000)]
+    assert a == [uniform(7, 3, i) for i in range(1000)] and all(0.0 <= x < 1.0 for x in a)
+    assert abs(sum(a) / 1000 - 0.5) < 0.05
+    assert uniform(7, 3, 0) != uniform(7, 4, 0) != uniform(8, 3, 0)
