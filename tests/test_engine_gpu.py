@@ -1,0 +1,204 @@
+"""The engine against the plain implementation on the GPU, in 32-bit and in bfloat16,
+under every way of cutting the work: each request alone and whole; with the last 32
+tokens one by one; in batches of unequal lengths whose shorter requests end earlier, one
+batch after another so that slots are used again; long decoding; the first tokens."""
+import numpy as np
+import pytest
+import torch
+
+import braidinfer_amd as B
+import plain_mistral as P
+from braidinfer_amd import StepEntry
+
+pytestmark = pytest.mark.gpu
+
+# Bounds, fixed up front.  32-bit: the engine and the plain implementation differ only in
+# the order of float additions: 1e-4 of the largest logit.  bfloat16: activations, keys and
+# values carry 8 significant bits (relative 2^-9 per rounding), a few dozen roundings deep:
+# 3e-2 of the largest logit, and every position's logits point the same way (cosine).
+TOL = {"float32": 1e-4, "bfloat16": 3e-2}
+COS = {"float32": 0.999999, "bfloat16": 0.999}
+# the same position through different cuts, both from the engine: equal in 32-bit (the
+# 32-bit kernels add in an order that does not depend on the cut), rounding apart in bf16
+CUT_TOL = {"float32": 0.0, "bfloat16": 2e-2}
+
+
+def tokens(cfg, n, seed):
+    return [int(t) for t in np.random.default_rng(seed).integers(0, cfg["vocab_size"], n)]
+
+
+def close(got, want, dtype, what=""):
+    got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite logits"
+    scale = np.abs(want).max()
+    err = np.abs(got - want).max()
+    assert err <= TOL[dtype] * scale, f"{what}: max error {err:.3e} against {scale:.3e} ({dtype})"
+    cos = (got * want).sum(-1) / (np.linalg.norm(got, axis=-1) * np.linalg.norm(want, axis=-1))
+    assert cos.min() >= COS[dtype], f"{what}: cosine {cos.min():.6f} at position {int(cos.argmin())}"
+
+
+def whole(engine, toks):
+    s = engine.alloc_slot()
+    try:
+        return engine.step([StepEntry(s, toks, list(range(len(toks))))]).cpu().numpy()
+    finally:
+        engine.free_slot(s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_each_request_alone_and_whole(engines, tiny_folders, name, dtype):
+    _, cfg, w = tiny_folders[name]
+    eng = engines(name, dtype)
+    for n, seed in ((1, 0), (7, 1), (64, 2), (65, 3), (200, 4)):
+        toks = tokens(cfg, n, seed)
+        close(whole(eng, toks), P.forward(cfg, w, toks), dtype, f"{name} whole n={n}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_last_32_tokens_one_by_one(engines, tiny_folders, name, dtype):
+    _, cfg, w = tiny_folders[name]
+    eng = engines(name, dtype)
+    toks = tokens(cfg, 150, 10)
+    ref = P.forward(cfg, w, toks)
+    one = whole(eng, toks)
+    s = eng.alloc_slot()
+    n0 = len(toks) - 32
+    parts = [eng.step([StepEntry(s, toks[:n0], list(range(n0)))]).cpu().numpy()]
+    for t in toks[n0:]:
+        parts.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    assert eng.length(s) == len(toks)
+    eng.free_slot(s)
+    cut = np.concatenate(parts)
+    close(cut, ref, dtype, f"{name} last 32 one by one")
+    assert np.abs(cut - one).max() <= CUT_TOL[dtype] * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_unequal_batches_one_after_another(engines, tiny_folders, name, dtype):
+    """Prompts of unequal lengths in one step, then one token each; shorter requests end
+    earlier; three batches on one engine so that slots and pages are used again."""
+    _, cfg, w = tiny_folders[name]
+    eng = engines(name, dtype)
+    free_before = [g.pool.free_count for g in eng.cache.groups]
+    for round_, lens in enumerate(([3, 11, 17, 20], [70, 5, 129, 64, 1], [40, 41])):
+        total = [n + 6 + 3 * i for i, n in enumerate(lens)]        # requests end at different steps
+        seqs = [tokens(cfg, t, 100 * round_ + i) for i, t in enumerate(total)]
+        refs = [P.forward(cfg, w, s) for s in seqs]
+        slots = [eng.alloc_slot() for _ in seqs]
+        got = [[] for _ in seqs]
+        out = eng.step([StepEntry(sl, s[:n], list(range(n))) for sl, s, n in zip(slots, seqs, lens)]).cpu().numpy()
+        o = 0
+        for i, n in enumerate(lens):
+            got[i].append(out[o:o + n]); o += n
+        pos = list(lens)
+        live = list(range(len(seqs)))
+        while live:
+            out = eng.step([StepEntry(slots[i], [seqs[i][pos[i]]], [0]) for i in live]).cpu().numpy()
+            for r, i in enumerate(live):
+                got[i].append(out[r:r + 1]); pos[i] += 1
+            for i in [i for i in live if pos[i] == total[i]]:
+                eng.free_slot(slots[i]); live.remove(i)
+        for i in range(len(seqs)):
+            close(np.concatenate(got[i]), refs[i], dtype, f"{name} batch {round_} request {i}")
+    assert [g.pool.free_count for g in eng.cache.groups] == free_before     # every page came back
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_crosses_pages_and_the_window(engines, tiny_folders, dtype):
+    name = "c"                                     # window 70 on layers 0 and 2, full on 1 and 3
+    _, cfg, w = tiny_folders[name]
+    eng = engines(name, dtype)
+    toks = tokens(cfg, 5 + 300, 20)
+    ref = P.forward(cfg, w, toks)
+    s = eng.alloc_slot()
+    got = [eng.step([StepEntry(s, toks[:5], [4])]).cpu().numpy()]
+    for t in toks[5:]:
+        got.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    gw = eng.cache.groups[0]
+    assert gw.need.window == 70 and gw.pool.held_count <= 3       # pages behind the window went back
+    eng.free_slot(s)
+    close(np.concatenate(got), ref[4:], dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(engines, tiny_folders, dtype):
+    """Positions 0, 1, 2: a one-token prompt, then single tokens (the reference sends a
+    one-token prompt through its decode path, generate.rs:328-329)."""
+    for name in ("a", "b"):
+        _, cfg, w = tiny_folders[name]
+        eng = engines(name, dtype)
+        toks = tokens(cfg, 4, 30)
+        ref = P.forward(cfg, w, toks)
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, [t], [0])]).cpu().numpy() for t in toks]
+        eng.free_slot(s)
+        close(np.concatenate(got), ref, dtype, f"{name} first tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_wanted_places_and_chunked_prompts(engines, tiny_folders, dtype):
+    _, cfg, w = tiny_folders["b"]
+    eng = engines("b", dtype)
+    toks = tokens(cfg, 90, 40)
+    ref = P.forward(cfg, w, toks)
+    a, b = eng.alloc_slot(), eng.alloc_slot()
+    # nothing wanted in the first step; prompts cut at different places in the second
+    out = eng.step([StepEntry(a, toks[:50], []), StepEntry(b, toks[:13], [12, 0])]).cpu().numpy()
+    close(out, ref[[12, 0]], dtype, "wanted places")
+    out = eng.step([StepEntry(a, toks[50:], [39]), StepEntry(b, toks[13:70], [0, 56])]).cpu().numpy()
+    close(out, ref[[89, 13, 69]], dtype, "chunked prompt")
+    eng.free_slot(a); eng.free_slot(b)
+
+
+def test_a_far_key_among_hundreds_is_found(tmp_path):
+    """Random weights give near-uniform attention, which would hide a lost key.  Here the
+    weights are made so that the last token's query matches one early key far more than
+    any other: one head copies that token's value, and its identity shows in the logits."""
+    cfg = B.MistralConfig.from_dict(dict(num_hidden_layers=1, hidden_size=32, num_attention_heads=2,
+                                         num_key_value_heads=1, head_dim=16, intermediate_size=16,
+                                         vocab_size=40, rope_theta=10000.0, rms_norm_eps=1e-5,
+                                         max_position_embeddings=4096))
+    folder = B.Engine.write_random_folder(str(tmp_path / "m"), cfg, seed=1, std=0.02)
+    from braidinfer_amd.weights import SafetensorsFolder, write_safetensors
+    st = SafetensorsFolder(folder)
+    t = {n: st.tensor(n).clone() for n in st.names()}
+    H, hd = 32, 16
+    emb = torch.zeros(40, H)
+    content = torch.randn(40, 8, generator=torch.Generator().manual_seed(0))
+    emb[:, :8] = content / content.norm(dim=-1, keepdim=True) * 8 ** 0.5              # content, equal norms
+    emb[1, 8] = 8.0          # token 1 is the marker: it alone has a large key direction
+    emb[2, 9] = 8.0          # token 2 is the asker: it alone has the matching query direction
+    t["model.embed_tokens.weight"] = emb.bfloat16()
+    q = torch.zeros(2 * hd, H); k = torch.zeros(hd, H); v = torch.zeros(hd, H); o = torch.zeros(H, 2 * hd)
+    # rotary leaves the last pair of each half almost unrotated at these positions (lowest
+    # frequency): put the matching direction there (elements 7 and 15 pair up in "half")
+    q[7, 9] = 6.0; k[7, 8] = 6.0
+    v[:8, :8] = torch.eye(8) * 4
+    o[10:18, :8] = torch.eye(8)
+    for n_, m in (("q", q), ("k", k), ("v", v), ("o", o)):
+        t[f"model.layers.0.self_attn.{n_}_proj.weight"] = m.bfloat16()
+    for n_ in ("gate", "up", "down"):
+        t[f"model.layers.0.mlp.{n_}_proj.weight"] = torch.zeros_like(t[f"model.layers.0.mlp.{n_}_proj.weight"])
+    head = torch.zeros(40, H); head[:, 10:18] = emb[:, :8]
+    t["lm_head.weight"] = head.bfloat16()
+    write_safetensors(f"{folder}/model.safetensors", t.items())
+    pc, pw = P.read_folder(folder)
+    rng = np.random.default_rng(0)
+    for dtype in ("float32", "bfloat16"):
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=1024)
+        for far in (0, 63, 64, 300):
+            toks = [int(x) for x in rng.integers(3, 40, 500)]
+            toks[far] = 1                     # the marker sits `far`; its value is its own content...
+            toks[-1] = 2
+            ref = P.forward(pc, pw, toks)[-1]
+            s = eng.alloc_slot()
+            eng.step([StepEntry(s, toks[:-1], [])])
+            got = eng.step([StepEntry(s, [toks[-1]], [0])]).cpu().numpy()[0]
+            eng.free_slot(s)
+            assert int(ref.argmax()) == 1, "the test's weights must make the marker win in the plain implementation"
+            assert int(got.argmax()) == 1, f"{dtype}: the key at position {far} was lost"
+            close(got[None], ref[None], dtype, f"far key at {far}")

@@ -1,0 +1,93 @@
+"""Generation through the entry points against the plain implementation's greedy loop."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import braidinfer_amd as B
+import plain_mistral as P
+from braidinfer_amd import SamplingParams
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def prompts_of(cfg, lens, seed):
+    rng = np.random.default_rng(seed)
+    return [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in lens]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_matches_the_plain_loop(engines, tiny_folders, dtype):
+    # the first configuration of the benchmark description: prompts of 5, 9 and 12, 8 tokens, greedy
+    _, cfg, w = tiny_folders["a"]
+    eng = engines("a", dtype)
+    prompts = prompts_of(cfg, [5, 9, 12], 0)
+    got = eng.generate(prompts, max_new_tokens=8, temperature=0.0, stop_token_ids=[])
+    want = [P.greedy_generate(cfg, w, p, 8) for p in prompts]
+    if dtype == "float32":
+        assert got == want
+    else:
+        # bf16 may pick the runner-up where two logits are within rounding: the sequences agree
+        # up to the first such place, and there the plain logits are nearly tied
+        for g, wnt, p in zip(got, want, prompts):
+            for i, (a, b) in enumerate(zip(g, wnt)):
+                if a != b:
+                    l = P.forward(cfg, w, p + wnt[:i])[-1]
+                    assert abs(l[a] - l[b]) < 3e-2 * np.abs(l).max()
+                    break
+
+
+def test_stop_tokens_and_unequal_ends(engines, tiny_folders):
+    _, cfg, w = tiny_folders["b"]
+    eng = engines("b", "float32")
+    prompts = prompts_of(cfg, [3, 11, 17, 20], 1)
+    free = [g.pool.free_count for g in eng.cache.groups]
+    plain = [P.greedy_generate(cfg, w, p, 12) for p in prompts]
+    stop = plain[1][4]                                  # a token request 1 meets at its fifth step
+    want = [P.greedy_generate(cfg, w, p, 12, stop_ids=[stop]) for p in prompts]
+    assert len(want[1]) <= 4
+    got, stats = eng.generate(prompts, max_new_tokens=12, stop_token_ids=[stop], return_stats=True)
+    assert got == want
+    assert [g.pool.free_count for g in eng.cache.groups] == free and eng.cache.slots.free_count == eng.cache.n_slots
+    assert stats.prefill_tokens == 51 and "PPTG pp=" in stats.pptg_line()
+
+
+def test_alone_or_in_a_batch_gives_the_same_tokens(engines, tiny_folders):
+    _, cfg, _ = tiny_folders["b"]
+    eng = engines("b", "float32")
+    prompts = prompts_of(cfg, [3, 11, 17, 20], 2)
+    # the second configuration of the benchmark description: 12 tokens at temperature 0.7, seeded
+    kw = dict(max_new_tokens=12, temperature=0.7, seed=1234, top_k=0, stop_token_ids=[])
+    together = eng.generate(prompts, **kw)
+    assert together == eng.generate(prompts, **kw)                       # seeded: the same again
+    assert together != eng.generate(prompts, **{**kw, "seed": 99})
+    assert eng.generate(prompts[0], **kw) == together[0]                 # request 0 alone
+    by_two = eng.generate(prompts, max_batch=2, **kw)                    # two batches, slots used again
+    assert by_two == together
+
+
+def test_command_line(tiny_folders):
+    folder, cfg, w = tiny_folders["a"]
+    p = [7, 3, 200, 5]
+    want = P.greedy_generate(cfg, w, p, 6)
+    env = dict(os.environ, MODEL=folder, MAX_TOKENS="6")
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), "--dtype", "float32",
+                        "--prompt-ids", ",".join(map(str, p))], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    assert [int(t) for t in r.stdout.split()] == want
+    assert "PPTG pp=" in r.stderr and "tokens in" in r.stderr and "stop tokens:" in r.stderr
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), folder, "--dtype", "float32",
+                        "--prompt-ids", "1,2", "--prompt-ids", "3,4,5"],
+                       env={k: v for k, v in env.items() if k != "MODEL"}, capture_output=True, text=True)
+    assert r.returncode == 0 and len(r.stdout.strip().splitlines()) == 2
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), "some words"], env=env,
+                       capture_output=True, text=True)
+    assert r.returncode == 2 and "tokenizer" in r.stderr
+
+
+def test_smoke_entry():
+    import __graft_entry__
+    __graft_entry__.smoke()

@@ -1,0 +1,302 @@
+"""Each HIP kernel alone against a plain float32 expression of the same operation, at
+sizes other than the engine's tiny models (head sizes in steps of 16, widths and
+vocabularies that are no power of two, one row and many)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from braidinfer_amd import kernels as K
+from braidinfer_amd.errors import KernelError
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(v):
+    return torch.tensor(v, dtype=torch.int32, device=DEV)
+
+
+# ------------------------------------------------------------------ embedding ------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding(dtype):
+    # reference vector: V=256, H=1024, token 42 (tests/embedding_test.rs:14-65); exact
+    table = rnd(257, 1000, dtype=dtype)
+    toks = i32([42, 0, 256, 42, 7])
+    out = torch.empty(5, 1000, device=DEV)
+    K.embedding(table, toks, out)
+    assert torch.equal(out, table.float()[toks.long()])
+
+
+# -------------------------------------------------------------------- RMSNorm ------
+@pytest.mark.parametrize("H", [48, 1000, 4096, 5120])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(H, out_dtype):
+    x, w = rnd(7, H, scale=3.0), rnd(H, seed=1) * 0.1 + 1
+    out = torch.empty(7, H, device=DEV, dtype=out_dtype)
+    K.rmsnorm(x, w, out, 1e-6)
+    want = x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-6) * w.double()
+    tol = 1e-5 if out_dtype == torch.float32 else 2e-2
+    assert (out.double() - want).abs().max() < tol * want.abs().max()
+    rows = i32([6, 0, 3])
+    out2 = torch.empty(3, H, device=DEV, dtype=out_dtype)
+    K.rmsnorm(x, w, out2, 1e-6, rows)
+    assert torch.equal(out2, out[rows.long()])
+
+
+def test_rmsnorm_reference_vector():
+    # tests/op_rmsnorm_test.rs:51-66,109: H=1024, 4 rows, eps 1e-6, x = sin(0.01 i), w = bf16(1 + 0.001 i), tol 1e-4
+    H = 1024
+    x = torch.sin(0.01 * torch.arange(4 * H, dtype=torch.float64)).reshape(4, H)
+    w = (1 + 0.001 * torch.arange(H, dtype=torch.float32)).bfloat16().float()
+    out = torch.empty(4, H, device=DEV)
+    K.rmsnorm(x.float().to(DEV), w.to(DEV), out, 1e-6)
+    want = x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-6) * w.double()
+    assert (out.cpu().double() - want).abs().max() < 1e-4
+
+
+# ----------------------------------------------------------------------- GEMM ------
+SHAPES = [(1, 64, 64), (5, 100, 96), (17, 192, 320), (64, 301, 100), (33, 1000, 264), (3, 50, 44),
+          (130, 514, 100), (257, 129, 72), (300, 260, 1032)]
+
+
+@pytest.mark.parametrize("M,N,Kd", SHAPES)
+def test_gemm_f32(M, N, Kd):
+    a, w = rnd(M, Kd, seed=1), rnd(N, Kd, seed=2)
+    out = torch.empty(M, N, device=DEV)
+    K.gemm(a, w, out)
+    want = a.double() @ w.double().T
+    assert (out.double() - want).abs().max() < 1e-5 * want.abs().max()
+    base = rnd(M, N, seed=3)
+    acc = base.clone()
+    K.gemm(a, w, acc, accumulate=True)
+    assert (acc.double() - (base.double() + want)).abs().max() < 1e-5 * want.abs().max()
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch():
+    a, w = rnd(70, 200, seed=1), rnd(90, 200, seed=2)
+    full = torch.empty(70, 90, device=DEV)
+    K.gemm(a, w, full)
+    one = torch.empty(1, 90, device=DEV)
+    K.gemm(a[33:34].contiguous(), w, one)
+    assert torch.equal(one[0], full[33])
+
+
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,N,Kd", SHAPES)
+def test_gemm_bf16(M, N, Kd, kernel):
+    if kernel == 3 and (Kd % 8 or M > 64):
+        pytest.skip("the skinny kernel takes M <= 64 and K in steps of 8")
+    a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
+    want = a.double() @ w.double().T
+    o32 = torch.empty(M, N, device=DEV)
+    K.gemm(a, w, o32, kernel=kernel)
+    assert (o32.double() - want).abs().max() < 1e-4 * want.abs().max()        # exact products, float sums
+    o16 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    K.gemm(a, w, o16, kernel=kernel)
+    assert (o16.double() - want).abs().max() < 1e-2 * want.abs().max()
+    base = rnd(M, N, seed=3)
+    acc = base.clone()
+    K.gemm(a, w, acc, accumulate=True, kernel=kernel)
+    assert (acc.double() - (base.double() + want)).abs().max() < 1e-4 * want.abs().max()
+
+
+def test_gemm_reference_vectors():
+    # tests/wmma_gemm_test.rs:27-69,72-114: sin/cos ramps times 0.5 / 0.3, tol 1e-3
+    for M, N, Kd in ((32, 32, 64), (256, 256, 1024)):
+        a = (0.5 * torch.sin(0.01 * torch.arange(M * Kd))).reshape(M, Kd).bfloat16().to(DEV)
+        w = (0.3 * torch.cos(0.01 * torch.arange(N * Kd))).reshape(N, Kd).bfloat16().to(DEV)
+        out = torch.empty(M, N, device=DEV)
+        K.gemm(a, w, out)
+        assert (out.double() - a.double() @ w.double().T).abs().max() < 1e-3
+
+
+def test_gemm_strided_rows_and_refusals():
+    wide = rnd(20, 300, dtype=torch.bfloat16)
+    a = wide[:, 100:164]                       # a view: rows 600 bytes apart
+    w = rnd(40, 64, seed=5, dtype=torch.bfloat16)
+    out = torch.empty(20, 40, device=DEV)
+    K.gemm(a, w, out)
+    assert (out.double() - a.double() @ w.double().T).abs().max() < 1e-4 * 20
+    with pytest.raises(KernelError):
+        K.gemm(a, rnd(40, 65, dtype=torch.bfloat16), out)
+    with pytest.raises(KernelError):
+        K.gemm(a.float(), w, out)
+    with pytest.raises(KernelError):
+        K.gemm(a.cpu(), w.cpu(), out.cpu())
+
+
+# ------------------------------------------------------------------ rotary, cache ----
+def _rope_ref(x, pos, inv, adjacent):
+    th = pos.double()[:, None] * inv.double()[None, :]
+    c, s = th.cos()[:, None, :], th.sin()[:, None, :]
+    P = inv.numel()
+    y = x.double().clone()
+    if adjacent:
+        a, b = x[..., 0:2 * P:2].double(), x[..., 1:2 * P:2].double()
+        y[..., 0:2 * P:2], y[..., 1:2 * P:2] = a * c - b * s, a * s + b * c
+    else:
+        a, b = x[..., :P].double(), x[..., P:2 * P].double()
+        y[..., :P], y[..., P:2 * P] = a * c - b * s, a * s + b * c
+    return y
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("adjacent", [False, True])
+@pytest.mark.parametrize("nq,nkv,hd,rd", [(8, 2, 256, 64), (5, 5, 48, 48), (4, 1, 80, 80)])
+def test_rope_and_paged_write(dtype, adjacent, nq, nkv, hd, rd):
+    # sizes of tests/mrope_test.rs:5-13 (nq 8, nkv 2, hd 256, rotary 64, theta 1e7) among them;
+    # page/offset cases of tests/op_kv_write_paged_batch_test.rs:196-198: starts 0 and 32, across pages
+    page, theta = 64, 1e7
+    lens, starts = [8, 128, 64], [0, 0, 32]
+    T = sum(lens)
+    pos = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int().to(DEV)
+    sot = torch.cat([torch.full((n,), b) for b, n in enumerate(lens)]).int().to(DEV)
+    slots = i32([2, 0, 3])
+    table = torch.full((4, 4), -1, dtype=torch.int32)
+    table[2, 0], table[0, 0], table[0, 1], table[3, 0], table[3, 1] = 5, 1, 6, 0, 3
+    table = table.to(DEV)
+    inv = (1.0 / theta ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd)).to(DEV)
+    cs, sn = torch.empty(T, rd // 2, device=DEV), torch.empty(T, rd // 2, device=DEV)
+    K.rope_table(pos, inv, cs, sn)
+    th = pos.float()[:, None] * inv[None, :]
+    assert (cs - th.cos()).abs().max() < 2e-6 and (sn - th.sin()).abs().max() < 2e-6
+    qkv = rnd(T, (nq + 2 * nkv) * hd, dtype=dtype)
+    src = qkv.clone()
+    cache = torch.full((8, 2, nkv, page, hd), 99.0, device=DEV, dtype=dtype)
+    K.rope_kv_write(qkv, cs, sn, pos, sot, slots, table, cache, nq, nkv, hd, rd, adjacent, page, True)
+    q_in = src[:, :nq * hd].reshape(T, nq, hd).float()
+    k_in = src[:, nq * hd:(nq + nkv) * hd].reshape(T, nkv, hd).float()
+    v_in = src[:, (nq + nkv) * hd:].reshape(T, nkv, hd)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    q_want, k_want = _rope_ref(q_in, pos, inv, adjacent), _rope_ref(k_in, pos, inv, adjacent)
+    assert (qkv[:, :nq * hd].reshape(T, nq, hd).double() - q_want).abs().max() < tol * q_want.abs().max()
+    assert torch.equal(qkv[:, nq * hd:], src[:, nq * hd:])            # k and v rows of the step buffer are untouched
+    written = torch.zeros(8, page, dtype=torch.bool)
+    for t in range(T):
+        p, slot = int(pos[t]), int(slots[int(sot[t])])
+        pg = int(table[slot, p // page])
+        written[pg, p % page] = True
+        assert (cache[pg, 0, :, p % page].double() - k_want[t]).abs().max() < tol * k_want.abs().max()
+        assert torch.equal(cache[pg, 1, :, p % page], v_in[t])         # values byte-equal
+    untouched = cache[:, :, :, :, :][~written[:, None, None, :].expand(8, 2, nkv, page)]
+    assert torch.all(untouched == 99.0)
+    # a padded sequence (slot -1) stores nothing; write_cache=False stores nothing
+    cache2 = torch.full_like(cache, 99.0)
+    K.rope_kv_write(src.clone(), cs, sn, pos, sot, i32([-1, -1, -1]), table, cache2, nq, nkv, hd, rd, adjacent, page, True)
+    K.rope_kv_write(src.clone(), cs, sn, pos, sot, slots, table, cache2, nq, nkv, hd, rd, adjacent, page, False)
+    assert torch.all(cache2 == 99.0)
+
+
+# ------------------------------------------------------------------ attention ------
+def _attn_ref(q, k, v, nq, nkv, window):
+    T, hd = q.shape[0], q.shape[-1]
+    i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+    mask = j <= i
+    if window:
+        mask &= j > i - window
+    out = torch.zeros(T, nq, hd, dtype=torch.float64)
+    for h in range(nq):
+        s = q[:, h].double() @ k[:, h // (nq // nkv)].double().T / math.sqrt(hd)
+        s = s.masked_fill(~mask, float("-inf"))
+        out[:, h] = torch.softmax(s, -1) @ v[:, h // (nq // nkv)].double()
+    return out
+
+
+def _paged(k, v, pages, page, n_pages, dtype):
+    """Scatter [T, nkv, hd] keys and values into a cache unit through a page list."""
+    T, nkv, hd = k.shape
+    cache = torch.zeros(n_pages, 2, nkv, page, hd, dtype=dtype, device=DEV)
+    for t in range(T):
+        cache[pages[t // page], 0, :, t % page] = k[t]
+        cache[pages[t // page], 1, :, t % page] = v[t]
+    return cache
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,hd,window", [(4, 2, 16, None), (6, 3, 32, 8), (5, 1, 48, 70), (8, 8, 128, None),
+                                              (2, 1, 80, 100), (4, 4, 256, None)])
+def test_attention_simple(dtype, nq, nkv, hd, window):
+    page, T = 64, 150
+    q, k, v = (rnd(T, n, hd, seed=s, dtype=dtype) for s, n in ((1, nq), (2, nkv), (3, nkv)))
+    pages = [7, 2, 9]
+    cache = _paged(k, v, pages, page, 12, dtype)
+    table = torch.full((3, 4), -1, dtype=torch.int32); table[1, :3] = torch.tensor(pages); table = table.to(DEV)
+    pos, sot, slots = torch.arange(T).int().to(DEV), torch.zeros(T).int().to(DEV), i32([1])
+    out = torch.empty(T, nq * hd, device=DEV, dtype=dtype)
+    qf = q.reshape(T, nq * hd).contiguous()
+    K.attention_simple(qf, nq * hd, out, pos, sot, slots, table, cache, T, nq, nkv, hd, page, window, 1 / math.sqrt(hd))
+    want = _attn_ref(q.cpu(), k.cpu(), v.cpu(), nq, nkv, window)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (out.reshape(T, nq, hd).cpu().double() - want).abs().max() < tol * want.abs().max()
+    # the last 20 queries alone (decode-like: queries whose keys were stored earlier)
+    out2 = torch.empty(20, nq * hd, device=DEV, dtype=dtype)
+    K.attention_simple(qf[-20:].contiguous(), nq * hd, out2, pos[-20:].contiguous(), sot[:20].contiguous(), slots, table,
+                       cache, 20, nq, nkv, hd, page, window, 1 / math.sqrt(hd))
+    assert torch.equal(out2, out[-20:])
+
+
+def test_attention_one_key_and_uniform_scores():
+    hd, page = 32, 64
+    k = torch.zeros(5, 1, hd); v = rnd(5, 1, hd, seed=4).cpu()
+    cache = _paged(k.to(DEV), v.to(DEV), [0], page, 1, torch.float32)
+    q = rnd(5, 2 * hd, seed=5)
+    table = i32([[0]])
+    out = torch.empty(5, 2 * hd, device=DEV)
+    K.attention_simple(q, 2 * hd, out, i32([0, 1, 2, 3, 4]), i32([0] * 5), i32([0]), table, cache, 5, 2, 1, hd, page, None, 1.0)
+    o = out.reshape(5, 2, hd).cpu()
+    assert torch.allclose(o[0, 0], v[0, 0], atol=1e-6)                            # one key: its value
+    assert torch.allclose(o[4, 1], v[:, 0].mean(0), atol=1e-6)                    # equal scores: the mean
+
+
+# ----------------------------------------------------------------- elementwise ------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul_and_residual(dtype):
+    # tests/op_silu_mul_test.rs:37-81: g = 3 sin(0.011 i), u = cos(0.009 i), tol 1e-3
+    I = 1025
+    i = torch.arange(3 * I, dtype=torch.float32)
+    g, u = (3 * torch.sin(0.011 * i)).reshape(3, I), torch.cos(0.009 * i).reshape(3, I)
+    gu = torch.cat([g, u], dim=1).to(dtype).to(DEV)
+    out = torch.empty(3, I, device=DEV, dtype=dtype)
+    K.silu_mul(gu, out)
+    gd, ud = gu[:, :I].double(), gu[:, I:].double()
+    want = gd / (1 + torch.exp(-gd)) * ud
+    assert (out.double() - want).abs().max() < (1e-6 if dtype == torch.float32 else 1e-2)
+    x, y = rnd(1000, seed=1), rnd(1000, seed=2, dtype=dtype)
+    want = x + y.float()
+    K.residual_add(x, y)
+    assert torch.equal(x, want)                                                   # tests/op_residual_add_test.rs: exact
+
+
+def test_gather_and_convert():
+    x = rnd(9, 100)
+    out = torch.empty(3, 100, device=DEV)
+    K.gather_rows(x, i32([8, 0, 8]), out)
+    assert torch.equal(out, x[[8, 0, 8]])
+    b = torch.empty(9, 100, device=DEV, dtype=torch.bfloat16)
+    K.convert(x, b)
+    assert torch.equal(b, x.bfloat16())                                           # round to nearest even
+    back = torch.empty_like(x)
+    K.convert(b, back)
+    assert torch.equal(back, b.float())
+
+
+# -------------------------------------------------------------------- sampling ------
+def test_argmax_lowest_index_wins():
+    l = rnd(5, 32768 + 3)
+    l[1, 100] = l[1, 20000] = 50.0
+    l[2, :] = 0.0
+    l[3, 32770] = 60.0
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    K.argmax(l, out)
+    want = [int(l[0].argmax()), 100, 0, 32770, int(l[4].argmax())]
+    assert out.tolist() == want
+    # reference vector: greedy on [0.1, 0.5, 0.2, 0.8, 0.3] -> 3 (sampling.rs:232-241)
+    K.argmax(torch.tensor([[0.1, 0.5, 0.2, 0.8, 0.3]], device=DEV), out)
+    assert out[0].item() == 3

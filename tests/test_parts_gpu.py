@@ -1,0 +1,331 @@
+"""Each part alone on the GPU against the plain implementation's function for it, and
+the generality of the arrangement: a toy mixer with state of its own that is registered,
+built and stepped without a change to the library; a layer run twice; a layer that reads
+another layer's cache."""
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+import braidinfer_amd as B
+import plain_mistral as P
+from braidinfer_amd import StepEntry
+from braidinfer_amd.cache import SequenceCache, StateNeed
+from braidinfer_amd.config import (LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture,
+                                   unregister_architecture)
+from braidinfer_amd.engine import Workspace, pack_step
+from braidinfer_amd.parts import (Mixer, MixerContext, Runtime, build_part, register_part, unregister_part)
+from braidinfer_amd.weights import TensorSpec
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def rt(dtype):
+    return Runtime(DEV, dtype)
+
+
+def bf(a):
+    """Values as the bf16 path stores them."""
+    return torch.tensor(a).bfloat16().float().numpy()
+
+
+def dev(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a, np.float32)).to(dtype).to(DEV)
+
+
+def make_step(lens, starts=None, slots=None):
+    starts = starts or [0] * len(lens)
+    slots = slots if slots is not None else list(range(len(lens)))
+    toks = [[1] * n for n in lens]
+    return pack_step(slots, toks, starts, DEV, Workspace(DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    part = build_part("norm", PartSpec("rmsnorm", {"size": 100, "eps": 3e-6}))
+    assert [(s.name, s.shape, s.kind) for s in part.weight_specs("n.")] == [("n.weight", (100,), "vector")]
+    rng = np.random.default_rng(0)
+    w, x = (1 + 0.3 * rng.normal(size=100)).astype(np.float32), rng.normal(size=(6, 100)).astype(np.float32) * 4
+    part.load({"n.weight": dev(w)}, "n.", rt(dtype))
+    out = torch.empty(6, 100, device=DEV, dtype=dtype)
+    part.forward(dev(x), out)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert np.abs(out.float().cpu().numpy() - P.rms_norm(x, w, 3e-6)).max() < tol * 8
+
+
+@pytest.mark.parametrize("pairing", ["half", "adjacent"])
+def test_position_part_gives_the_plain_angles(pairing):
+    part = build_part("position", PartSpec("rope", {"rotary_dim": 48, "theta": 5e5, "pairing": pairing}))
+    part.load({}, "", rt(torch.float32))
+    assert np.abs(part.inv_freq.cpu().numpy() - P.rope_inv_freq(48, 5e5)).max() < 1e-9
+    step = make_step([5, 3], starts=[100, 4000])
+    tabs = part.prepare(step)
+    pos = np.array([100, 101, 102, 103, 104, 4000, 4001, 4002], np.float32)
+    th = pos[:, None] * P.rope_inv_freq(48, 5e5)[None, :]
+    assert np.abs(tabs.cos.cpu().numpy() - np.cos(th)).max() < 1e-5
+    assert np.abs(tabs.sin.cpu().numpy() - np.sin(th)).max() < 1e-5
+    assert tabs.adjacent == (pairing == "adjacent") and tabs.rotary_dim == 48
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    part = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": 100, "intermediate_size": 172}))
+    rng = np.random.default_rng(1)
+    g, u, d = (bf(rng.normal(size=s).astype(np.float32) * 0.1) for s in ((172, 100), (172, 100), (100, 172)))
+    wdt = dtype
+    part.load({"f.gate_proj.weight": dev(g, wdt), "f.up_proj.weight": dev(u, wdt), "f.down_proj.weight": dev(d, wdt)},
+              "f.", rt(dtype))
+    h = bf(rng.normal(size=(9, 100)).astype(np.float32))
+    x0 = rng.normal(size=(9, 100)).astype(np.float32)
+    x = dev(x0)
+    part.forward(dev(h, dtype), x, make_step([9]))
+    want = x0 + P.swiglu(h, g, u, d)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert np.abs(x.cpu().numpy() - want).max() < tol * np.abs(want).max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 5])
+def test_attention_part_with_its_cache(dtype, window):
+    nq, nkv, hd, H = 6, 3, 32, 96
+    part = build_part("mixer", PartSpec("gqa_attention", {"hidden_size": H, "num_heads": nq, "num_kv_heads": nkv,
+                                                          "head_dim": hd, "window": window, "position": "rope"}))
+    assert part.cache_need() == B.cache.CacheNeed(nkv, hd, window) if hasattr(B, "cache") else True
+    rope = build_part("position", PartSpec("rope", {"rotary_dim": hd, "theta": 1e4, "pairing": "half"}))
+    rng = np.random.default_rng(2)
+    w = {n: bf(rng.normal(size=s).astype(np.float32) * 0.15) for n, s in
+         (("q", (nq * hd, H)), ("k", (nkv * hd, H)), ("v", (nkv * hd, H)), ("o", (H, nq * hd)))}
+    part.load({f"a.{n}_proj.weight": dev(m, dtype) for n, m in w.items()}, "a.", rt(dtype))
+    rope.load({}, "", rt(dtype))
+    cache = SequenceCache({0: part.cache_need()}, {}, max_tokens=256, dtype=dtype, device=DEV)
+    T = 20
+    h = bf(rng.normal(size=(T, H)).astype(np.float32))
+    x0 = rng.normal(size=(T, H)).astype(np.float32)
+    # plain: the attention half of a block without its norm
+    q = P.rope(P.linear(h, w["q"]).reshape(T, nq, hd), np.arange(T), P.rope_inv_freq(hd, 1e4), "half")
+    k = P.rope(P.linear(h, w["k"]).reshape(T, nkv, hd), np.arange(T), P.rope_inv_freq(hd, 1e4), "half")
+    v = P.linear(h, w["v"]).reshape(T, nkv, hd)
+    want = x0 + P.linear(P.attention(q, k, v, nq, nkv, window).reshape(T, nq * hd), w["o"])
+    slot = cache.alloc_slot()
+    got = []
+    for lo, hi in ((0, 13), (13, 14), (14, 20)):          # a prompt, one token, a further chunk
+        cache.reserve([slot], [hi - lo])
+        step = pack_step([slot], [[1] * (hi - lo)], [lo], DEV, Workspace(DEV))
+        step.position_data = {"rope": rope.prepare(step)}
+        g = cache.unit_group(0)
+        ctx = MixerContext(unit=0, storage=g.storage[0], block_table=g.table_dev, page_tokens=g.page_tokens)
+        x = dev(x0[lo:hi])
+        part.forward(dev(h[lo:hi], dtype), x, step, ctx)
+        cache.commit([slot], [hi - lo])
+        got.append(x.cpu().numpy())
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert np.abs(np.concatenate(got) - want).max() < tol * np.abs(want).max()
+
+
+def test_embedding_and_head_parts():
+    emb = build_part("embedding", PartSpec("embedding", {"vocab_size": 301, "hidden_size": 100}))
+    head = build_part("lm_head", PartSpec("lm_head", {"vocab_size": 301, "hidden_size": 100,
+                                                      "tied_to": "e.weight"}))
+    assert head.weight_specs("lm_head.") == [] and head.optional_names("lm_head.") == ["lm_head.weight"]
+    table = bf(np.random.default_rng(3).normal(size=(301, 100)).astype(np.float32))
+    tensors = {"e.weight": dev(table, torch.bfloat16)}
+    emb.load(tensors, "e.", rt(torch.bfloat16))
+    head.load(tensors, "lm_head.", rt(torch.bfloat16))
+    x = torch.empty(4, 100, device=DEV)
+    emb.forward(torch.tensor([300, 0, 17, 17], dtype=torch.int32, device=DEV), x)
+    assert np.array_equal(x.cpu().numpy(), table[[300, 0, 17, 17]])
+    logits = torch.empty(4, 301, device=DEV)
+    head.forward(x.bfloat16(), logits, Workspace(DEV))
+    assert np.abs(logits.cpu().numpy() - table[[300, 0, 17, 17]] @ table.T).max() < 1e-3 * 100
+
+
+# ------------------------------------------------------------- a toy mixer with state ----
+class RunningSumMixer(Mixer):
+    """out[t] = W (sum of the sequence's inputs up to and including t).  Its per-sequence
+    state is the running sum: fixed size, kept in the cache's state area.  It uses torch
+    operations: it is a test's toy, not a part of the library."""
+
+    def __init__(self, hidden_size):
+        self.H = hidden_size
+
+    def weight_specs(self, prefix):
+        return [TensorSpec(prefix + "mix.weight", (self.H, self.H))]
+
+    def load(self, tensors, prefix, rt):
+        self.rt = rt
+        self.w = tensors[prefix + "mix.weight"].float()
+
+    def state_need(self):
+        return StateNeed((self.H,), torch.float32)
+
+    def forward(self, h, x, step, ctx):
+        o = 0
+        for b, n in enumerate(step.host_new):
+            slot = step.host_slots[b]
+            if slot >= 0:
+                c = torch.cumsum(h[o:o + n].float(), 0) + ctx.state[slot]
+                ctx.state[slot] = c[-1]
+                x[o:o + n] += c @ self.w.T
+            o += n
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    hidden_size: int = 40
+    vocab_size: int = 90
+    architecture = "ToyRunningSumForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d["hidden_size"], d["vocab_size"])
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], "hidden_size": self.hidden_size, "vocab_size": self.vocab_size}
+
+
+def toy_spec(cfg):
+    H = cfg.hidden_size
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                      "window": None, "position": "rope"})
+    layers = [
+        LayerSpec("toy.layers.0.", PartSpec("running_sum", {"hidden_size": H}), None, norm, None),
+        LayerSpec("toy.layers.1.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 56}), norm, norm),
+    ]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=cfg.vocab_size,
+                     embedding=PartSpec("embedding", {"vocab_size": cfg.vocab_size, "hidden_size": H}),
+                     layers=layers, schedule=[ScheduleEntry(0, None), ScheduleEntry(1, 0)], final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": cfg.vocab_size, "hidden_size": H, "tied_to": None}),
+                     positions={"rope": PartSpec("rope", {"rotary_dim": 16, "theta": 1e4, "pairing": "half"})},
+                     max_position_embeddings=512, embedding_prefix="toy.embed.", final_norm_prefix="toy.norm.",
+                     lm_head_prefix="toy.head.")
+
+
+@pytest.fixture
+def toy_registered():
+    register_part("mixer", "running_sum", RunningSumMixer)
+    register_architecture("ToyRunningSumForCausalLM", ToyConfig, toy_spec)
+    yield
+    unregister_architecture("ToyRunningSumForCausalLM")
+    unregister_part("mixer", "running_sum")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_mixer_with_state_is_registered_built_and_stepped(toy_registered, tmp_path, dtype):
+    cfg = ToyConfig()
+    folder = B.Engine.write_random_folder(str(tmp_path / "toy"), cfg, seed=4, std=0.1)
+    eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=512)      # the registry finds the toy by config.json
+    assert eng.cache.state_bytes_per_slot == 40 * 4 and len(eng.cache.groups) == 1
+    _, w = P.read_folder(folder)
+
+    def plain(toks):
+        x = P.embedding(w["toy.embed.weight"], toks)
+        n = P.rms_norm(x, w["toy.layers.0.input_layernorm.weight"], 1e-5)
+        x = x + np.cumsum(n, axis=0) @ w["toy.layers.0.self_attn.mix.weight"].T
+        sz = dict(nq=2, nkv=1, hd=16, theta=1e4, eps=1e-5, pairing="half")
+        x = P.attention_block(x, np.arange(len(toks)), w, "toy.layers.1.", sz, None)
+        x = P.ffn_block(x, w, "toy.layers.1.", sz)
+        return P.linear(P.rms_norm(x, w["toy.norm.weight"], 1e-5), w["toy.head.weight"])
+
+    rng = np.random.default_rng(0)
+    seqs = [[int(t) for t in rng.integers(0, 90, n)] for n in (30, 9, 17)]
+    refs = [plain(s) for s in seqs]
+    tol = 1e-4 if dtype == "float32" else 4e-2
+    for round_ in range(2):                                   # twice: the state of a reused slot starts at zero
+        slots = [eng.alloc_slot() for _ in seqs]
+        cut = [12, 4, 16]
+        out = eng.step([StepEntry(sl, s[:c], list(range(c))) for sl, s, c in zip(slots, seqs, cut)]).cpu().numpy()
+        got = [[out[sum(cut[:i]):sum(cut[:i + 1])]] for i in range(3)]
+        pos = list(cut)
+        live = [0, 1, 2]
+        while live:
+            out = eng.step([StepEntry(slots[i], [seqs[i][pos[i]]], [0]) for i in live]).cpu().numpy()
+            for r, i in enumerate(live):
+                got[i].append(out[r:r + 1]); pos[i] += 1
+            for i in [i for i in live if pos[i] == len(seqs[i])]:
+                eng.free_slot(slots[i]); live.remove(i)
+        for i in range(3):
+            g = np.concatenate(got[i])
+            assert np.abs(g - refs[i]).max() < tol * np.abs(refs[i]).max(), (round_, i)
+
+
+# ------------------------------------------------------- the run order is data too ----
+@dataclass(frozen=True)
+class LoopConfig:
+    mode: str = "twice"
+    architecture = "ToyLoopForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d["mode"])
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], "mode": self.mode}
+
+
+def loop_spec(cfg):
+    H = 48
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 1, "head_dim": 16,
+                                      "window": None, "position": "rope"})
+    layers = [LayerSpec(f"m.layers.{i}.", attn, None, norm, None) for i in range(2)]
+    if cfg.mode == "twice":       # layer 0, layer 1, layer 0 again with a cache of its own
+        schedule = [ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(0, 2)]
+    else:                         # layer 1 reads the keys and values layer 0 stored, and stores none
+        schedule = [ScheduleEntry(0, 0), ScheduleEntry(1, 0, writes_cache=False)]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=70,
+                     embedding=PartSpec("embedding", {"vocab_size": 70, "hidden_size": H}), layers=layers,
+                     schedule=schedule, final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": 70, "hidden_size": H, "tied_to": "m.embed.weight"}),
+                     positions={"rope": PartSpec("rope", {"rotary_dim": 16, "theta": 1e4, "pairing": "half"})},
+                     max_position_embeddings=512, embedding_prefix="m.embed.", final_norm_prefix="m.norm.",
+                     lm_head_prefix="m.head.")
+
+
+@pytest.mark.parametrize("mode", ["twice", "shared"])
+def test_schedule_names_a_layer_twice_or_shares_a_cache(tmp_path, mode):
+    register_architecture("ToyLoopForCausalLM", LoopConfig, loop_spec)
+    try:
+        folder = B.Engine.write_random_folder(str(tmp_path / mode), LoopConfig(mode), seed=2, std=0.15)
+        eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=256)
+        _, w = P.read_folder(folder)
+        sz = dict(nq=3, nkv=1, hd=16, theta=1e4, eps=1e-5, pairing="half")
+        toks = [int(t) for t in np.random.default_rng(1).integers(0, 70, 40)]
+        T = len(toks)
+        x = P.embedding(w["m.embed.weight"], toks)
+        if mode == "twice":
+            assert sorted(eng.cache.group_of_unit) == [0, 1, 2]
+            for p in ("m.layers.0.", "m.layers.1.", "m.layers.0."):
+                x = P.attention_block(x, np.arange(T), w, p, sz, None)
+        else:
+            assert sorted(eng.cache.group_of_unit) == [0]
+            inv = P.rope_inv_freq(16, 1e4)
+            n0 = P.rms_norm(x, w["m.layers.0.input_layernorm.weight"], 1e-5)
+            k0 = P.rope(P.linear(n0, w["m.layers.0.self_attn.k_proj.weight"]).reshape(T, 1, 16), np.arange(T), inv, "half")
+            v0 = P.linear(n0, w["m.layers.0.self_attn.v_proj.weight"]).reshape(T, 1, 16)
+            x = P.attention_block(x, np.arange(T), w, "m.layers.0.", sz, None)
+            n1 = P.rms_norm(x, w["m.layers.1.input_layernorm.weight"], 1e-5)
+            q1 = P.rope(P.linear(n1, w["m.layers.1.self_attn.q_proj.weight"]).reshape(T, 3, 16), np.arange(T), inv, "half")
+            x = x + P.linear(P.attention(q1, k0, v0, 3, 1).reshape(T, 48), w["m.layers.1.self_attn.o_proj.weight"])
+        ref = P.linear(P.rms_norm(x, w["m.norm.weight"], 1e-5), w["m.embed.weight"])
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, toks[:25], list(range(25)))]).cpu().numpy()]
+        for t in toks[25:]:
+            got.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+        eng.free_slot(s)
+        assert np.abs(np.concatenate(got) - ref).max() < 1e-4 * np.abs(ref).max()
+    finally:
+        unregister_architecture("ToyLoopForCausalLM")
+
+
+def test_a_schedule_that_reads_an_unwritten_cache_is_refused():
+    register_architecture("ToyLoopForCausalLM", LoopConfig, loop_spec)
+    try:
+        spec = loop_spec(LoopConfig("shared"))
+        bad = ModelSpec(**{**spec.__dict__, "schedule": [ScheduleEntry(1, 0, writes_cache=False), ScheduleEntry(0, 0)]})
+        with pytest.raises(B.ConfigError, match="before"):
+            B.DecoderModel(bad)
+    finally:
+        unregister_architecture("ToyLoopForCausalLM")
