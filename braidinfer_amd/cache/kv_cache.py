@@ -6,8 +6,10 @@ reference, whose page holds all layers of 64 tokens as f32,
 crates/braidinfer-runtime/src/paged_kv.rs:17-21): a *group* gathers the cache units
 whose needs are equal (kv heads, head size, full or windowed).  A group owns one page
 pool and one block table `[slot, page index in sequence] -> page`; every unit of the
-group owns storage `[n_pages, 2 (K|V), kv_heads, page_tokens, head_dim]` indexed by the
-same page numbers.  Keys are stored after rotation, values as they are.  A windowed
+group owns storage `[n_pages, 2 (K|V), kv_heads, page_tokens * head_dim]` indexed by the
+same page numbers: keys as `[token, head_dim]` after rotation, values transposed as
+`[head_dim, token]` (the operand layout of the matrix-core attention kernels; the tensor's
+last two dimensions are declared `[page_tokens, head_dim]` for both).  A windowed
 group returns pages that lie wholly before the window to its pool after every step.
 """
 from __future__ import annotations

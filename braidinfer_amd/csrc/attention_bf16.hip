@@ -1,0 +1,405 @@
+// Attention over the paged bf16 cache on the gfx950 matrix cores: a flash kernel for
+// steps with several tokens per sequence (prompts, chunks) and a split-context kernel
+// for single-token steps.  Both compute, per (query row, kv head), the online softmax
+// of the reference (m' = max(m, s), c = exp(m - m'), d = d c + w, acc = acc c + w v;
+// kernels/megakernel_ops.hip:2310-2342) in float, with kv head = q head / (nq / nkv)
+// (:2192), scores scaled by `scale` (:2194), causality as a bound on the key index and a
+// window i - W < j <= i.
+//
+// Operand layout.  A page of one kv head holds keys row-major [token][hd] and values
+// transposed [hd][token].  Scores are computed transposed, S^T = K Q^T, so that the
+// accumulator of the first product (a lane holds one query column and several keys) is,
+// after exp and rounding to bf16, exactly the B operand of the second, O^T = V^T P^T,
+// with V^T rows read as the A operand: no shuffle and no LDS between the two products.
+// The k-slots of the second product are a fixed permutation of the keys (a lane's slots
+// are the keys its accumulator registers hold); V^T is read with the same permutation.
+#include "common.h"
+
+#define PAGE 64
+
+__device__ __forceinline__ bf16x8 zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+    return z;
+}
+__device__ __forceinline__ bf16x8 join4(bf16x4 a, bf16x4 b) {
+    bf16x8 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+    return v;
+}
+__device__ __forceinline__ bf16x4 zero4() {
+    bf16x4 z;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) z[i] = (bf16)0.f;
+    return z;
+}
+// 4 values V^T[dim][k .. k+3] of a page; keys at or beyond `limit` read as zero
+__device__ __forceinline__ bf16x4 load_vt4(const bf16* __restrict__ vrow, int k, int limit_local) {
+    bf16x4 v = *(const bf16x4*)(vrow + k);
+    if (k + 4 > limit_local) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) if (k + i >= limit_local) v[i] = (bf16)0.f;
+    }
+    return v;
+}
+
+// --------------------------------------------------------------------- prefill ------
+// grid = (row tiles of 128, nkv, sequences), block = 256.  A row is a (token, q head of
+// the group) pair: row = token * G + head.  Each wave owns 32 rows and walks the key
+// blocks of 32 its rows can see; NB = ceil(hd / 32).
+template <int NB>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
+    int table_stride, const bf16* __restrict__ cache, int nq, int nkv, int hd, int window, float scale) {
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int slot = slots[b];
+    const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
+    const int G = nq / nkv;
+    const int rows_total = n_new * G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row0 = blockIdx.x * 128 + wave * 32;
+    if (row0 >= rows_total) return;
+    const int c = lane & 31, g = lane >> 5;
+    const int row = row0 + c;
+    const bool row_ok = row < rows_total;
+    const int rr = row_ok ? row : rows_total - 1;
+    const int tok = rr / G, head = kvh * G + rr % G;
+    bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * hd;
+    if (slot < 0) {       // padding: no cache behind it
+        if (row_ok && g == 0) for (int d = 0; d < hd; ++d) orow[d] = (bf16)0.f;
+        return;
+    }
+    const int ctx = ctx_lens[b], start = ctx - n_new;
+    const int pq = start + tok;
+    const int pq_min = start + row0 / G;
+    const int last_row = (row0 + 31 < rows_total ? row0 + 31 : rows_total - 1);
+    const int pq_max = start + last_row / G;
+
+    const bf16* qrow = q + (size_t)(t0 + tok) * q_stride + (size_t)head * hd;
+    bf16x8 qf[2 * NB];
+#pragma unroll
+    for (int s = 0; s < 2 * NB; ++s) {
+        const int d = s * 16 + 8 * g;
+        qf[s] = (d < hd) ? *(const bf16x8*)(qrow + d) : zero8();
+    }
+    f32x16 acc_o[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+
+    const int* bt = block_table + (size_t)slot * table_stride;
+    const size_t page_elems = (size_t)2 * nkv * PAGE * hd;
+    const size_t k_off = (size_t)kvh * PAGE * hd, v_off = ((size_t)nkv + kvh) * PAGE * hd;
+    int lo = 0;
+    if (window > 0 && pq_min - window + 1 > 0) lo = pq_min - window + 1;
+    for (int kb = (lo / 32) * 32; kb <= pq_max; kb += 32) {
+        const bf16* pg = cache + (size_t)bt[kb / PAGE] * page_elems;
+        const int kl = kb % PAGE;                       // 0 or 32: the block's place in its page
+        const bf16* krow = pg + k_off + (size_t)(kl + c) * hd;
+        f32x16 s_acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 2 * NB; ++s) {
+            const int d = s * 16 + 8 * g;
+            const bf16x8 kf = (d < hd) ? *(const bf16x8*)(krow + d) : zero8();
+            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+        }
+        // s_acc[r]: key kb + 8 (r / 4) + 4 g + r % 4, query row = this lane's column
+        float sv[16];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
+            const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
+            sv[r] = ok ? s_acc[r] * scale : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = expf(m - m_use);
+        float psum = 0.f;
+        bf16x8 p1, p2;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float p = expf(sv[r] - m_use);
+            psum += p;
+            if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
+        }
+        lsum = lsum * corr + psum;
+        m = m_new;
+        const int limit_local = ctx - (kb - kl);        // keys of this page at or beyond it are not written yet
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
+            const int dim = i * 32 + c;
+            bf16x8 v1 = zero8(), v2 = zero8();
+            if (dim < hd) {
+                const bf16* vrow = pg + v_off + (size_t)dim * PAGE;
+                v1 = join4(load_vt4(vrow, kl + 4 * g, limit_local), load_vt4(vrow, kl + 8 + 4 * g, limit_local));
+                v2 = join4(load_vt4(vrow, kl + 16 + 4 * g, limit_local), load_vt4(vrow, kl + 24 + 4 * g, limit_local));
+            }
+            acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i], 0, 0, 0);
+            acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i], 0, 0, 0);
+        }
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (!row_ok) return;
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int d = i * 32 + 8 * r4 + 4 * g;      // acc_o[i][4 r4 + e]: dim d + e
+            if (d < hd) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16)(acc_o[i][4 * r4 + e] * inv);
+                *(bf16x4*)(orow + d) = o;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------- decode ------
+// One token per sequence.  grid = (splits, nkv * head blocks, sequences), block = 256.
+// The pages a query sees are cut into `nsplit` runs; the 4 waves of a workgroup take a
+// run's pages in turn and are combined in LDS in wave order.  With one split the
+// workgroup writes the output; otherwise it writes (m, l, unnormalised O) for its split
+// and attn_decode_combine_kernel adds the splits in split order.  NB = ceil(hd / 32).
+template <int NB>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ slots,
+    const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
+    const bf16* __restrict__ cache, int nq, int nkv, int hd, int window, float scale, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    extern __shared__ float lds[];
+    const int G = nq / nkv, nhb = (G + 15) / 16;
+    const int split = blockIdx.x, kvh = blockIdx.y / nhb, hb = blockIdx.y % nhb, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int nheads = (G - hb * 16 < 16) ? G - hb * 16 : 16;     // heads of this block
+    const int head0 = kvh * G + hb * 16;
+    const int slot = slots[b];
+    const int ctx = slot < 0 ? 0 : ctx_lens[b];
+    int lo = 0;
+    if (window > 0 && ctx - window > 0) lo = ctx - window;         // the query sits at ctx - 1
+    const int pg_lo = lo / PAGE, npg = ctx > 0 ? (ctx - 1) / PAGE - pg_lo + 1 : 0;
+    const int pps = (npg + nsplit - 1) / nsplit;
+    const int pg_begin = pg_lo + split * pps;
+    int pg_end = pg_begin + pps;
+    if (pg_end > pg_lo + npg) pg_end = pg_lo + npg;
+
+    const bool head_ok = c < nheads;
+    const bf16* qrow = q + (size_t)b * q_stride + (size_t)(head0 + (head_ok ? c : 0)) * hd;
+    bf16x8 qf[NB];
+#pragma unroll
+    for (int s = 0; s < NB; ++s) {
+        const int d = s * 32 + 8 * g;
+        qf[s] = (head_ok && d < hd) ? *(const bf16x8*)(qrow + d) : zero8();
+    }
+    f32x4 acc_o[2 * NB];
+#pragma unroll
+    for (int i = 0; i < 2 * NB; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc_o[i][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+    const int* bt = block_table + (size_t)(slot < 0 ? 0 : slot) * table_stride;
+    const size_t page_elems = (size_t)2 * nkv * PAGE * hd;
+    const size_t k_off = (size_t)kvh * PAGE * hd, v_off = ((size_t)nkv + kvh) * PAGE * hd;
+
+    for (int pi = pg_begin + wave; pi < pg_end; pi += 4) {
+        const bf16* pg = cache + (size_t)bt[pi] * page_elems;
+        const int pos0 = pi * PAGE;
+        const int limit_local = ctx - pos0;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int kl = half * 32, kb = pos0 + kl;
+            if (kb >= ctx || kb + 32 <= lo) continue;
+            f32x4 s_acc[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s_acc[j][r] = 0.f;
+                const bf16* krow = pg + k_off + (size_t)(kl + 16 * j + c) * hd;
+#pragma unroll
+                for (int s = 0; s < NB; ++s) {
+                    const int d = s * 32 + 8 * g;
+                    const bf16x8 kf = (d < hd) ? *(const bf16x8*)(krow + d) : zero8();
+                    s_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s_acc[j], 0, 0, 0);
+                }
+            }
+            // s_acc[j][r]: key kb + 16 j + 4 g + r, head = this lane's column
+            float sv[8];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int key = kb + 16 * (e >> 2) + 4 * g + (e & 3);
+                const bool ok = key >= lo && key < ctx;
+                sv[e] = ok ? s_acc[e >> 2][e & 3] * scale : -INFINITY;
+                mx = fmaxf(mx, sv[e]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);           // finite: the block holds at least one visible key
+            const float corr = expf(m - m_new);
+            float psum = 0.f;
+            bf16x8 pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = expf(sv[e] - m_new);
+                psum += p;
+                pf[e] = (bf16)p;
+            }
+            lsum = lsum * corr + psum;
+            m = m_new;
+#pragma unroll
+            for (int i = 0; i < 2 * NB; ++i) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc_o[i][r] *= corr;
+                const int dim = i * 16 + c;
+                bf16x8 vf = zero8();
+                if (dim < hd) {
+                    const bf16* vrow = pg + v_off + (size_t)dim * PAGE;
+                    vf = join4(load_vt4(vrow, kl + 4 * g, limit_local), load_vt4(vrow, kl + 16 + 4 * g, limit_local));
+                }
+                acc_o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc_o[i], 0, 0, 0);
+            }
+        }
+    }
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
+    // LDS: per wave [16 heads][hd] O, then [16] m, [16] l
+    const int wstride = 16 * hd + 32;
+    float* my = lds + wave * wstride;
+#pragma unroll
+    for (int i = 0; i < 2 * NB; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int d = i * 16 + 4 * g + r;           // acc_o[i][r]: dim d, head c
+            if (d < hd) my[c * hd + d] = acc_o[i][r];
+        }
+    if (g == 0) { my[16 * hd + c] = m; my[16 * hd + 16 + c] = lsum; }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nheads * hd; e += 256) {
+        const int h = e / hd, d = e - h * hd;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, lds[w * wstride + 16 * hd + h]);
+        float L = 0.f, O = 0.f;
+        if (M > -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float f = expf(lds[w * wstride + 16 * hd + h] - M);
+                L += lds[w * wstride + 16 * hd + 16 + h] * f;
+                O += lds[w * wstride + h * hd + d] * f;
+            }
+        }
+        const int head = head0 + h;
+        if (nsplit == 1) {
+            out[((size_t)b * nq + head) * hd + d] = (bf16)(L > 0.f ? O / L : 0.f);
+        } else {
+            const size_t pidx = ((size_t)b * nq + head) * nsplit + split;
+            part_o[pidx * hd + d] = O;
+            if (d == 0) { part_ml[pidx * 2] = M; part_ml[pidx * 2 + 1] = L; }
+        }
+    }
+}
+
+// grid = (nq, sequences), block = 64: add the splits in split order
+__global__ __launch_bounds__(64) void attn_decode_combine_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16* __restrict__ out, int nq, int hd, int nsplit) {
+    const int head = blockIdx.x, b = blockIdx.y;
+    const size_t base = ((size_t)b * nq + head) * nsplit;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+    float L = 0.f;
+    if (M > -INFINITY)
+        for (int s = 0; s < nsplit; ++s) L += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - M);
+    for (int d = threadIdx.x; d < hd; d += 64) {
+        float O = 0.f;
+        if (M > -INFINITY)
+            for (int s = 0; s < nsplit; ++s) O += part_o[(base + s) * hd + d] * expf(part_ml[(base + s) * 2] - M);
+        out[((size_t)b * nq + head) * hd + d] = (bf16)(L > 0.f ? O / L : 0.f);
+    }
+}
+
+static int nb_of(int hd) { return (hd + 31) / 32; }
+
+extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, const int* cu_seqlens,
+                                    const int* slots, const int* ctx_lens, const int* block_table,
+                                    int table_stride, const void* cache, int B, int max_new, int nq, int nkv,
+                                    int hd, int page, int window, float scale, hipStream_t s) {
+    if (B <= 0 || max_new <= 0) return BR_OK;
+    if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
+        q_stride % 8 || ((uintptr_t)q % 16) || nkv > 65535 || B > 65535)
+        return BR_BAD_ARG;
+    const int G = nq / nkv;
+    dim3 grid(((size_t)max_new * G + 127) / 128, nkv, B);
+#define BR_PREFILL(N)                                                                                      \
+    attn_prefill_kernel<N><<<grid, 256, 0, s>>>((const bf16*)q, q_stride, (bf16*)out, cu_seqlens, slots,  \
+                                                 ctx_lens, block_table, table_stride, (const bf16*)cache,  \
+                                                 nq, nkv, hd, window, scale)
+    switch (nb_of(hd)) {
+        case 1: BR_PREFILL(1); break;
+        case 2: BR_PREFILL(2); break;
+        case 3: BR_PREFILL(3); break;
+        case 4: BR_PREFILL(4); break;
+        case 5: case 6: BR_PREFILL(6); break;
+        default: BR_PREFILL(8); break;
+    }
+#undef BR_PREFILL
+    return br_check_launch();
+}
+
+// part_o: float [B, nq, nsplit, hd]; part_ml: float [B, nq, nsplit, 2] (unused when nsplit == 1)
+extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, const int* slots,
+                                   const int* ctx_lens, const int* block_table, int table_stride,
+                                   const void* cache, int B, int nq, int nkv, int hd, int page, int window,
+                                   float scale, int nsplit, float* part_o, float* part_ml, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
+        q_stride % 8 || ((uintptr_t)q % 16) || nsplit < 1 || nsplit > 1024 || B > 65535 ||
+        (nsplit > 1 && (!part_o || !part_ml)))
+        return BR_BAD_ARG;
+    const int G = nq / nkv, nhb = (G + 15) / 16;
+    if ((long long)nkv * nhb > 65535) return BR_BAD_ARG;
+    dim3 grid(nsplit, nkv * nhb, B);
+    const size_t lds = (size_t)4 * (16 * hd + 32) * sizeof(float);
+#define BR_DECODE(N)                                                                                        \
+    do {                                                                                                    \
+        auto kern = attn_decode_kernel<N>;                                                                  \
+        if (lds > 48 * 1024) {                                                                              \
+            static bool set = false;                                                                        \
+            if (!set) {                                                                                     \
+                if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,      \
+                                        (int)(4 * (16 * 256 + 32) * sizeof(float))) != hipSuccess)          \
+                    return BR_LAUNCH_FAILED;                                                                \
+                set = true;                                                                                 \
+            }                                                                                               \
+        }                                                                                                   \
+        kern<<<grid, 256, lds, s>>>((const bf16*)q, q_stride, (bf16*)out, slots, ctx_lens, block_table,     \
+                                    table_stride, (const bf16*)cache, nq, nkv, hd, window, scale, nsplit,   \
+                                    part_o, part_ml);                                                       \
+    } while (0)
+    switch (nb_of(hd)) {
+        case 1: BR_DECODE(1); break;
+        case 2: BR_DECODE(2); break;
+        case 3: BR_DECODE(3); break;
+        case 4: BR_DECODE(4); break;
+        case 5: case 6: BR_DECODE(6); break;
+        default: BR_DECODE(8); break;
+    }
+#undef BR_DECODE
+    int rc = br_check_launch();
+    if (rc != BR_OK || nsplit == 1) return rc;
+    attn_decode_combine_kernel<<<dim3(nq, B), 64, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
+    return br_check_launch();
+}

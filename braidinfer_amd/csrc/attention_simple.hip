@@ -39,7 +39,8 @@ __global__ __launch_bounds__(64) void attn_simple_kernel(
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int* bt = block_table + (size_t)slot * table_stride;
-    const size_t page_elems = (size_t)2 * nkv * page * hd;  // one page: [K|V][kvh][tok][hd]
+    // one page: [K|V][kvh], keys [tok][hd], values transposed [hd][tok]
+    const size_t page_elems = (size_t)2 * nkv * page * hd;
     const size_t k_off = (size_t)kvh * page * hd, v_off = ((size_t)nkv + kvh) * page * hd;
 
     float m = -INFINITY, l = 0.f;
@@ -68,12 +69,12 @@ __global__ __launch_bounds__(64) void attn_simple_kernel(
         for (int i = 0; i < MAX_DPL; ++i) acc[i] *= corr;
         for (int jj = 0; jj < nk; ++jj) {
             const int jk = j0 + jj;
-            const T* vr = cache + (size_t)bt[jk / page] * page_elems + v_off + (size_t)(jk % page) * hd;
+            const T* vc = cache + (size_t)bt[jk / page] * page_elems + v_off + (jk % page);
             const float pw = ps[jj];
 #pragma unroll
             for (int i = 0; i < MAX_DPL; ++i) {
                 const int d = lane + 64 * i;
-                if (d < hd) acc[i] = fmaf(pw, to_f32<T>(vr[d]), acc[i]);
+                if (d < hd) acc[i] = fmaf(pw, to_f32<T>(vc[(size_t)d * page]), acc[i]);
             }
         }
         m = m_new;

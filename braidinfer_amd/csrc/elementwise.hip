@@ -95,7 +95,9 @@ extern "C" int br_rope_table(const int* pos, const float* inv_freq, float* cs, f
 // (2p, 2p+1) when adjacent, (p, p + rd/2) when half), write q back in place, and store
 // the rotated k and the untouched v in the token's cache page (reference:
 // op_kv_write_paged_batch.hip:58-73 for the page/offset arithmetic; keys are stored
-// after rotation, once).  Cache layout per unit: [page][K|V][kv_head][token_in_page][hd].
+// after rotation, once).  Cache layout per unit: [page][K|V][kv_head], then keys as
+// [token_in_page][hd] and values transposed, [hd][token_in_page], which is the operand
+// layout of the matrix-core attention kernels.
 // A token whose sequence has slot < 0 is padding: q is still rotated, nothing is stored.
 // grid = (T, nq + 2 nkv), block = 64.
 template <typename T>
@@ -117,7 +119,13 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
         const int p = pos[t];
         const int pg = block_table[(size_t)slot * table_stride + p / page];
         const int kvh = is_k ? h - nq : h - nq - nkv;
-        dst = cache + ((((size_t)pg * 2 + (is_k ? 0 : 1)) * nkv + kvh) * page + (p % page)) * hd;
+        T* unit = cache + (((size_t)pg * 2 + (is_k ? 0 : 1)) * nkv + kvh) * page * hd;
+        if (is_k) dst = unit + (size_t)(p % page) * hd;
+        else {
+            T* col = unit + (p % page);                  // values: element i of the head at [i][token]
+            for (int i = threadIdx.x; i < hd; i += blockDim.x) col[(size_t)i * page] = src[i];
+            return;
+        }
     }
     if (is_q || is_k) {
         const int P = rd / 2;
@@ -132,8 +140,6 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
             o[i1] = from_f32<T>(a * si + b * co);
         }
         if (is_k) for (int i = rd + threadIdx.x; i < hd; i += blockDim.x) o[i] = src[i];
-    } else {
-        for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
     }
 }
 

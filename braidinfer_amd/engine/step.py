@@ -51,6 +51,7 @@ class StepBatch:
     is_decode: bool = False          # every sequence brings exactly one token
     max_new: int = 0
     max_ctx: int = 0
+    max_ctx_bound: int = 0           # an upper bound of max_ctx that kernels may size their grids by
     ws: Optional[Workspace] = None
     position_data: Dict[str, Any] = field(default_factory=dict)
     extras: Dict[str, Any] = field(default_factory=dict)     # per-step scratch of parts (keyed by them)
@@ -95,4 +96,4 @@ def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts
         n_tokens=T, n_seqs=B, tokens=tokens, positions=positions, seq_of_token=seq_of_token,
         cu_seqlens=cu_seqlens, slots=slots_d, ctx_lens=ctx_d, host_slots=all_slots, host_new=new,
         host_start=all_starts, is_decode=all(n == 1 for n in new), max_new=max(new) if new else 0,
-        max_ctx=max(ctx) if ctx else 0, ws=ws)
+        max_ctx=max(ctx) if ctx else 0, max_ctx_bound=max(ctx) if ctx else 0, ws=ws)

@@ -221,6 +221,48 @@ def attention_simple(q: torch.Tensor, q_stride: int, out: torch.Tensor, position
              int(window or 0), float(scale), _stream()), "attention_simple")
 
 
+def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu_seqlens: torch.Tensor,
+                           slots: torch.Tensor, ctx_lens: torch.Tensor, block_table: torch.Tensor,
+                           cache: torch.Tensor, B: int, max_new: int, nq: int, nkv: int, hd: int, page: int,
+                           window: Optional[int], scale: float) -> None:
+    """Flash attention on the matrix cores for steps with several tokens per sequence."""
+    _dev("attention_prefill_bf16", out, cu_seqlens, slots, ctx_lens, block_table, cache)
+    _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+         "attention_prefill_bf16: bfloat16 only")
+    _req(hd % 16 == 0 and hd <= 256, f"attention_prefill_bf16: head_dim {hd} must be a multiple of 16, at most 256")
+    _req(page == 64, "attention_prefill_bf16: pages of 64 tokens")
+    _req(cache.shape[1:] == (2, nkv, page, hd), "attention_prefill_bf16: cache unit must be [pages, 2, nkv, page, hd]")
+    _req(out.shape[1] == nq * hd and nq % nkv == 0, "attention_prefill_bf16: out must be [T, nq * hd]")
+    f = _fn("attention_bf16", "br_attn_prefill_bf16",
+            [_P, c_size_t, _P, _P, _P, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, _P])
+    _check(f(_ptr(q), q_stride, _ptr(out), _ptr(cu_seqlens), _ptr(slots), _ptr(ctx_lens), _ptr(block_table),
+             block_table.shape[1], _ptr(cache), B, max_new, nq, nkv, hd, page, int(window or 0), float(scale),
+             _stream()), "attention_prefill_bf16")
+
+
+def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slots: torch.Tensor,
+                          ctx_lens: torch.Tensor, block_table: torch.Tensor, cache: torch.Tensor, B: int,
+                          nq: int, nkv: int, hd: int, page: int, window: Optional[int], scale: float,
+                          nsplit: int, part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor]) -> None:
+    """Attention of one new token per sequence over its pages, cut into `nsplit` runs."""
+    _dev("attention_decode_bf16", out, slots, ctx_lens, block_table, cache, part_o, part_ml)
+    _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+         "attention_decode_bf16: bfloat16 only")
+    _req(hd % 16 == 0 and hd <= 256, f"attention_decode_bf16: head_dim {hd} must be a multiple of 16, at most 256")
+    _req(page == 64, "attention_decode_bf16: pages of 64 tokens")
+    _req(cache.shape[1:] == (2, nkv, page, hd), "attention_decode_bf16: cache unit must be [pages, 2, nkv, page, hd]")
+    _req(out.shape == (B, nq * hd) and nq % nkv == 0, "attention_decode_bf16: out must be [B, nq * hd]")
+    if nsplit > 1:
+        _req(part_o is not None and part_o.dtype == torch.float32 and part_o.numel() >= B * nq * nsplit * hd
+             and part_ml is not None and part_ml.numel() >= B * nq * nsplit * 2,
+             "attention_decode_bf16: scratch for the splits is too small")
+    f = _fn("attention_bf16", "br_attn_decode_bf16",
+            [_P, c_size_t, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, c_int, _P, _P, _P])
+    _check(f(_ptr(q), q_stride, _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1],
+             _ptr(cache), B, nq, nkv, hd, page, int(window or 0), float(scale), nsplit, _ptr(part_o),
+             _ptr(part_ml), _stream()), "attention_decode_bf16")
+
+
 # -------------------------------------------------------------------- sampling -----
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _dev("argmax", logits, out)

@@ -24,6 +24,16 @@ from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
 from .linear import fuse_rows, linear
 
 
+def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
+    """Into how many runs a sequence's pages are cut for single-token steps: enough
+    workgroups to fill the 256 CUs about twice, at least two pages per run.  It depends
+    on the step's shape only (batch and an upper bound of the context), never on the
+    tokens."""
+    pages = max(1, -(-max_ctx // page))
+    want = -(-512 // max(1, batch * nkv))
+    return max(1, min(want, pages // 2 if pages >= 2 else 1, 64))
+
+
 class GQAAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: Optional[int] = None, position: Optional[str] = "rope", scale: Optional[float] = None):
@@ -36,6 +46,7 @@ class GQAAttention(Mixer):
         self.position = position
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
         self.w_qkv = self.w_o = None
+        self.force_simple = False          # tests set it to run the one-wave-per-query kernel in bf16
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         return [
@@ -71,7 +82,27 @@ class GQAAttention(Mixer):
         linear(o, self.w_o, x, step.ws, accumulate=True)
 
     def attend(self, qkv, o, step, ctx: MixerContext) -> None:
+        """bf16 with a head size the matrix-core kernels take: split-context kernel when
+        every sequence brings one token, flash kernel otherwise.  Else (32-bit path, head
+        sizes beyond 256 or not in steps of 16) the one-wave-per-query kernel."""
         T = step.n_tokens
+        nq, nkv, hd = self.nq, self.nkv, self.hd
+        if qkv.dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and ctx.page_tokens == 64 and not self.force_simple:
+            B = step.n_seqs
+            if step.is_decode:
+                nsplit = decode_splits(B, nkv, step.max_ctx_bound, ctx.page_tokens)
+                part_o = part_ml = None
+                if nsplit > 1:
+                    part_o = step.ws.get("attn_part_o", (B * nq * nsplit * hd,), torch.float32)
+                    part_ml = step.ws.get("attn_part_ml", (B * nq * nsplit * 2,), torch.float32)
+                K.attention_decode_bf16(qkv, qkv.stride(0), o, step.slots, step.ctx_lens, ctx.block_table,
+                                        ctx.storage, B, nq, nkv, hd, ctx.page_tokens, self.window, self.scale,
+                                        nsplit, part_o, part_ml)
+            else:
+                K.attention_prefill_bf16(qkv, qkv.stride(0), o, step.cu_seqlens, step.slots, step.ctx_lens,
+                                         ctx.block_table, ctx.storage, B, step.max_new, nq, nkv, hd,
+                                         ctx.page_tokens, self.window, self.scale)
+            return
         K.attention_simple(qkv, qkv.stride(0), o, step.positions, step.seq_of_token, step.slots,
                            ctx.block_table, ctx.storage, T, self.nq, self.nkv, self.hd, ctx.page_tokens,
                            self.window, self.scale)

@@ -179,14 +179,18 @@ def test_rope_and_paged_write(dtype, adjacent, nq, nkv, hd, rd):
     assert (qkv[:, :nq * hd].reshape(T, nq, hd).double() - q_want).abs().max() < tol * q_want.abs().max()
     assert torch.equal(qkv[:, nq * hd:], src[:, nq * hd:])            # k and v rows of the step buffer are untouched
     written = torch.zeros(8, page, dtype=torch.bool)
+    written_v = torch.zeros(8, page, dtype=torch.bool)
     for t in range(T):
         p, slot = int(pos[t]), int(slots[int(sot[t])])
         pg = int(table[slot, p // page])
         written[pg, p % page] = True
         assert (cache[pg, 0, :, p % page].double() - k_want[t]).abs().max() < tol * k_want.abs().max()
-        assert torch.equal(cache[pg, 1, :, p % page], v_in[t])         # values byte-equal
-    untouched = cache[:, :, :, :, :][~written[:, None, None, :].expand(8, 2, nkv, page)]
-    assert torch.all(untouched == 99.0)
+        vt = cache[pg, 1].reshape(nkv, hd, page)                      # values are stored transposed
+        assert torch.equal(vt[:, :, p % page], v_in[t])                # and byte-equal
+        written_v[pg, p % page] = True
+    assert torch.all(cache[:, 0][~written[:, None, :].expand(8, nkv, page)] == 99.0)
+    vt_all = cache[:, 1].reshape(8, nkv, hd, page).permute(0, 1, 3, 2)
+    assert torch.all(vt_all[~written_v[:, None, :].expand(8, nkv, page)] == 99.0)
     # a padded sequence (slot -1) stores nothing; write_cache=False stores nothing
     cache2 = torch.full_like(cache, 99.0)
     K.rope_kv_write(src.clone(), cs, sn, pos, sot, i32([-1, -1, -1]), table, cache2, nq, nkv, hd, rd, adjacent, page, True)
@@ -215,7 +219,7 @@ def _paged(k, v, pages, page, n_pages, dtype):
     cache = torch.zeros(n_pages, 2, nkv, page, hd, dtype=dtype, device=DEV)
     for t in range(T):
         cache[pages[t // page], 0, :, t % page] = k[t]
-        cache[pages[t // page], 1, :, t % page] = v[t]
+        cache[pages[t // page], 1].view(nkv, hd, page)[:, :, t % page] = v[t]      # values transposed
     return cache
 
 
@@ -300,3 +304,88 @@ def test_argmax_lowest_index_wins():
     # reference vector: greedy on [0.1, 0.5, 0.2, 0.8, 0.3] -> 3 (sampling.rs:232-241)
     K.argmax(torch.tensor([[0.1, 0.5, 0.2, 0.8, 0.3]], device=DEV), out)
     assert out[0].item() == 3
+
+
+# ------------------------------------------- matrix-core attention kernels (bf16) ----
+def _multi_seq_cache(lens, nkv, hd, seed):
+    """Keys/values of several sequences scattered over shuffled pages: (k, v lists, cache, table)."""
+    page = 64
+    n_pages = sum(-(-n // page) for n in lens) + 3
+    order = torch.randperm(n_pages, generator=torch.Generator().manual_seed(seed)).tolist()
+    # stale, non-zero contents in every page: a kernel that reads beyond a sequence's end shows
+    cache = torch.full((n_pages, 2, nkv, page, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    table = torch.full((len(lens) + 2, max(-(-n // page) for n in lens) + 1), -1, dtype=torch.int32)
+    ks, vs = [], []
+    for b, n in enumerate(lens):
+        k, v = rnd(n, nkv, hd, seed=seed + 10 * b + 1, dtype=torch.bfloat16), rnd(n, nkv, hd, seed=seed + 10 * b + 2, dtype=torch.bfloat16)
+        ks.append(k); vs.append(v)
+        for i in range(-(-n // page)):
+            pg = order.pop()
+            table[b + 1, i] = pg                       # sequence b lives in slot b + 1
+            m = min(page, n - i * page)
+            cache[pg, 0, :, :m] = k[i * page:i * page + m].permute(1, 0, 2)
+            cache[pg, 1].view(nkv, hd, page)[:, :, :m] = v[i * page:i * page + m].permute(1, 2, 0)
+    return ks, vs, cache, table.to(DEV)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,window", [(4, 2, 16, None), (6, 3, 32, 8), (5, 1, 48, 70), (32, 8, 128, None),
+                                              (8, 2, 128, 100), (3, 3, 80, None), (2, 1, 256, 33), (20, 1, 64, None)])
+def test_attention_prefill_matrix_cores(nq, nkv, hd, window):
+    lens = [200, 37, 64, 1, 130]             # lengths after the step
+    new = [200, 30, 3, 1, 65]                # tokens of this step (the rest is earlier context)
+    ks, vs, cache, table = _multi_seq_cache(lens, nkv, hd, seed=nq + hd)
+    T = sum(new)
+    q = rnd(T, nq, hd, seed=99, dtype=torch.bfloat16)
+    cu = [0]
+    for n in new:
+        cu.append(cu[-1] + n)
+    out = torch.full((T, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
+    K.attention_prefill_bf16(q.reshape(T, nq * hd), nq * hd, out, i32(cu), i32([1, 2, 3, 4, 5]), i32(lens), table, cache,
+                             len(lens), max(new), nq, nkv, hd, 64, window, 1 / math.sqrt(hd))
+    pos = torch.cat([torch.arange(l - n, l) for l, n in zip(lens, new)]).int().to(DEV)
+    sot = torch.cat([torch.full((n,), b) for b, n in enumerate(new)]).int().to(DEV)
+    simple = torch.empty_like(out)
+    K.attention_simple(q.reshape(T, nq * hd), nq * hd, simple, pos, sot, i32([1, 2, 3, 4, 5]), table, cache, T, nq, nkv, hd,
+                       64, window, 1 / math.sqrt(hd))
+    for b, (l, n) in enumerate(zip(lens, new)):
+        qq = torch.zeros(l, nq, hd); qq[l - n:] = q[cu[b]:cu[b + 1]].float().cpu()
+        want = _attn_ref(qq, ks[b].float().cpu(), vs[b].float().cpu(), nq, nkv, window)[l - n:]
+        got = out[cu[b]:cu[b + 1]].reshape(n, nq, hd).cpu().double()
+        assert torch.isfinite(got).all()
+        assert (got - want).abs().max() < 2e-2 * want.abs().max(), f"sequence {b}"
+        assert (got - simple[cu[b]:cu[b + 1]].reshape(n, nq, hd).cpu().double()).abs().max() < 2e-2 * want.abs().max()
+
+
+@pytest.mark.parametrize("nsplit", [1, 2, 5, 16])
+@pytest.mark.parametrize("nq,nkv,hd,window", [(4, 2, 16, None), (6, 3, 32, 8), (5, 1, 48, 70), (32, 8, 128, None),
+                                              (8, 2, 128, 100), (2, 1, 256, 33), (20, 1, 64, None)])
+def test_attention_decode_matrix_cores(nq, nkv, hd, window, nsplit):
+    lens = [200, 37, 64, 1, 130, 65, 513]
+    ks, vs, cache, table = _multi_seq_cache(lens, nkv, hd, seed=nq + hd + 1)
+    B = len(lens)
+    q = rnd(B + 1, nq, hd, seed=98, dtype=torch.bfloat16)        # the last row is padding (slot -1)
+    slots = i32(list(range(1, B + 1)) + [-1])
+    ctx = i32(lens + [0])
+    out = torch.full((B + 1, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
+    part_o = torch.empty((B + 1) * nq * nsplit * hd, device=DEV)
+    part_ml = torch.empty((B + 1) * nq * nsplit * 2, device=DEV)
+    K.attention_decode_bf16(q.reshape(B + 1, nq * hd), nq * hd, out, slots, ctx, table, cache, B + 1, nq, nkv, hd, 64,
+                            window, 1 / math.sqrt(hd), nsplit, part_o, part_ml)
+    assert torch.all(out[B] == 0)                                  # padding gives zeros, not garbage
+    for b, l in enumerate(lens):
+        qq = torch.zeros(l, nq, hd); qq[-1] = q[b].float().cpu()
+        want = _attn_ref(qq, ks[b].float().cpu(), vs[b].float().cpu(), nq, nkv, window)[-1]
+        got = out[b].reshape(nq, hd).cpu().double()
+        assert torch.isfinite(got).all()
+        assert (got - want).abs().max() < 2e-2 * want.abs().max(), f"sequence {b} of length {l}"
+
+
+def test_attention_kernels_refuse_what_they_do_not_take():
+    q = rnd(4, 2 * 24, dtype=torch.bfloat16)
+    cache = torch.zeros(2, 2, 1, 64, 24, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(4, 48, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="multiple of 16"):
+        K.attention_decode_bf16(q, 48, out, i32([0, 0, 0, 0]), i32([1, 1, 1, 1]), i32([[0]]), cache, 4, 2, 1, 24, 64, None,
+                                1.0, 1, None, None)
+    with pytest.raises(KernelError, match="multiple of 16"):
+        K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
