@@ -50,7 +50,7 @@ def _require_gpu(device: torch.device) -> None:
 
 class Engine:
     def __init__(self, config, model: DecoderModel, rt: Runtime, max_tokens: int,
-                 max_seq_len: Optional[int] = None, n_slots: Optional[int] = None):
+                 max_seq_len: Optional[int] = None, n_slots: Optional[int] = None, use_graphs: bool = True):
         self.config = config
         self.model = model
         self.spec = model.spec
@@ -60,11 +60,15 @@ class Engine:
         self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens=max_tokens,
                                    max_seq_len=max_seq_len, n_slots=n_slots, dtype=rt.dtype, device=rt.device)
         self.vocab_size = self.spec.vocab_size
+        # single-token steps are replayed from HIP graphs when every part allows it
+        self.use_graphs = bool(use_graphs) and model.graph_safe()
+        self._graphs = None
 
     # ---- construction ------------------------------------------------------------------
     @classmethod
     def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
-                    max_seq_len: Optional[int] = None, n_slots: Optional[int] = None) -> "Engine":
+                    max_seq_len: Optional[int] = None, n_slots: Optional[int] = None,
+                    use_graphs: bool = True) -> "Engine":
         device = torch.device(device)
         _require_gpu(device)
         config = config_from_folder(folder)
@@ -73,12 +77,12 @@ class Engine:
         tensors = load_tensors(folder, model.weight_specs(), device, rt.dtype,
                                allow_unexpected=model.optional_names())
         model.load(tensors, rt)
-        return cls(config, model, rt, max_tokens, max_seq_len, n_slots)
+        return cls(config, model, rt, max_tokens, max_seq_len, n_slots, use_graphs)
 
     @classmethod
     def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
                max_seq_len: Optional[int] = None, n_slots: Optional[int] = None, std: float = 0.02,
-               num_layers: Optional[int] = None) -> "Engine":
+               use_graphs: bool = True) -> "Engine":
         """Seeded random weights made on the device (no folder): bf16 N(0, std) matrices,
         norm weights 1, as the random-weights folder mode makes them."""
         device = torch.device(device)
@@ -92,7 +96,7 @@ class Engine:
             widen = kinds[name] == "vector" or rt.dtype == torch.float32
             tensors[name] = t.to(torch.float32) if (widen and kinds[name] != "int") else t
         model.load(tensors, rt)
-        return cls(config, model, rt, max_tokens, max_seq_len, n_slots)
+        return cls(config, model, rt, max_tokens, max_seq_len, n_slots, use_graphs)
 
     @staticmethod
     def write_random_folder(folder: str, config, seed: int = 0, std: float = 0.02,
@@ -139,8 +143,17 @@ class Engine:
         new = [len(tl) for tl in token_lists]
         self.cache.reserve(slots, new)          # all or nothing
         starts = [self.cache.lengths[s] for s in slots]
-        step = pack_step(slots, token_lists, starts, self.device, self.ws)
         n_want = len(rows)
+        if self.use_graphs and all(n == 1 for n in new) and len(slots) <= 256:
+            if self._graphs is None:
+                from .graph import DecodeGraphs
+                self._graphs = DecodeGraphs(self)
+            all_logits = self._graphs.run(slots, [tl[0] for tl in token_lists], starts)
+            self.cache.commit(slots, new)
+            if rows == list(range(len(slots))):
+                return all_logits.clone()          # the graph's buffer is overwritten by the next step
+            return all_logits[torch.tensor(rows, dtype=torch.long, device=self.device)]
+        step = pack_step(slots, token_lists, starts, self.device, self.ws)
         want_rows = (torch.tensor(rows, dtype=torch.int32).to(self.device) if n_want
                      else torch.empty(0, dtype=torch.int32, device=self.device))
         logits = self.model.forward(step, self.cache, want_rows, n_want)

@@ -99,6 +99,10 @@ class DecoderModel:
         for layer in self.layers:
             layer.rt = rt
 
+    def graph_safe(self) -> bool:
+        """True when every part may run under HIP graph capture (see `Part.graph_safe`)."""
+        return all(getattr(part, "graph_safe", False) for part, _ in self._named_parts())
+
     # ---- what the cache must hold ----------------------------------------------------
     def cache_needs(self) -> Dict[int, CacheNeed]:
         needs: Dict[int, CacheNeed] = {}

@@ -35,6 +35,8 @@ def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
 
 
 class GQAAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: Optional[int] = None, position: Optional[str] = "rope", scale: Optional[float] = None):
         if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:

@@ -40,7 +40,14 @@ class Runtime:
 
 
 class Part:
-    """Base of every part: declares tensors by name, receives them once loaded."""
+    """Base of every part: declares tensors by name, receives them once loaded.
+
+    `graph_safe`: the part's forward launches the same kernels with the same arguments
+    for every step of one shape and reads everything that varies from device arrays of
+    the step, so a single-token step may be captured in a HIP graph and replayed.  Parts
+    that decide anything on the host from the step's contents leave it False."""
+
+    graph_safe = False
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         return []

@@ -18,6 +18,8 @@ from .linear import linear
 
 
 class TokenEmbedding(Embedding):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.V, self.H = int(vocab_size), int(hidden_size)
         self.weight = None
@@ -34,6 +36,8 @@ class TokenEmbedding(Embedding):
 
 
 class LMHead(OutputHead):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None):
         self.V, self.H, self.tied_to = int(vocab_size), int(hidden_size), tied_to
         self.weight = None

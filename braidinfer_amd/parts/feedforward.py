@@ -14,6 +14,8 @@ from .linear import fuse_rows, linear
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.H, self.I = int(hidden_size), int(intermediate_size)
         self.w_gu = self.w_d = None

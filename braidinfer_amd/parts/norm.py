@@ -12,6 +12,8 @@ from .base import Norm, Runtime, register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size, self.eps = int(size), float(eps)
         self.weight: Optional[torch.Tensor] = None

@@ -19,6 +19,8 @@ from .base import PositionEncoding, RotaryTables, Runtime, register_part
 
 
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, rotary_dim: int, theta: float, pairing: str = "half"):
         if rotary_dim <= 0 or rotary_dim % 2:
             raise ConfigError(f"rotary_dim must be positive and even, got {rotary_dim}")
@@ -43,6 +45,8 @@ class RotaryEncoding(PositionEncoding):
 
 class NoPositionEncoding(PositionEncoding):
     """Mixers that ask for this encoding rotate nothing."""
+    graph_safe = True
+
 
     def load(self, tensors, prefix, rt):
         self.rt = rt

@@ -202,3 +202,47 @@ def test_a_far_key_among_hundreds_is_found(tmp_path):
             assert int(ref.argmax()) == 1, "the test's weights must make the marker win in the plain implementation"
             assert int(got.argmax()) == 1, f"{dtype}: the key at position {far} was lost"
             close(got[None], ref[None], dtype, f"far key at {far}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(tiny_folders, dtype):
+    """Single-token steps are replayed from HIP graphs.  Every replay is checked against
+    the same step run eagerly on a second engine, with eager work (prompts of other
+    requests, slots freed and used again, batch sizes that change) between the replays."""
+    folder, cfg, w = tiny_folders["b"]
+    g = B.Engine.from_folder(folder, dtype=dtype, max_tokens=2048)
+    e = B.Engine.from_folder(folder, dtype=dtype, max_tokens=2048, use_graphs=False)
+    assert g.use_graphs and not e.use_graphs
+    rng = np.random.default_rng(0)
+    seqs = [tokens(cfg, 90, 50 + i) for i in range(5)]
+    slots_g, slots_e, pos = {}, {}, {}
+
+    def start(i, n):
+        slots_g[i], slots_e[i], pos[i] = g.alloc_slot(), e.alloc_slot(), n
+        a = g.step([StepEntry(slots_g[i], seqs[i][:n], [n - 1])]).cpu().numpy()
+        b_ = e.step([StepEntry(slots_e[i], seqs[i][:n], [n - 1])]).cpu().numpy()
+        assert np.array_equal(a, b_)
+
+    def stop(i):
+        g.free_slot(slots_g.pop(i)); e.free_slot(slots_e.pop(i)); pos.pop(i)
+
+    start(0, 10); start(1, 3)
+    for it in range(60):
+        live = sorted(pos)
+        a = g.step([StepEntry(slots_g[i], [seqs[i][pos[i]]], [0]) for i in live]).cpu().numpy()
+        b_ = e.step([StepEntry(slots_e[i], [seqs[i][pos[i]]], [0]) for i in live]).cpu().numpy()
+        ref = np.stack([P.forward(cfg, w, seqs[i][:pos[i] + 1])[-1] for i in live])
+        close(a, ref, dtype, f"replay {it}")
+        # the split count of the graph follows the cache's longest sequence, the eager step's its
+        # own: the same numbers added in another order
+        assert np.abs(a - b_).max() <= CUT_TOL[dtype] * np.abs(ref).max() + 1e-5 * np.abs(ref).max()
+        for i in live:
+            pos[i] += 1
+        if it == 5: start(2, 40)
+        if it == 9: stop(1)
+        if it == 12: start(3, 64); start(1, 7)
+        if it == 30: stop(0); start(4, 5)
+        for i in [i for i in pos if pos[i] >= 89]:
+            stop(i)
+        if not pos:
+            break
