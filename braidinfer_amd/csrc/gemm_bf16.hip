@@ -21,12 +21,19 @@
 #define OUT_BF16 0
 #define OUT_F32 1
 #define OUT_F32_ACC 2
+// SwiGLU epilogue: W holds gate and up rows interleaved in blocks of 16 (8 gate rows, then
+// the 8 up rows of the same outputs); the output is bf16 [M, N / 2] with
+// out[m][8 b + j] = silu(gate) * up, silu(g) = g / (1 + exp(-g))
+// (reference: kernels/megakernel_ops.hip:1538-1544, fused there too, per output row).
+#define OUT_SWIGLU 3
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
 
 template <int MODE>
 __device__ __forceinline__ void store_out(void* C, size_t idx, float v) {
     if (MODE == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
     else if (MODE == OUT_F32) ((float*)C)[idx] = v;
-    else ((float*)C)[idx] += v;
+    else if (MODE == OUT_F32_ACC) ((float*)C)[idx] += v;
 }
 
 __device__ __forceinline__ bf16x8 zero8() {
@@ -148,6 +155,17 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int n = n0 + wn + j * 32 + (lane & 31);
+            if (MODE == OUT_SWIGLU) {
+                // the up value of a gate column sits 8 columns on, in lane ^ 8
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float other = __shfl_xor(acc[i][j][r], 8, 64);
+                    const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if ((lane & 8) == 0 && n < N && m < M)
+                        ((bf16*)C)[(size_t)m * ldc + (n >> 4) * 8 + (n & 7)] = (bf16)silu_mul(acc[i][j][r], other);
+                }
+                continue;
+            }
             if (n >= N) continue;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -180,24 +198,29 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
     if (aligned) {
         if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16, true);
         else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32, true);
-        else BR_LAUNCH_TILE(OUT_F32_ACC, true);
+        else if (mode == OUT_F32_ACC) BR_LAUNCH_TILE(OUT_F32_ACC, true);
+        else BR_LAUNCH_TILE(OUT_SWIGLU, true);
     } else {
         if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16, false);
         else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32, false);
-        else BR_LAUNCH_TILE(OUT_F32_ACC, false);
+        else if (mode == OUT_F32_ACC) BR_LAUNCH_TILE(OUT_F32_ACC, false);
+        else BR_LAUNCH_TILE(OUT_SWIGLU, false);
     }
 #undef BR_LAUNCH_TILE
     return br_check_launch();
 }
 
 // ----------------------------------------------------------------- gemm_skinny ------
-// grid = ceil(N / (16 RB)); block = 256 (4 waves).  Needs K % 8 == 0 and 16-byte aligned rows.
-template <int MB, int RB, int MODE>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
-                                                          void* __restrict__ C, int M, int N, int K,
-                                                          size_t lda, size_t ldc) {
+// grid = ceil(N / (16 RB)); block = 64 NW.  Needs K % 8 == 0 and 16-byte aligned rows.
+// Every wave keeps U chunks of 128 k in flight (the loads of all U are issued before the
+// first product), which is what fills the memory pipeline; rows beyond N or M are read
+// from the last valid row instead of being masked, and dropped at the store.
+template <int MB, int RB, int U, int NW, int MODE>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                              void* __restrict__ C, int M, int N, int K,
+                                                              size_t lda, size_t ldc) {
     constexpr int ROWS = 16 * RB, COLS = 16 * MB;
-    __shared__ float red[4][ROWS][COLS + 1];
+    __shared__ float red[NW][ROWS][COLS + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * ROWS;
@@ -209,26 +232,66 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
         for (int j = 0; j < MB; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
-
-    const int nchunks = (K + 127) / 128;
-    for (int c = wave; c < nchunks; c += 4) {
-        const int kb = c * 128 + g * 32;
-        bf16x8 fw[RB][4], fx[MB][4];
+    const bf16* wp[RB];
+    const bf16* xp[MB];
 #pragma unroll
-        for (int i = 0; i < RB; ++i)
+    for (int i = 0; i < RB; ++i) {
+        int row = n0 + i * 16 + r16;
+        if (row > N - 1) row = N - 1;
+        wp[i] = W + (size_t)row * K + g * 8;
+    }
 #pragma unroll
-            for (int s = 0; s < 4; ++s) fw[i][s] = load8<true>(W, (size_t)K, n0 + i * 16 + r16, N, kb + s * 8, K);
+    for (int j = 0; j < MB; ++j) {
+        int row = j * 16 + r16;
+        if (row > M - 1) row = M - 1;
+        xp[j] = A + (size_t)row * lda + g * 8;
+    }
+    // lane (row r16, group g) holds k = chunk * 128 + s * 32 + g * 8 + [0, 8) for s = 0..3
+    const int nfull = K / 128;
+    int c = wave * U;
+    for (; c + U <= nfull; c += NW * U) {
+        bf16x8 fw[U][RB][4], fx[U][MB][4];
 #pragma unroll
-        for (int j = 0; j < MB; ++j)
-#pragma unroll
-            for (int s = 0; s < 4; ++s) fx[j][s] = load8<true>(A, lda, j * 16 + r16, M, kb + s * 8, K);
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int u = 0; u < U; ++u) {
+            const int kb = (c + u) * 128;
 #pragma unroll
             for (int i = 0; i < RB; ++i)
 #pragma unroll
-                for (int j = 0; j < MB; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i][s], fx[j][s], acc[i][j], 0, 0, 0);
+                for (int s = 0; s < 4; ++s) fw[u][i][s] = *(const bf16x8*)(wp[i] + kb + s * 32);
+#pragma unroll
+            for (int j = 0; j < MB; ++j)
+#pragma unroll
+                for (int s = 0; s < 4; ++s) fx[u][j][s] = *(const bf16x8*)(xp[j] + kb + s * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+#pragma unroll
+                    for (int j = 0; j < MB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[u][i][s], fx[u][j][s], acc[i][j], 0, 0, 0);
+    }
+    // this wave's leftover chunks (fewer than U, or the partial last chunk), guarded along k
+    const int nch = (K + 127) / 128;
+    for (int u = 0; u < U; ++u) {
+        const int cc = c + u;
+        if (cc >= nch) break;
+        const int kb = cc * 128;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const bool in = kb + s * 32 + g * 8 + 8 <= K;
+#pragma unroll
+            for (int i = 0; i < RB; ++i) {
+                const bf16x8 a = in ? *(const bf16x8*)(wp[i] + kb + s * 32) : zero8();
+#pragma unroll
+                for (int j = 0; j < MB; ++j) {
+                    const bf16x8 b = in ? *(const bf16x8*)(xp[j] + kb + s * 32) : zero8();
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i][j], 0, 0, 0);
+                }
+            }
+        }
     }
     // acc[i][j][r]: weight row = 16 i + 4 (lane / 16) + r, batch row = 16 j + lane % 16
 #pragma unroll
@@ -238,23 +301,43 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
 #pragma unroll
             for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * g + r][j * 16 + r16] = acc[i][j][r];
     __syncthreads();
-    for (int e = tid; e < ROWS * COLS; e += 256) {
+    if (MODE == OUT_SWIGLU) {
+        for (int e = tid; e < (ROWS / 2) * COLS; e += NW * 64) {
+            const int m = e / (ROWS / 2), jl = e - m * (ROWS / 2);
+            const int gl = (jl >> 3) * 16 + (jl & 7);            // gate row in the tile; its up row is 8 on
+            if (m < M && n0 + gl + 8 < N) {
+                float gv = 0.f, uv = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) { gv += red[w][gl][m]; uv += red[w][gl + 8][m]; }
+                ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
+            }
+        }
+        return;
+    }
+    for (int e = tid; e < ROWS * COLS; e += NW * 64) {
         const int m = e / ROWS, nl = e - m * ROWS;   // consecutive threads: consecutive weight rows
         const int n = n0 + nl;
         if (m < M && n < N) {
-            const float v = ((red[0][nl][m] + red[1][nl][m]) + red[2][nl][m]) + red[3][nl][m];
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) v += red[w][nl][m];     // in wave order, always
             store_out<MODE>(C, (size_t)m * ldc + n, v);
         }
     }
 }
 
-template <int MB, int RB>
+template <int MB, int RB, int U, int NW>
 static int launch_skinny(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                          int mode, hipStream_t s) {
     const unsigned grid = (unsigned)((N + 16 * RB - 1) / (16 * RB));
-    if (mode == OUT_BF16) gemm_skinny_kernel<MB, RB, OUT_BF16><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
-    else if (mode == OUT_F32) gemm_skinny_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
-    else gemm_skinny_kernel<MB, RB, OUT_F32_ACC><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    if (mode == OUT_BF16)
+        gemm_skinny_kernel<MB, RB, U, NW, OUT_BF16><<<grid, NW * 64, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else if (mode == OUT_SWIGLU)
+        gemm_skinny_kernel<MB, RB, U, NW, OUT_SWIGLU><<<grid, NW * 64, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else if (mode == OUT_F32)
+        gemm_skinny_kernel<MB, RB, U, NW, OUT_F32><<<grid, NW * 64, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else
+        gemm_skinny_kernel<MB, RB, U, NW, OUT_F32_ACC><<<grid, NW * 64, 0, s>>>(A, W, C, M, N, K, lda, ldc);
     return br_check_launch();
 }
 
@@ -262,21 +345,22 @@ static int launch_skinny(const bf16* A, const bf16* W, void* C, int M, int N, in
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
                                size_t ldc, int mode, int kernel, hipStream_t s) {
     if (M <= 0 || N <= 0) return BR_OK;
-    if (K <= 0 || lda < (size_t)K || ldc < (size_t)N || mode < 0 || mode > 2) return BR_BAD_ARG;
+    if (K <= 0 || lda < (size_t)K || mode < 0 || mode > 3) return BR_BAD_ARG;
+    if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
     const bf16* A = (const bf16*)A_;
     const bf16* W = (const bf16*)W_;
     const bool aligned = (K % 8 == 0) && (lda % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     if (kernel == 3 && (!aligned || M > 64)) return BR_BAD_ARG;
     if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : ((M >= 1024 && N >= 1024) ? 2 : 1);
     if (kernel == 3) {
-        // rows per workgroup: keep at least ~2 workgroups per CU when N allows it
+        // shapes measured on cold weights (cycled through more than the 256 MB cache)
         const bool wide = N >= 16384;
-        if (M <= 16) return wide ? launch_skinny<1, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
-                                 : launch_skinny<1, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
-        if (M <= 32) return wide ? launch_skinny<2, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
-                                 : launch_skinny<2, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
-        return wide ? launch_skinny<4, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
-                    : launch_skinny<4, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
+        if (M <= 16) return (wide && M > 4) ? launch_skinny<1, 1, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                            : launch_skinny<1, 1, 4, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
+        if (M <= 32) return wide ? launch_skinny<2, 4, 1, 4>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                 : launch_skinny<2, 2, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
+        return wide ? launch_skinny<4, 4, 1, 4>(A, W, C, M, N, K, lda, ldc, mode, s)
+                    : launch_skinny<4, 2, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
     }
     if (kernel == 2) return launch_tile<256, 128, 32, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, aligned, s);
     return launch_tile<128, 128, 64, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, aligned, s);

@@ -26,12 +26,13 @@ __device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int o
     if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
 }
 
-__global__ __launch_bounds__(SBLOCK) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
-    __shared__ float sv[SBLOCK / 64];
-    __shared__ int si[SBLOCK / 64];
+#define ABLOCK 1024
+__global__ __launch_bounds__(ABLOCK) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+    __shared__ float sv[ABLOCK / 64];
+    __shared__ int si[ABLOCK / 64];
     const float* r = logits + (size_t)blockIdx.x * V;
     float bv = -INFINITY; int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += SBLOCK) argmax_combine(bv, bi, r[i], i);
+    for (int i = threadIdx.x; i < V; i += ABLOCK) argmax_combine(bv, bi, r[i], i);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         float ov = __shfl_xor(bv, o, 64); int oi = __shfl_xor(bi, o, 64);
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(SBLOCK) void argmax_kernel(const float* __restrict_
     if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < SBLOCK / 64; ++w) argmax_combine(bv, bi, sv[w], si[w]);
+        for (int w = 1; w < ABLOCK / 64; ++w) argmax_combine(bv, bi, sv[w], si[w]);
         out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
     }
 }
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(SBLOCK) void argmax_kernel(const float* __restrict_
 extern "C" int br_argmax(const float* logits, int* out, int B, int V, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0) return BR_BAD_ARG;
-    argmax_kernel<<<B, SBLOCK, 0, s>>>(logits, out, V);
+    argmax_kernel<<<B, ABLOCK, 0, s>>>(logits, out, V);
     return br_check_launch();
 }
 

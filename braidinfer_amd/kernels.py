@@ -203,6 +203,30 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"gemm: a is {a.dtype} and w is {w.dtype}; both float32 or both bfloat16")
 
 
+def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: int = 0) -> None:
+    """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) in one bf16 product: `w_gu` [2 I, K] holds
+    gate and up rows interleaved in blocks of 16 (see `interleave_gate_up`)."""
+    for t in (a, w_gu, out):
+        if not t.is_cuda:
+            raise KernelError(f"gemm_swiglu: tensor on {t.device}; kernels run on the GPU only")
+    _req(a.dtype == w_gu.dtype == out.dtype == torch.bfloat16, "gemm_swiglu: bfloat16 only")
+    M, K = a.shape
+    N = w_gu.shape[0]
+    _req(N % 16 == 0 and w_gu.shape[1] == K and out.shape == (M, N // 2), "gemm_swiglu: shapes")
+    _req(w_gu.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1, "gemm_swiglu: rows must be dense")
+    lda, ldc = (a.stride(0) if M > 1 else K), (out.stride(0) if M > 1 else N // 2)
+    f = _fn("gemm_bf16", "br_gemm_bf16_ex", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P])
+    _check(f(_ptr(a), _ptr(w_gu), _ptr(out), M, N, K, lda, ldc, 3, kernel, _stream()), "gemm_swiglu")
+
+
+def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:
+    """[2 I, K]: blocks of 8 gate rows followed by the 8 up rows of the same outputs."""
+    I, K = w_gate.shape
+    if I % 8:
+        raise KernelError(f"interleave_gate_up: intermediate size {I} is not a multiple of 8")
+    return torch.stack([w_gate.view(I // 8, 8, K), w_up.view(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
+
+
 # ------------------------------------------------------------------- attention -----
 def attention_simple(q: torch.Tensor, q_stride: int, out: torch.Tensor, positions: torch.Tensor,
                      seq_of_token: torch.Tensor, slots: torch.Tensor, block_table: torch.Tensor,

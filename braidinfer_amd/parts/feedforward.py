@@ -29,16 +29,23 @@ class SwiGLU(FeedForward):
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.w_gu = fuse_rows([tensors[prefix + "gate_proj.weight"], tensors[prefix + "up_proj.weight"]])
+        g, u = tensors[prefix + "gate_proj.weight"], tensors[prefix + "up_proj.weight"]
+        # bf16: gate and up rows interleaved so that the product's epilogue applies silu * up
+        # and the [T, 2 I] intermediate is never written
+        self.fused = g.dtype == u.dtype == torch.bfloat16 and rt.is_bf16 and self.I % 8 == 0
+        self.w_gu = K.interleave_gate_up(g, u) if self.fused else fuse_rows([g, u])
         self.w_d = tensors[prefix + "down_proj.weight"].contiguous()
 
     def forward(self, h, x, step) -> None:
         T = step.n_tokens
         dt = self.rt.dtype
-        gu = step.ws.get("ffn_gu", (T, 2 * self.I), dt)
-        linear(h, self.w_gu, gu, step.ws)
         a = step.ws.get("ffn_act", (T, self.I), dt)
-        K.silu_mul(gu, a)
+        if self.fused:
+            K.gemm_swiglu(h, self.w_gu, a)
+        else:
+            gu = step.ws.get("ffn_gu", (T, 2 * self.I), dt)
+            linear(h, self.w_gu, gu, step.ws)
+            K.silu_mul(gu, a)
         linear(a, self.w_d, x, step.ws, accumulate=True)
 
 

@@ -389,3 +389,17 @@ def test_attention_kernels_refuse_what_they_do_not_take():
                                 1.0, 1, None, None)
     with pytest.raises(KernelError, match="multiple of 16"):
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
+
+
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,I,Kd", [(1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032)])
+def test_gemm_with_swiglu_epilogue(M, I, Kd, kernel):
+    if kernel == 3 and (Kd % 8 or M > 64):
+        pytest.skip("the skinny kernel takes M <= 64 and K in steps of 8")
+    a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
+    wg, wu = rnd(I, Kd, seed=2, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=3, scale=0.3, dtype=torch.bfloat16)
+    out = torch.empty(M, I, device=DEV, dtype=torch.bfloat16)
+    K.gemm_swiglu(a, K.interleave_gate_up(wg, wu), out, kernel=kernel)
+    g, u = a.double() @ wg.double().T, a.double() @ wu.double().T
+    want = g / (1 + torch.exp(-g)) * u
+    assert (out.double() - want).abs().max() < 1e-2 * want.abs().max()
