@@ -167,6 +167,189 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         }
 }
 
+// ----------------------------------------------------------- prefill through LDS ----
+// The same computation with the keys and values of a page staged in LDS once per
+// workgroup: grid = (row tiles of 256, nkv, sequences), block = 512 (8 waves of 32 rows).
+// The page after the current one is fetched into registers while the current one is
+// multiplied, and written to the other LDS buffer afterwards.  Tiles are taken from the
+// last (most keys) to the first so the long workgroups start first.
+#define KPAD 8
+#define VLD 72
+template <int NB>
+__global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
+    const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
+    int table_stride, const bf16* __restrict__ cache, int nq, int nkv, int hd, int window, float scale) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int slot = slots[b];
+    const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
+    const int G = nq / nkv;
+    const int rows_total = n_new * G;
+    const int tile = gridDim.x - 1 - blockIdx.x;
+    if (tile * 256 >= rows_total) return;                 // the whole workgroup leaves together
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = tile * 256 + wave * 32;
+    const bool wave_ok = row0 < rows_total;
+    const int c = lane & 31, g = lane >> 5;
+    const int row = row0 + c;
+    const bool row_ok = row < rows_total;
+    const int rr = row_ok ? row : rows_total - 1;
+    const int tok = rr / G, head = kvh * G + rr % G;
+    bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * hd;
+    if (slot < 0) {
+        if (row_ok && g == 0) for (int d = 0; d < hd; ++d) orow[d] = (bf16)0.f;
+        return;
+    }
+    const int ctx = ctx_lens[b], start = ctx - n_new;
+    const int pq = start + tok;
+    // per wave and per workgroup: the positions of the first and last query row
+    const int w_last_row = (row0 + 31 < rows_total ? row0 + 31 : rows_total - 1);
+    const int pq_min_w = start + (wave_ok ? row0 : rows_total - 1) / G, pq_max_w = start + w_last_row / G;
+    const int g_last_row = (tile * 256 + 255 < rows_total ? tile * 256 + 255 : rows_total - 1);
+    const int pq_min_g = start + (tile * 256) / G, pq_max_g = start + g_last_row / G;
+
+    const int kld = hd + KPAD;
+    bf16* Ks = (bf16*)smem_raw;                          // [2][64][kld]
+    bf16* Vs = Ks + 2 * PAGE * kld;                      // [2][NB * 32][VLD]
+
+    const bf16* qrow = q + (size_t)(t0 + tok) * q_stride + (size_t)head * hd;
+    bf16x8 qf[2 * NB];
+#pragma unroll
+    for (int s = 0; s < 2 * NB; ++s) {
+        const int d = s * 16 + 8 * g;
+        qf[s] = (d < hd) ? *(const bf16x8*)(qrow + d) : zero8();
+    }
+    f32x16 acc_o[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+
+    const int* bt = block_table + (size_t)slot * table_stride;
+    const size_t page_elems = (size_t)2 * nkv * PAGE * hd;
+    const size_t k_off = (size_t)kvh * PAGE * hd, v_off = ((size_t)nkv + kvh) * PAGE * hd;
+    int lo = 0;
+    if (window > 0 && pq_min_g - window + 1 > 0) lo = pq_min_g - window + 1;
+    const int pg_first = lo / PAGE, pg_last = pq_max_g / PAGE;
+
+    // cooperative loads: chunk id -> 8 consecutive elements of the page's K part / V^T part
+    constexpr int CH = (NB * 32 * PAGE / 8 + 511) / 512;  // 16-byte chunks per thread and part (NB * 32 >= hd)
+    bf16x8 rk[CH], rv[CH];
+    const int kchunks = PAGE * hd / 8;                   // chunks that exist in each part
+    auto gload = [&](int pi) {
+        const bf16* pg = cache + (size_t)bt[pi] * page_elems;
+        const int limit_local = ctx - pi * PAGE;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            const int id = tid + j * 512;
+            if (id < kchunks) {
+                rk[j] = *(const bf16x8*)(pg + k_off + (size_t)id * 8);
+                bf16x8 v = *(const bf16x8*)(pg + v_off + (size_t)id * 8);
+                const int key0 = (id * 8) % PAGE;        // V^T: [dim][key]
+                if (key0 + 8 > limit_local) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) if (key0 + e >= limit_local) v[e] = (bf16)0.f;
+                }
+                rv[j] = v;
+            }
+        }
+    };
+    auto sstore = [&](int buf) {
+        bf16* ks = Ks + buf * PAGE * kld;
+        bf16* vs = Vs + buf * NB * 32 * VLD;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            const int id = tid + j * 512;
+            if (id < kchunks) {
+                const int e0 = id * 8;
+                *(bf16x8*)(ks + (e0 / hd) * kld + (e0 % hd)) = rk[j];
+                *(bf16x8*)(vs + (e0 / PAGE) * VLD + (e0 % PAGE)) = rv[j];
+            }
+        }
+    };
+
+    gload(pg_first);
+    sstore(0);
+    __syncthreads();
+    for (int pi = pg_first; pi <= pg_last; ++pi) {
+        const int buf = (pi - pg_first) & 1;
+        if (pi < pg_last) gload(pi + 1);
+        const bf16* ks = Ks + buf * PAGE * kld;
+        const bf16* vs = Vs + buf * NB * 32 * VLD;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int kl = half * 32, kb = pi * PAGE + kl;
+            // blocks no row of this wave can see are skipped
+            if (!wave_ok || kb > pq_max_w || (window > 0 && kb + 31 <= pq_min_w - window)) continue;
+            const bf16* krow = ks + (kl + c) * kld;
+            f32x16 s_acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < 2 * NB; ++s) {
+                const int d = s * 16 + 8 * g;
+                const bf16x8 kf = (d < hd) ? *(const bf16x8*)(krow + d) : zero8();
+                s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+            }
+            float sv[16];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
+                const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
+                sv[r] = ok ? s_acc[r] * scale : -INFINITY;
+                mx = fmaxf(mx, sv[r]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float corr = expf(m - m_use);
+            float psum = 0.f;
+            bf16x8 p1, p2;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = expf(sv[r] - m_use);
+                psum += p;
+                if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
+            }
+            lsum = lsum * corr + psum;
+            m = m_new;
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
+                const bf16* vrow = vs + (i * 32 + c) * VLD + kl + 4 * g;   // rows at or beyond hd hold zeros or stale
+                bf16x8 v1 = zero8(), v2 = zero8();
+                if (i * 32 + c < hd) {
+                    v1 = join4(*(const bf16x4*)(vrow), *(const bf16x4*)(vrow + 8));
+                    v2 = join4(*(const bf16x4*)(vrow + 16), *(const bf16x4*)(vrow + 24));
+                }
+                acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i], 0, 0, 0);
+                acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i], 0, 0, 0);
+            }
+        }
+        if (pi < pg_last) sstore(buf ^ 1);
+        __syncthreads();
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (!row_ok) return;
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int d = i * 32 + 8 * r4 + 4 * g;
+            if (d < hd) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16)(acc_o[i][4 * r4 + e] * inv);
+                *(bf16x4*)(orow + d) = o;
+            }
+        }
+}
+
 // ---------------------------------------------------------------------- decode ------
 // One token per sequence.  grid = (splits, nkv * head blocks, sequences), block = 256.
 // The pages a query sees are cut into `nsplit` runs; the 4 waves of a workgroup take a
@@ -336,12 +519,43 @@ static int nb_of(int hd) { return (hd + 31) / 32; }
 extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, const int* cu_seqlens,
                                     const int* slots, const int* ctx_lens, const int* block_table,
                                     int table_stride, const void* cache, int B, int max_new, int nq, int nkv,
-                                    int hd, int page, int window, float scale, hipStream_t s) {
+                                    int hd, int page, int window, float scale, int variant, hipStream_t s) {
     if (B <= 0 || max_new <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
         q_stride % 8 || ((uintptr_t)q % 16) || nkv > 65535 || B > 65535)
         return BR_BAD_ARG;
     const int G = nq / nkv;
+    // variant 0: choose; 1: fragments straight from the cache; 2: pages staged in LDS
+    if (variant == 0) variant = ((size_t)max_new * G >= 256 && hd <= 192) ? 2 : 1;   // beyond 192 the LDS form spills registers
+    if (variant == 2) {
+        dim3 grid2(((size_t)max_new * G + 255) / 256, nkv, B);
+        const int nb = nb_of(hd) == 5 ? 6 : (nb_of(hd) == 7 ? 8 : nb_of(hd));
+        const size_t lds = (size_t)2 * (PAGE * (hd + KPAD) + nb * 32 * VLD) * sizeof(bf16);
+#define BR_PREFILL_LDS(N)                                                                                  \
+    do {                                                                                                   \
+        auto kern = attn_prefill_lds_kernel<N>;                                                            \
+        static bool set = false;                                                                           \
+        if (!set) {                                                                                        \
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,         \
+                                    (int)((size_t)2 * (PAGE * (N * 32 + KPAD) + N * 32 * VLD) * 2)) != hipSuccess) \
+                return BR_LAUNCH_FAILED;                                                                   \
+            set = true;                                                                                    \
+        }                                                                                                  \
+        kern<<<grid2, 512, lds, s>>>((const bf16*)q, q_stride, (bf16*)out, cu_seqlens, slots, ctx_lens,   \
+                                     block_table, table_stride, (const bf16*)cache, nq, nkv, hd, window,   \
+                                     scale);                                                               \
+    } while (0)
+        switch (nb) {
+            case 1: BR_PREFILL_LDS(1); break;
+            case 2: BR_PREFILL_LDS(2); break;
+            case 3: BR_PREFILL_LDS(3); break;
+            case 4: BR_PREFILL_LDS(4); break;
+            case 6: BR_PREFILL_LDS(6); break;
+            default: BR_PREFILL_LDS(8); break;
+        }
+#undef BR_PREFILL_LDS
+        return br_check_launch();
+    }
     dim3 grid(((size_t)max_new * G + 127) / 128, nkv, B);
 #define BR_PREFILL(N)                                                                                      \
     attn_prefill_kernel<N><<<grid, 256, 0, s>>>((const bf16*)q, q_stride, (bf16*)out, cu_seqlens, slots,  \

@@ -58,7 +58,7 @@ __device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, size_t ld
 }
 
 // ------------------------------------------------------------------ gemm_tile -------
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MODE, bool ALIGNED>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MODE, bool ALIGNED, bool KFULL>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                         void* __restrict__ C, int M, int N, int K,
                                                         size_t lda, size_t ldc, int tiles_m, int tiles_n) {
@@ -95,17 +95,39 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+    // Rows beyond M or N are read from the last valid row (and dropped at the store), so a
+    // load needs a guard along k only; with K a multiple of BK and 16-byte aligned rows
+    // (KFULL) it needs none.
     bf16x8 ra[A_CHUNKS], rb[B_CHUNKS];
+    const bf16* ap[A_CHUNKS];
+    const bf16* bp[B_CHUNKS];
+    int akc[A_CHUNKS], bkc[B_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < A_CHUNKS; ++c) {
+        const int id = tid + c * 256;
+        int r = m0 + id / CPR;
+        if (r > M - 1) r = M - 1;
+        akc[c] = (id % CPR) * 8;
+        ap[c] = A + (size_t)r * lda + akc[c];
+    }
+#pragma unroll
+    for (int c = 0; c < B_CHUNKS; ++c) {
+        const int id = tid + c * 256;
+        int r = n0 + id / CPR;
+        if (r > N - 1) r = N - 1;
+        bkc[c] = (id % CPR) * 8;
+        bp[c] = W + (size_t)r * K + bkc[c];
+    }
     auto gload = [&](int k0) {
 #pragma unroll
         for (int c = 0; c < A_CHUNKS; ++c) {
-            const int id = tid + c * 256, r = id / CPR, kc = (id % CPR) * 8;
-            ra[c] = load8<ALIGNED>(A, lda, m0 + r, M, k0 + kc, K);
+            if (KFULL) ra[c] = *(const bf16x8*)(ap[c] + k0);
+            else ra[c] = load8<ALIGNED>(ap[c] - akc[c], 0, 0, 1, k0 + akc[c], K);
         }
 #pragma unroll
         for (int c = 0; c < B_CHUNKS; ++c) {
-            const int id = tid + c * 256, r = id / CPR, kc = (id % CPR) * 8;
-            rb[c] = load8<ALIGNED>(W, (size_t)K, n0 + r, N, k0 + kc, K);
+            if (KFULL) rb[c] = *(const bf16x8*)(bp[c] + k0);
+            else rb[c] = load8<ALIGNED>(bp[c] - bkc[c], 0, 0, 1, k0 + bkc[c], K);
         }
     };
     auto sstore = [&](int buf) {
@@ -182,9 +204,9 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
     const long long total = (long long)tm * tn;
     if (total > 0x7fffffffLL) return BR_BAD_ARG;
     const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
-#define BR_LAUNCH_TILE(MODE, AL)                                                                        \
+#define BR_LAUNCH_TILE_(MODE, AL, KF)                                                                    \
     do {                                                                                                \
-        auto kern = gemm_tile_kernel<BM, BN, BK, WAVES_M, WAVES_N, MODE, AL>;                           \
+        auto kern = gemm_tile_kernel<BM, BN, BK, WAVES_M, WAVES_N, MODE, AL, KF>;                       \
         if (lds > 48 * 1024) {                                                                          \
             static bool set = false;                                                                    \
             if (!set) {                                                                                 \
@@ -195,17 +217,17 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
         }                                                                                               \
         kern<<<(unsigned)total, 256, lds, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);                     \
     } while (0)
-    if (aligned) {
-        if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16, true);
-        else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32, true);
-        else if (mode == OUT_F32_ACC) BR_LAUNCH_TILE(OUT_F32_ACC, true);
-        else BR_LAUNCH_TILE(OUT_SWIGLU, true);
-    } else {
-        if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16, false);
-        else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32, false);
-        else if (mode == OUT_F32_ACC) BR_LAUNCH_TILE(OUT_F32_ACC, false);
-        else BR_LAUNCH_TILE(OUT_SWIGLU, false);
-    }
+#define BR_LAUNCH_TILE(MODE)                                                 \
+    do {                                                                     \
+        if (aligned && K % BK == 0) BR_LAUNCH_TILE_(MODE, true, true);       \
+        else if (aligned) BR_LAUNCH_TILE_(MODE, true, false);                \
+        else BR_LAUNCH_TILE_(MODE, false, false);                            \
+    } while (0)
+    if (mode == OUT_BF16) BR_LAUNCH_TILE(OUT_BF16);
+    else if (mode == OUT_F32) BR_LAUNCH_TILE(OUT_F32);
+    else if (mode == OUT_F32_ACC) BR_LAUNCH_TILE(OUT_F32_ACC);
+    else BR_LAUNCH_TILE(OUT_SWIGLU);
+#undef BR_LAUNCH_TILE_
 #undef BR_LAUNCH_TILE
     return br_check_launch();
 }
@@ -351,7 +373,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     const bf16* W = (const bf16*)W_;
     const bool aligned = (K % 8 == 0) && (lda % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     if (kernel == 3 && (!aligned || M > 64)) return BR_BAD_ARG;
-    if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : ((M >= 1024 && N >= 1024) ? 2 : 1);
+    if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : 1;
     if (kernel == 3) {
         // shapes measured on cold weights (cycled through more than the 256 MB cache)
         const bool wide = N >= 16384;

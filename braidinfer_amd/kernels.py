@@ -248,8 +248,10 @@ def attention_simple(q: torch.Tensor, q_stride: int, out: torch.Tensor, position
 def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu_seqlens: torch.Tensor,
                            slots: torch.Tensor, ctx_lens: torch.Tensor, block_table: torch.Tensor,
                            cache: torch.Tensor, B: int, max_new: int, nq: int, nkv: int, hd: int, page: int,
-                           window: Optional[int], scale: float) -> None:
-    """Flash attention on the matrix cores for steps with several tokens per sequence."""
+                           window: Optional[int], scale: float, variant: int = 0) -> None:
+    """Flash attention on the matrix cores for steps with several tokens per sequence.
+    `variant` 1 reads operand fragments straight from the cache, 2 stages pages in LDS
+    (for long prompts), 0 chooses by the step's longest sequence."""
     _dev("attention_prefill_bf16", out, cu_seqlens, slots, ctx_lens, block_table, cache)
     _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
          "attention_prefill_bf16: bfloat16 only")
@@ -258,10 +260,10 @@ def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu
     _req(cache.shape[1:] == (2, nkv, page, hd), "attention_prefill_bf16: cache unit must be [pages, 2, nkv, page, hd]")
     _req(out.shape[1] == nq * hd and nq % nkv == 0, "attention_prefill_bf16: out must be [T, nq * hd]")
     f = _fn("attention_bf16", "br_attn_prefill_bf16",
-            [_P, c_size_t, _P, _P, _P, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, _P])
+            [_P, c_size_t, _P, _P, _P, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P])
     _check(f(_ptr(q), q_stride, _ptr(out), _ptr(cu_seqlens), _ptr(slots), _ptr(ctx_lens), _ptr(block_table),
              block_table.shape[1], _ptr(cache), B, max_new, nq, nkv, hd, page, int(window or 0), float(scale),
-             _stream()), "attention_prefill_bf16")
+             variant, _stream()), "attention_prefill_bf16")
 
 
 def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slots: torch.Tensor,

@@ -330,7 +330,8 @@ def _multi_seq_cache(lens, nkv, hd, seed):
 
 @pytest.mark.parametrize("nq,nkv,hd,window", [(4, 2, 16, None), (6, 3, 32, 8), (5, 1, 48, 70), (32, 8, 128, None),
                                               (8, 2, 128, 100), (3, 3, 80, None), (2, 1, 256, 33), (20, 1, 64, None)])
-def test_attention_prefill_matrix_cores(nq, nkv, hd, window):
+@pytest.mark.parametrize("variant", [1, 2])
+def test_attention_prefill_matrix_cores(nq, nkv, hd, window, variant):
     lens = [200, 37, 64, 1, 130]             # lengths after the step
     new = [200, 30, 3, 1, 65]                # tokens of this step (the rest is earlier context)
     ks, vs, cache, table = _multi_seq_cache(lens, nkv, hd, seed=nq + hd)
@@ -341,7 +342,7 @@ def test_attention_prefill_matrix_cores(nq, nkv, hd, window):
         cu.append(cu[-1] + n)
     out = torch.full((T, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
     K.attention_prefill_bf16(q.reshape(T, nq * hd), nq * hd, out, i32(cu), i32([1, 2, 3, 4, 5]), i32(lens), table, cache,
-                             len(lens), max(new), nq, nkv, hd, 64, window, 1 / math.sqrt(hd))
+                             len(lens), max(new), nq, nkv, hd, 64, window, 1 / math.sqrt(hd), variant)
     pos = torch.cat([torch.arange(l - n, l) for l, n in zip(lens, new)]).int().to(DEV)
     sot = torch.cat([torch.full((n,), b) for b, n in enumerate(new)]).int().to(DEV)
     simple = torch.empty_like(out)
