@@ -31,6 +31,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the prefill of --prefill-tokens (for profiles); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -57,6 +59,27 @@ def main() -> int:
     layer_params = (nq + 2 * nkv) * hd * H + H * nq * hd + 3 * H * I
     weight_bytes = (layers * layer_params + V * H) * esz + (2 * layers + 1) * H * 4
     kv_bytes_per_token = 2 * nkv * hd * esz * layers
+
+    def prefill(T, reps=4):
+        rng = np.random.default_rng(5)
+        prompt = [int(t) for t in rng.integers(0, V, T)]
+        times = []
+        for rep in range(reps):
+            s = eng.alloc_slot()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            eng.step([StepEntry(s, prompt, [T - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.free_slot(s)
+        pt = min(times[1:])
+        flops = 2.0 * layers * layer_params * T + 2.0 * V * H + 2.0 * T * T * hd * nq * layers
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3), "frac": round(flops / pt / peak, 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s", "layers": layers, "prefill": prefill(args.prefill_tokens)}), flush=True)
+        return 0
 
     def decode(batch, steps, warmup, seed):
         rng = np.random.default_rng(seed)
@@ -105,8 +128,8 @@ def main() -> int:
                    "hidden": H, "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
                    "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
                    "sliding_window": cfg.sliding_window, "global_batch": args.batch, "seq_len": args.context,
-                   "prompt_len_min": 128, "prompt_len_max": 2048, "mean_prompt_len": round(mean_len, 1),
-                   "weights": "random N(0,0.02)", "parallelism": "single GPU"},
+                   "prompt_lens": "uniform[128,2048]", "mean_prompt_len": round(mean_len, 1),
+                   "weights": "random N(0,0.02) bf16", "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(nbytes / dt / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(nbytes / dt / PEAK_HBM, 4)},
     }
@@ -121,24 +144,7 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / d, 2)
             print(f"[bench] batch {b}: {d * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
         line["points"] = points
-        # prefill of one prompt
-        T = args.prefill_tokens
-        rng = np.random.default_rng(5)
-        prompt = [int(t) for t in rng.integers(0, V, T)]
-        times = []
-        for rep in range(4):
-            s = eng.alloc_slot()
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            eng.step([StepEntry(s, prompt, [T - 1])])
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t)
-            eng.free_slot(s)
-        pt = min(times[1:])
-        flops = 2.0 * layers * layer_params * T + 2.0 * V * H + 2.0 * T * T * hd * nq * layers
-        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-        line["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                           "frac": round(flops / pt / peak, 4)}
+        line["prefill"] = prefill(args.prefill_tokens)
     print(json.dumps(line), flush=True)
     return 0
 

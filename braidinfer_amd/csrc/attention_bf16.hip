@@ -405,18 +405,35 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         for (int half = 0; half < 2; ++half) {
             const int kl = half * 32, kb = pos0 + kl;
             if (kb >= ctx || kb + 32 <= lo) continue;
+            // every load of the block is issued before the first product: keys and values
+            // arrive in one memory round trip instead of two
+            bf16x8 kf[2][NB], vf[2 * NB];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bf16* krow = pg + k_off + (size_t)(kl + 16 * j + c) * hd;
+#pragma unroll
+                for (int s = 0; s < NB; ++s) {
+                    const int d = s * 32 + 8 * g;
+                    kf[j][s] = (d < hd) ? *(const bf16x8*)(krow + d) : zero8();
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 2 * NB; ++i) {
+                const int dim = i * 16 + c;
+                vf[i] = zero8();
+                if (dim < hd) {
+                    const bf16* vrow = pg + v_off + (size_t)dim * PAGE;
+                    vf[i] = join4(load_vt4(vrow, kl + 4 * g, limit_local), load_vt4(vrow, kl + 16 + 4 * g, limit_local));
+                }
+            }
             f32x4 s_acc[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) s_acc[j][r] = 0.f;
-                const bf16* krow = pg + k_off + (size_t)(kl + 16 * j + c) * hd;
 #pragma unroll
-                for (int s = 0; s < NB; ++s) {
-                    const int d = s * 32 + 8 * g;
-                    const bf16x8 kf = (d < hd) ? *(const bf16x8*)(krow + d) : zero8();
-                    s_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s_acc[j], 0, 0, 0);
-                }
+                for (int s = 0; s < NB; ++s)
+                    s_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j][s], qf[s], s_acc[j], 0, 0, 0);
             }
             // s_acc[j][r]: key kb + 16 j + 4 g + r, head = this lane's column
             float sv[8];
@@ -446,13 +463,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
             for (int i = 0; i < 2 * NB; ++i) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc_o[i][r] *= corr;
-                const int dim = i * 16 + c;
-                bf16x8 vf = zero8();
-                if (dim < hd) {
-                    const bf16* vrow = pg + v_off + (size_t)dim * PAGE;
-                    vf = join4(load_vt4(vrow, kl + 4 * g, limit_local), load_vt4(vrow, kl + 16 + 4 * g, limit_local));
-                }
-                acc_o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc_o[i], 0, 0, 0);
+                acc_o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[i], pf, acc_o[i], 0, 0, 0);
             }
         }
     }

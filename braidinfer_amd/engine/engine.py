@@ -12,6 +12,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from ..cache import SequenceCache
@@ -132,9 +133,14 @@ class Engine:
         for e, tl in zip(entries, token_lists):
             if not tl:
                 raise StepError(f"slot {e.slot}: an entry brings no tokens")
-            for t in tl:
-                if not isinstance(t, int) or isinstance(t, bool) or not 0 <= t < V:
-                    raise StepError(f"slot {e.slot}: token {t!r} is outside the vocabulary of {V}")
+            try:
+                arr = np.asarray(tl)
+            except (ValueError, TypeError):
+                arr = np.asarray([], dtype=object)
+            if arr.ndim != 1 or arr.dtype.kind not in "iu" or int(arr.min()) < 0 or int(arr.max()) >= V:
+                bad = next((t for t in tl if not isinstance(t, (int, np.integer)) or isinstance(t, bool)
+                            or not 0 <= t < V), None)
+                raise StepError(f"slot {e.slot}: token {bad!r} is outside the vocabulary of {V}")
             for w in e.want:
                 if not isinstance(w, int) or not 0 <= w < len(tl):
                     raise StepError(f"slot {e.slot}: wanted place {w!r} is outside its {len(tl)} tokens")
@@ -147,7 +153,7 @@ class Engine:
         if self.use_graphs and all(n == 1 for n in new) and len(slots) <= 256:
             if self._graphs is None:
                 from .graph import DecodeGraphs
-                self._graphs = DecodeGraphs(self)
+                self._graphs = DecodeGraphs(self.model, self.cache, self.device)
             all_logits = self._graphs.run(slots, [tl[0] for tl in token_lists], starts)
             self.cache.commit(slots, new)
             if rows == list(range(len(slots))):

@@ -11,6 +11,7 @@ step clears memory.
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Sequence
 
 import torch
@@ -26,10 +27,15 @@ def bucket_of(n: int) -> int:
 
 
 class DecodeGraph:
-    def __init__(self, engine, batch: int):
-        self.engine = engine
+    """One recorded step of `batch` sequences.  It refers to the model and the cache, not
+    to the engine that owns it: an engine dropped by its user is then freed at once by
+    reference counting, never by the cycle collector at an arbitrary later moment (which
+    may be another graph's capture, where destroying a graph or freeing device memory is
+    not permitted)."""
+
+    def __init__(self, model, cache, device, batch: int):
         self.B = B = batch
-        dev = engine.device
+        dev = device
         self.ws = Workspace(dev)            # its buffers belong to the recorded graph for good
         # one int32 array: tokens | positions | slots | ctx   (refreshed per step)
         self.ints = torch.zeros(4 * B, dtype=torch.int32, device=dev)
@@ -40,15 +46,22 @@ class DecodeGraph:
             n_tokens=B, n_seqs=B, tokens=self.ints[0:B], positions=self.ints[B:2 * B],
             seq_of_token=self.want_rows, cu_seqlens=ar, slots=self.ints[2 * B:3 * B],
             ctx_lens=self.ints[3 * B:4 * B], host_slots=[-1] * B, host_new=[1] * B, host_start=[0] * B,
-            is_decode=True, max_new=1, max_ctx=engine.cache.max_seq_len,
-            max_ctx_bound=engine.cache.max_seq_len, ws=self.ws)
-        model, cache = engine.model, engine.cache
+            is_decode=True, max_new=1, max_ctx=cache.max_seq_len,
+            max_ctx_bound=cache.max_seq_len, ws=self.ws)
         # once eagerly with padding only: loads the kernels, sizes the workspace, stores nothing
         model.forward(self.step, cache, self.want_rows, B)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits = model.forward(self.step, cache, self.want_rows, B)
+        # no garbage collection while the stream is capturing: a collected tensor or graph
+        # would call into the runtime in the middle of the capture
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = model.forward(self.step, cache, self.want_rows, B)
+        finally:
+            if gc_was_on:
+                gc.enable()
         torch.cuda.synchronize(dev)
 
     def run(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int]) -> torch.Tensor:
@@ -64,8 +77,8 @@ class DecodeGraph:
 class DecodeGraphs:
     """The graphs of one engine, by batch size bucket."""
 
-    def __init__(self, engine, max_batch: int = 256):
-        self.engine = engine
+    def __init__(self, model, cache, device, max_batch: int = 256):
+        self.model, self.cache, self.device = model, cache, device
         self.max_batch = max_batch
         self.graphs: Dict[int, DecodeGraph] = {}
 
@@ -73,5 +86,5 @@ class DecodeGraphs:
         b = bucket_of(len(slots))
         g = self.graphs.get(b)
         if g is None:
-            g = self.graphs[b] = DecodeGraph(self.engine, b)
+            g = self.graphs[b] = DecodeGraph(self.model, self.cache, self.device, b)
         return g.run(slots, tokens, starts)

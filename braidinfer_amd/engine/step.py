@@ -9,6 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 
@@ -64,27 +65,21 @@ def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts
     B = len(slots) + pad_seqs
     new = [len(t) for t in token_lists] + [1] * pad_seqs
     T = sum(new)
-    flat: List[int] = []
-    # layout of the one int32 staging array: tokens | positions | seq_of_token | cu | slots | ctx
-    toks: List[int] = []
-    pos: List[int] = []
-    sot: List[int] = []
-    cu = [0]
-    ctx: List[int] = []
     all_slots = list(slots) + [-1] * pad_seqs
     all_starts = list(starts) + [0] * pad_seqs
-    for b in range(B):
-        tl = token_lists[b] if b < len(token_lists) else [0]
-        st = all_starts[b]
-        toks.extend(tl)
-        pos.extend(range(st, st + len(tl)))
-        sot.extend([b] * len(tl))
-        cu.append(cu[-1] + len(tl))
-        ctx.append(st + len(tl) if all_slots[b] >= 0 else 0)
-    flat = toks + pos + sot + cu + all_slots + ctx
-    host = torch.tensor(flat, dtype=torch.int32)
-    dev = host.to(device)
+    new_a = np.asarray(new, dtype=np.int64)
+    starts_a = np.asarray(all_starts, dtype=np.int64)
+    cu = np.zeros(B + 1, dtype=np.int64)
+    np.cumsum(new_a, out=cu[1:])
+    sot = np.repeat(np.arange(B, dtype=np.int64), new_a)
+    pos = np.arange(T, dtype=np.int64) - cu[sot] + starts_a[sot]
+    toks = np.concatenate([np.asarray(t, dtype=np.int64) for t in token_lists] + [np.zeros(pad_seqs, dtype=np.int64)])
+    ctx = np.where(np.asarray(all_slots) >= 0, starts_a + new_a, 0)
+    # layout of the one int32 staging array: tokens | positions | seq_of_token | cu | slots | ctx
+    flat = np.concatenate([toks, pos, sot, cu, np.asarray(all_slots, dtype=np.int64), ctx]).astype(np.int32)
+    dev = torch.from_numpy(flat).to(device)
     o = 0
+
     def take(n):
         nonlocal o
         v = dev[o:o + n]
@@ -92,8 +87,9 @@ def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts
         return v
     tokens, positions, seq_of_token = take(T), take(T), take(T)
     cu_seqlens, slots_d, ctx_d = take(B + 1), take(B), take(B)
+    max_ctx = int(ctx.max()) if B else 0
     return StepBatch(
         n_tokens=T, n_seqs=B, tokens=tokens, positions=positions, seq_of_token=seq_of_token,
         cu_seqlens=cu_seqlens, slots=slots_d, ctx_lens=ctx_d, host_slots=all_slots, host_new=new,
         host_start=all_starts, is_decode=all(n == 1 for n in new), max_new=max(new) if new else 0,
-        max_ctx=max(ctx) if ctx else 0, max_ctx_bound=max(ctx) if ctx else 0, ws=ws)
+        max_ctx=max_ctx, max_ctx_bound=max_ctx, ws=ws)

@@ -246,3 +246,32 @@ def test_graph_replays_equal_eager_steps(tiny_folders, dtype):
             stop(i)
         if not pos:
             break
+
+
+@pytest.mark.parametrize("which", ["all", "some"])
+def test_tensors_stored_in_32_bit_stay_so_in_the_bfloat16_engine(tmp_path, which):
+    """A matrix stored as F32 is multiplied in 32-bit even when the engine runs in bfloat16
+    (its activations are widened for it); bf16 and F32 matrices may meet in one model."""
+    import torch
+    from braidinfer_amd.weights import SafetensorsFolder, write_safetensors
+    cfg = B.MistralConfig.from_dict(dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4,
+                                         num_key_value_heads=2, head_dim=16, intermediate_size=96, vocab_size=120,
+                                         max_position_embeddings=512))
+    folder = B.Engine.write_random_folder(str(tmp_path / "m"), cfg, seed=3, std=0.1, vector_jitter=0.2)
+    st = SafetensorsFolder(folder)
+    wide = (lambda n: True) if which == "all" else (lambda n: n in ("lm_head.weight", "model.layers.0.self_attn.q_proj.weight",
+                                                                    "model.layers.1.mlp.up_proj.weight", "model.norm.weight"))
+    write_safetensors(f"{folder}/model.safetensors",
+                      [(n, st.tensor(n).float() if wide(n) else st.tensor(n).clone()) for n in st.names()])
+    pc, pw = P.read_folder(folder)
+    eng = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=512)
+    assert eng.model.lm_head.weight.dtype == torch.float32
+    assert eng.model.layers[1].feed_forward.w_d.dtype == (torch.float32 if which == "all" else torch.bfloat16)
+    toks = tokens(pc, 70, 3)
+    ref = P.forward(pc, pw, toks)
+    s = eng.alloc_slot()
+    got = [eng.step([StepEntry(s, toks[:50], list(range(50)))]).cpu().numpy()]
+    for t in toks[50:]:
+        got.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    eng.free_slot(s)
+    close(np.concatenate(got), ref, "bfloat16", f"32-bit tensors ({which})")
