@@ -363,6 +363,119 @@ static int launch_skinny(const bf16* A, const bf16* W, void* C, int M, int N, in
     return br_check_launch();
 }
 
+// ------------------------------------------------------------- gemm_skinny_lds ------
+// 16 < M <= 64: the activations of a 512-wide k-slab are staged in LDS once per workgroup
+// with direct global-to-LDS loads (one 1 KB row per wave-load, no registers), because at
+// these M the activation fragments, not the weights, dominate the load instructions.
+// A row's 16-byte columns are stored XOR-swizzled by the row number, so that the 16 rows
+// an operand read touches fall into different banks; the swizzle is applied by choosing
+// which global column each lane fetches.  Weights stream from memory into the operands
+// as in gemm_skinny; the 4 waves split the slab's k and are added in wave order.
+#define SLAB_K 512
+template <int MB, int RB, int MODE>
+__global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                              void* __restrict__ C, int M, int N, int K,
+                                                              size_t lda, size_t ldc) {
+    constexpr int ROWS = 16 * RB, COLS = 16 * MB;
+    constexpr int SLAB_BYTES = COLS * SLAB_K * 2;
+    constexpr int RED_BYTES = 4 * ROWS * (COLS + 1) * 4;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[SLAB_BYTES > RED_BYTES ? SLAB_BYTES : RED_BYTES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+    f32x4 acc[RB][MB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+    const bf16* wp[RB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+        int row = n0 + i * 16 + r16;
+        if (row > N - 1) row = N - 1;
+        wp[i] = W + (size_t)row * K + wave * 128 + g * 8;
+    }
+    const int nslab = (K + SLAB_K - 1) / SLAB_K;
+    for (int sl = 0; sl < nslab; ++sl) {
+        const int k0 = sl * SLAB_K;
+        bf16x8 fw[RB][4];                                  // this wave's weight fragments of the slab
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int k = k0 + wave * 128 + s * 32 + g * 8;
+                fw[i][s] = (k + 8 <= K) ? *(const bf16x8*)(wp[i] + k0 + s * 32) : zero8();
+            }
+#pragma unroll
+        for (int rr = 0; rr < COLS / 4; ++rr) {
+            const int row = rr * 4 + wave;                 // slab row = batch row; lane l fetches column l ^ (row & 15)
+            int grow = row;
+            if (grow > M - 1) grow = M - 1;
+            int kk = k0 + ((lane ^ (row & 15)) * 8);
+            if (kk + 8 > K) kk = 0;                        // never multiplied: the weight fragment there is zero
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(A + (size_t)grow * lda + kk),
+                                             (__attribute__((address_space(3))) void*)(smem + row * 1024), 16, 0, 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int c = wave * 16 + s * 4 + g;
+#pragma unroll
+            for (int j = 0; j < MB; ++j) {
+                const bf16x8 fx = *(const bf16x8*)(smem + (j * 16 + r16) * 1024 + ((c ^ r16) * 16));
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i][s], fx, acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    float (*red)[ROWS][COLS + 1] = (float (*)[ROWS][COLS + 1])smem;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * g + r][j * 16 + r16] = acc[i][j][r];
+    __syncthreads();
+    if (MODE == OUT_SWIGLU) {
+        for (int e = tid; e < (ROWS / 2) * COLS; e += 256) {
+            const int m = e / (ROWS / 2), jl = e - m * (ROWS / 2);
+            const int gl = (jl >> 3) * 16 + (jl & 7);
+            if (m < M && n0 + gl + 8 < N) {
+                float gv = 0.f, uv = 0.f;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) { gv += red[w][gl][m]; uv += red[w][gl + 8][m]; }
+                ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
+            }
+        }
+        return;
+    }
+    for (int e = tid; e < ROWS * COLS; e += 256) {
+        const int m = e / ROWS, nl = e - m * ROWS;
+        const int n = n0 + nl;
+        if (m < M && n < N) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) v += red[w][nl][m];
+            store_out<MODE>(C, (size_t)m * ldc + n, v);
+        }
+    }
+}
+
+template <int MB, int RB>
+static int launch_skinny_lds(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                             int mode, hipStream_t s) {
+    const unsigned grid = (unsigned)((N + 16 * RB - 1) / (16 * RB));
+    if (mode == OUT_BF16) gemm_skinny_lds_kernel<MB, RB, OUT_BF16><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else if (mode == OUT_F32) gemm_skinny_lds_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else if (mode == OUT_F32_ACC) gemm_skinny_lds_kernel<MB, RB, OUT_F32_ACC><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    else gemm_skinny_lds_kernel<MB, RB, OUT_SWIGLU><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    return br_check_launch();
+}
+
 // kernel: 0 = choose, 1 = tile 128x128, 2 = tile 256x128, 3 = skinny (tests force one)
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
                                size_t ldc, int mode, int kernel, hipStream_t s) {
@@ -379,10 +492,11 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
         const bool wide = N >= 16384;
         if (M <= 16) return (wide && M > 4) ? launch_skinny<1, 1, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s)
                                             : launch_skinny<1, 1, 4, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
-        if (M <= 32) return wide ? launch_skinny<2, 4, 1, 4>(A, W, C, M, N, K, lda, ldc, mode, s)
-                                 : launch_skinny<2, 2, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
-        return wide ? launch_skinny<4, 4, 1, 4>(A, W, C, M, N, K, lda, ldc, mode, s)
-                    : launch_skinny<4, 2, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
+        if (M <= 32) return wide ? launch_skinny_lds<2, 4>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                 : launch_skinny_lds<2, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
+        if (wide) return launch_skinny_lds<4, 4>(A, W, C, M, N, K, lda, ldc, mode, s);
+        return (N >= 6144) ? launch_skinny_lds<4, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
+                           : launch_skinny_lds<4, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
     }
     if (kernel == 2) return launch_tile<256, 128, 32, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, aligned, s);
     return launch_tile<128, 128, 64, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, aligned, s);
