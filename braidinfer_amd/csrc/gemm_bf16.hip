@@ -57,6 +57,43 @@ __device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, size_t ld
     return v;
 }
 
+// Store a wave's TM x TN grid of 32x32 accumulator blocks whose first element is (m1, n1).
+// acc[i][j][r]: row = 8 (r / 4) + 4 (lane / 32) + r % 4, column = lane % 32 of the block.
+template <int TM, int TN, int MODE>
+__device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[TM][TN], void* __restrict__ C, int M, int N, size_t ldc,
+                                              int m1, int n1, int lane) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n1 + j * 32 + (lane & 31);
+            if (MODE == OUT_SWIGLU) {
+                // the up value of a gate column sits 8 columns on, in lane ^ 8
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float other = __shfl_xor(acc[i][j][r], 8, 64);
+                    const int m = m1 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if ((lane & 8) == 0 && n < N && m < M)
+                        ((bf16*)C)[(size_t)m * ldc + (n >> 4) * 8 + (n & 7)] = (bf16)silu_mul(acc[i][j][r], other);
+                }
+                continue;
+            }
+            if (n >= N) continue;
+            // one 64-bit address per block; the 16 rows of a lane are reached by 32-bit offsets
+            const int mb = m1 + i * 32 + 4 * (lane >> 5);
+            const size_t base = (size_t)mb * ldc + n;
+            const unsigned ld32 = (unsigned)ldc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int dm = 8 * (r >> 2) + (r & 3);
+                if (mb + dm < M) store_out<MODE>(C, base + (size_t)(dm * ld32), acc[i][j][r]);
+            }
+            // keep the blocks' stores apart: moving every accumulator out of the matrix-core
+            // registers at once would not fit the register file of the large tiles
+            __builtin_amdgcn_sched_barrier(0);
+        }
+}
+
 // ------------------------------------------------------------------ gemm_tile -------
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int MODE, bool ALIGNED, bool KFULL>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
@@ -171,30 +208,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
         __syncthreads();
     }
 
-    // acc[i][j][r]: row = 8 (r / 4) + 4 (lane / 32) + r % 4, column = lane % 32 of the block
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + wn + j * 32 + (lane & 31);
-            if (MODE == OUT_SWIGLU) {
-                // the up value of a gate column sits 8 columns on, in lane ^ 8
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float other = __shfl_xor(acc[i][j][r], 8, 64);
-                    const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if ((lane & 8) == 0 && n < N && m < M)
-                        ((bf16*)C)[(size_t)m * ldc + (n >> 4) * 8 + (n & 7)] = (bf16)silu_mul(acc[i][j][r], other);
-                }
-                continue;
-            }
-            if (n >= N) continue;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M) store_out<MODE>(C, (size_t)m * ldc + n, acc[i][j][r]);
-            }
-        }
+    tile_epilogue<TM, TN, MODE>(acc, C, M, N, ldc, m0 + wm, n0 + wn, lane);
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
@@ -229,6 +243,175 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
     else BR_LAUNCH_TILE(OUT_SWIGLU);
 #undef BR_LAUNCH_TILE_
 #undef BR_LAUNCH_TILE
+    return br_check_launch();
+}
+
+// -------------------------------------------------------------- gemm_tile_dma -------
+// The tile product for aligned shapes (K a multiple of 64, 16-byte aligned rows): tiles
+// go from memory to LDS by direct global-to-LDS loads (global_load_lds_dwordx4: a wave
+// writes 1 KB = 8 tile rows of 64 k, no registers, no ds_write), into a ring of S stages.
+// A row's eight 16-byte columns are stored XOR-swizzled by (row / 2) % 8, which makes the
+// operand reads of 16 consecutive rows conflict-free; the swizzle is applied by choosing
+// the global column each lane fetches.  Rows beyond M or N are fetched from the last
+// valid row and dropped at the store.
+//
+// The loads are issued from inline assembly and counted by hand: before a stage is
+// read, `s_waitcnt vmcnt(n)` leaves only the younger stages' loads outstanding, then a
+// barrier makes every wave's part of the stage visible (and says that the stage about to
+// be overwritten has been read by all).  The kernel issues no other vector memory
+// operation inside the loop, so the count is exact.
+#define DMA_BK 64
+#define DMA_ISSUE(ST, kt)                                                                                      \
+    do {                                                                                                       \
+        _Pragma("unroll") for (int q = 0; q < INSTR; ++q) {                                                    \
+            const unsigned lds_ = __builtin_amdgcn_readfirstlane(                                              \
+                (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)(ST)) + dst[q]);          \
+            const bf16* gp_ = src[q] + (size_t)(kt) * DMA_BK;                                                  \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) \
+                         : "m0");                                                                              \
+        }                                                                                                      \
+    } while (0)
+#define DMA_COMPUTE(ST)                                                                                        \
+    do {                                                                                                       \
+        _Pragma("unroll") for (int kk = 0; kk < 4; ++kk) {                                                     \
+            bf16x8 fa[TM], fb[TN];                                                                             \
+            const int c = kk * 2 + g;                                                                          \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                                   \
+                const int r = wm + i * 32 + lrow;                                                              \
+                fa[i] = *(const bf16x8*)((ST) + r * 128 + ((c ^ ((r >> 1) & 7)) * 16));                        \
+            }                                                                                                  \
+            _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                                   \
+                const int r = BM + wn + j * 32 + lrow;                                                         \
+                fb[j] = *(const bf16x8*)((ST) + r * 128 + ((c ^ ((r >> 1) & 7)) * 16));                        \
+            }                                                                                                  \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                     \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                 \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);     \
+        }                                                                                                      \
+    } while (0)
+#define DMA_WAITBAR(N)                                              \
+    do {                                                            \
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");    \
+        __builtin_amdgcn_s_barrier();                               \
+        asm volatile("" ::: "memory");                              \
+    } while (0)
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int S, int MODE>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
+    const bf16* __restrict__ A, const bf16* __restrict__ W, void* __restrict__ C, int M, int N, int K, size_t lda,
+    size_t ldc, int tiles_m, int tiles_n) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+    constexpr int STAGE_BYTES = (BM + BN) * DMA_BK * 2;
+    constexpr int INSTR = (BM + BN) / 8 / NW;           // 1 KB wave-loads per wave and stage
+    static_assert(S == 2 || S == 3, "2 or 3 stages");
+    __shared__ __attribute__((aligned(1024))) unsigned char st0[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char st1[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char st2[S >= 3 ? STAGE_BYTES : 16];
+
+    // each XCD takes a contiguous run of tiles, in groups of 8 tile columns by all tile rows
+    const int total = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = total / 8, xcd = pid % 8, idx = pid / 8;
+        if (pid < per * 8) pid = xcd * per + idx;
+    }
+    const int grp = pid / (8 * tiles_m), in = pid - grp * 8 * tiles_m;
+    int gn = tiles_n - grp * 8;
+    if (gn > 8) gn = 8;
+    const int tile_n = grp * 8 + in % gn, tile_m = in / gn;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
+    const int lrow = lane & 31, g = lane >> 5;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // wave-load q of this wave covers rows (q NW + wave) 8 .. + 8 of the stacked tile [A rows | W rows]
+    const bf16* src[INSTR];
+    int dst[INSTR];
+#pragma unroll
+    for (int q = 0; q < INSTR; ++q) {
+        const int R = (q * NW + wave) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ ((R >> 1) & 7);       // the global 16-byte column this lane fetches
+        if (R < BM) {
+            int r = m0 + R;
+            if (r > M - 1) r = M - 1;
+            src[q] = A + (size_t)r * lda + c * 8;
+        } else {
+            int r = n0 + R - BM;
+            if (r > N - 1) r = N - 1;
+            src[q] = W + (size_t)r * K + c * 8;
+        }
+        dst[q] = (q * NW + wave) * 1024;
+    }
+    const int nk = K / DMA_BK;
+    if (S == 2) {
+        DMA_ISSUE(st0, 0);
+        for (int kt = 0; kt < nk; kt += 2) {
+            DMA_WAITBAR(0);
+            if (kt + 1 < nk) DMA_ISSUE(st1, kt + 1);
+            DMA_COMPUTE(st0);
+            if (kt + 1 >= nk) break;
+            DMA_WAITBAR(0);
+            if (kt + 2 < nk) DMA_ISSUE(st0, kt + 2);
+            DMA_COMPUTE(st1);
+        }
+    } else {
+        DMA_ISSUE(st0, 0);
+        if (nk > 1) DMA_ISSUE(st1, 1);
+        int kt = 0;
+        // steady state: two stages are in flight at every wait, the older one is waited for
+        for (; kt + 5 <= nk; kt += 3) {
+            DMA_WAITBAR(INSTR);
+            DMA_ISSUE(st2, kt + 2);
+            DMA_COMPUTE(st0);
+            DMA_WAITBAR(INSTR);
+            DMA_ISSUE(st0, kt + 3);
+            DMA_COMPUTE(st1);
+            DMA_WAITBAR(INSTR);
+            DMA_ISSUE(st1, kt + 4);
+            DMA_COMPUTE(st2);
+        }
+        // the last tiles: wait for everything in flight
+        for (; kt < nk; kt += 3) {
+            DMA_WAITBAR(0);
+            if (kt + 2 < nk) DMA_ISSUE(st2, kt + 2);
+            DMA_COMPUTE(st0);
+            if (kt + 1 >= nk) break;
+            DMA_WAITBAR(0);
+            if (kt + 3 < nk) DMA_ISSUE(st0, kt + 3);
+            DMA_COMPUTE(st1);
+            if (kt + 2 >= nk) break;
+            DMA_WAITBAR(0);
+            if (kt + 4 < nk) DMA_ISSUE(st1, kt + 4);
+            DMA_COMPUTE(st2);
+        }
+    }
+    tile_epilogue<TM, TN, MODE>(acc, C, M, N, ldc, m0 + wm, n0 + wn, lane);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int S>
+static int launch_tile_dma(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                           int mode, hipStream_t s) {
+    const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    const long long total = (long long)tm * tn;
+    if (total > 0x7fffffffLL) return BR_BAD_ARG;
+    constexpr int NT = 64 * WAVES_M * WAVES_N;
+    if (mode == OUT_BF16)
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_BF16><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+    else if (mode == OUT_F32)
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+    else if (mode == OUT_F32_ACC)
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32_ACC><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+    else
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_SWIGLU><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
     return br_check_launch();
 }
 
@@ -476,7 +659,10 @@ static int launch_skinny_lds(const bf16* A, const bf16* W, void* C, int M, int N
     return br_check_launch();
 }
 
-// kernel: 0 = choose, 1 = tile 128x128, 2 = tile 256x128, 3 = skinny (tests force one)
+// kernel: 0 = choose, 1 = tile 128x128 through registers (any shape), 2 = the same 256x128,
+// 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
+// of 64, aligned rows); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
+// of registers in three of the four epilogues and was no faster in the fourth.)
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
                                size_t ldc, int mode, int kernel, hipStream_t s) {
     if (M <= 0 || N <= 0) return BR_OK;
@@ -486,7 +672,12 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     const bf16* W = (const bf16*)W_;
     const bool aligned = (K % 8 == 0) && (lda % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     if (kernel == 3 && (!aligned || M > 64)) return BR_BAD_ARG;
-    if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : 1;
+    const bool dma_ok = aligned && K % DMA_BK == 0;
+    if (kernel >= 4 && (!dma_ok || kernel > 6)) return BR_BAD_ARG;
+    if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
+    if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
+    if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
+    if (kernel == 6) return launch_tile_dma<128, 128, 2, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s);
     if (kernel == 3) {
         // shapes measured on cold weights (cycled through more than the 256 MB cache)
         const bool wide = N >= 16384;

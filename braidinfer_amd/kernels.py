@@ -172,8 +172,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     matrix-core kernels with float accumulation; out is bfloat16, or float32 (and may
     then accumulate, which is how a projection adds into the residual stream).
     Rows of `a` and `out` may be strided (a view of a wider buffer); w is contiguous.
-    `kernel` forces one bf16 kernel (1: 128x128 tiles, 2: 256x128 tiles, 3: skinny, for
-    M <= 64); 0 chooses by shape.
+    `kernel` forces one bf16 kernel (1, 2: 128x128 and 256x128 tiles staged through
+    registers, any shape; 3: skinny, M <= 64; 4, 5, 6: 256x128, 128x256 and 128x128 tiles
+    loaded straight into LDS, K in steps of 64); 0 chooses by shape.
     """
     name = "gemm"
     for t in (a, w, out):

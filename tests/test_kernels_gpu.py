@@ -63,7 +63,15 @@ def test_rmsnorm_reference_vector():
 
 # ----------------------------------------------------------------------- GEMM ------
 SHAPES = [(1, 64, 64), (5, 100, 96), (17, 192, 320), (64, 301, 100), (33, 1000, 264), (3, 50, 44),
-          (130, 514, 100), (257, 129, 72), (300, 260, 1032)]
+          (130, 514, 100), (257, 129, 72), (300, 260, 1032), (130, 514, 128), (257, 129, 192), (300, 700, 1024),
+          (65, 301, 64), (513, 260, 320)]
+
+
+def _skip_unless_kernel_takes(kernel, M, Kd):
+    if kernel == 3 and (Kd % 8 or M > 64):
+        pytest.skip("the skinny kernels take M <= 64 and K in steps of 8")
+    if kernel >= 4 and Kd % 64:
+        pytest.skip("the direct-to-LDS tile kernels take K in steps of 64")
 
 
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
@@ -88,11 +96,10 @@ def test_gemm_f32_rows_do_not_depend_on_the_batch():
     assert torch.equal(one[0], full[33])
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
 def test_gemm_bf16(M, N, Kd, kernel):
-    if kernel == 3 and (Kd % 8 or M > 64):
-        pytest.skip("the skinny kernel takes M <= 64 and K in steps of 8")
+    _skip_unless_kernel_takes(kernel, M, Kd)
     a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
     want = a.double() @ w.double().T
     o32 = torch.empty(M, N, device=DEV)
@@ -392,11 +399,11 @@ def test_attention_kernels_refuse_what_they_do_not_take():
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3])
-@pytest.mark.parametrize("M,I,Kd", [(1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032)])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("M,I,Kd", [(1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
+                                    (300, 512, 1024), (129, 200, 192)])
 def test_gemm_with_swiglu_epilogue(M, I, Kd, kernel):
-    if kernel == 3 and (Kd % 8 or M > 64):
-        pytest.skip("the skinny kernel takes M <= 64 and K in steps of 8")
+    _skip_unless_kernel_takes(kernel, M, Kd)
     a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
     wg, wu = rnd(I, Kd, seed=2, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=3, scale=0.3, dtype=torch.bfloat16)
     out = torch.empty(M, I, device=DEV, dtype=torch.bfloat16)
