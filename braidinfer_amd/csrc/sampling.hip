@@ -105,6 +105,39 @@ extern "C" int br_sample_prepare(const float* logits, float* work, int B, int V,
     return br_check_launch();
 }
 
+// The first index i in [0, n) at which the running sum of f(0..i) reaches `target` (as
+// `target <= sum`), or n.  Sums run in index order, blockDim.x at a time: a scan inside
+// each wave, then the waves' totals in wave order.  Every thread of the block calls it;
+// `wsum` holds one float per wave, `found` one int.
+template <typename F>
+__device__ __forceinline__ int block_first_reach(int n, float target, F f, float* wsum, int* found) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    if (threadIdx.x == 0) *found = 0x7fffffff;
+    float base = 0.f;
+    for (int i0 = 0; i0 < n; i0 += blockDim.x) {
+        const int i = i0 + threadIdx.x;
+        const float p = i < n ? f(i) : 0.f;
+        float sc = p;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+        __syncthreads();
+        if (lane == 63) wsum[wv] = sc;
+        __syncthreads();
+        float before = base;
+        for (int x = 0; x < wv; ++x) before += wsum[x];
+        if (i < n && target <= before + sc) atomicMin(found, i);
+        float tot = base;
+        for (int x = 0; x < nw; ++x) tot += wsum[x];
+        base = tot;
+        __syncthreads();
+        if (*found != 0x7fffffff) break;
+    }
+    __syncthreads();
+    const int r = *found;
+    __syncthreads();
+    return r == 0x7fffffff ? n : r;
+}
+
 // ------------------------------------------------- top-k / min-p / top-p filter ----
 // Masks entries of work[b, :] to -inf as sampling.rs:89-151 does.  The row is sorted
 // once, descending by value with the lower index first among equals, as 64-bit keys
@@ -118,6 +151,7 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_kernel(
     const int* __restrict__ top_k, const float* __restrict__ min_p, const float* __restrict__ top_p,
     const float* __restrict__ temperature) {
     __shared__ float red[16];
+    __shared__ float wsum[FBLOCK / 64];
     __shared__ int keep_s;
     const int b = blockIdx.x;
     const int k = top_k[b]; const float mp = min_p[b], tp = top_p[b];
@@ -160,18 +194,14 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_kernel(
             if (v > -INFINITY) part += expf(v - vmax);
         }
         const float sum = block_sum(part, red);
-        if (threadIdx.x == 0) {
-            float cum = 0.f; int cut = keep;
-            for (int i = 0; i < keep; ++i) {
-                float v = key2f((uint32_t)(ks[i] >> 32));
-                if (!(v > -INFINITY)) { cut = i; break; }
-                cum += expf(v - vmax) / sum;
-                if (cum >= tp) { cut = i + 1; break; }
-            }
-            keep_s = cut;
-        }
-        __syncthreads();
-        keep = keep_s;
+        // survivors with a finite value are a prefix too (masked entries sort last)
+        float fin = 0.f;
+        for (int i = threadIdx.x; i < keep; i += FBLOCK)
+            if (key2f((uint32_t)(ks[i] >> 32)) > -INFINITY) fin += 1.f;
+        const int nfin = (int)(block_sum(fin, red) + 0.5f);
+        const int hit = block_first_reach(nfin, tp, [&](int i) {
+            return expf(key2f((uint32_t)(ks[i] >> 32)) - vmax) / sum; }, wsum, &keep_s);
+        keep = hit < nfin ? hit + 1 : nfin;
     }
     for (int i = keep + threadIdx.x; i < V; i += FBLOCK) w[~(uint32_t)(ks[i] & 0xffffffffu)] = -INFINITY;
 }
@@ -208,7 +238,6 @@ __global__ __launch_bounds__(SBLOCK) void sample_draw_kernel(const float* __rest
         argmax_combine(bv, bi, ov, oi);
     }
     if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
-    if (threadIdx.x == 0) found = 0x7fffffff;
     __syncthreads();
     for (int ww = 0; ww < SBLOCK / 64; ++ww) argmax_combine(bv, bi, sv[ww], si[ww]);
     if (bi == 0x7fffffff) bi = 0;
@@ -217,31 +246,8 @@ __global__ __launch_bounds__(SBLOCK) void sample_draw_kernel(const float* __rest
     float part = 0.f;
     for (int i = threadIdx.x; i < V; i += SBLOCK) part += expf(w[i] - vmax);
     const float sum = block_sum(part, red);
-    const float target = u[b];
-    float base = 0.f;   // cumulative probability before this chunk
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    for (int i0 = 0; i0 < V; i0 += SBLOCK) {
-        const int i = i0 + threadIdx.x;
-        const float p = i < V ? expf(w[i] - vmax) / sum : 0.f;
-        // inclusive scan inside the wave, then across the waves
-        float sc = p;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
-        __syncthreads();
-        if (lane == 63) wsum[wv] = sc;
-        __syncthreads();
-        float before = base;
-        for (int x = 0; x < wv; ++x) before += wsum[x];
-        const float cum = before + sc;
-        // the first index with u <= cum: every later index satisfies it too, take the minimum
-        if (i < V && target <= cum) atomicMin(&found, i);
-        float tot = base;
-        for (int x = 0; x < SBLOCK / 64; ++x) tot += wsum[x];
-        base = tot;
-        __syncthreads();
-        if (found != 0x7fffffff) break;
-    }
-    if (threadIdx.x == 0) out[b] = found != 0x7fffffff ? found : bi;
+    const int hit = block_first_reach(V, u[b], [&](int i) { return expf(w[i] - vmax) / sum; }, wsum, &found);
+    if (threadIdx.x == 0) out[b] = hit < V ? hit : bi;
 }
 
 extern "C" int br_sample_draw(const float* work, int* out, int B, int V, const float* temperature,

@@ -154,14 +154,13 @@ def test_wanted_places_and_chunked_prompts(engines, tiny_folders, dtype):
     eng.free_slot(a); eng.free_slot(b)
 
 
-def test_a_far_key_among_hundreds_is_found(tmp_path):
-    """Random weights give near-uniform attention, which would hide a lost key.  Here the
-    weights are made so that the last token's query matches one early key far more than
-    any other: one head copies that token's value, and its identity shows in the logits."""
+def _marker_model(tmp_path, sliding_window=None):
+    """A one-layer model in which token 2 (the asker) attends almost only to token 1 (the
+    marker), wherever it sits, and copies its content into the logits."""
     cfg = B.MistralConfig.from_dict(dict(num_hidden_layers=1, hidden_size=32, num_attention_heads=2,
                                          num_key_value_heads=1, head_dim=16, intermediate_size=16,
                                          vocab_size=40, rope_theta=10000.0, rms_norm_eps=1e-5,
-                                         max_position_embeddings=4096))
+                                         max_position_embeddings=4096, sliding_window=sliding_window))
     folder = B.Engine.write_random_folder(str(tmp_path / "m"), cfg, seed=1, std=0.02)
     from braidinfer_amd.weights import SafetensorsFolder, write_safetensors
     st = SafetensorsFolder(folder)
@@ -187,6 +186,14 @@ def test_a_far_key_among_hundreds_is_found(tmp_path):
     t["lm_head.weight"] = head.bfloat16()
     write_safetensors(f"{folder}/model.safetensors", t.items())
     pc, pw = P.read_folder(folder)
+    return folder, pc, pw
+
+
+def test_a_far_key_among_hundreds_is_found(tmp_path):
+    """Random weights give near-uniform attention, which would hide a lost key.  Here the
+    weights are made so that the last token's query matches one early key far more than
+    any other: one head copies that token's value, and its identity shows in the logits."""
+    folder, pc, pw = _marker_model(tmp_path)
     rng = np.random.default_rng(0)
     for dtype in ("float32", "bfloat16"):
         eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=1024)
@@ -275,3 +282,27 @@ def test_tensors_stored_in_32_bit_stay_so_in_the_bfloat16_engine(tmp_path, which
         got.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
     eng.free_slot(s)
     close(np.concatenate(got), ref, "bfloat16", f"32-bit tensors ({which})")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_windows_edge_is_exact(tmp_path, dtype):
+    """With a window of 100 the asker at position 499 sees position 400 and not 399.  The
+    marker on either side of that edge decides the logits, for the asker decoded alone, as
+    the end of a whole prompt, and as the end of a chunk."""
+    folder, pc, pw = _marker_model(tmp_path, sliding_window=100)
+    eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=1024)
+    rng = np.random.default_rng(1)
+    for at, seen in ((400, True), (399, False), (499 - 63, True), (401, True)):
+        toks = [int(x) for x in rng.integers(3, 40, 500)]
+        toks[at] = 1
+        toks[-1] = 2
+        ref = P.forward(pc, pw, toks)[-1]
+        assert (int(ref.argmax()) == 1) == seen, "the plain implementation must see the marker exactly inside the window"
+        for cut in (499, 0, 450):                    # asker alone; whole prompt; a last chunk of 50
+            s = eng.alloc_slot()
+            if cut:
+                eng.step([StepEntry(s, toks[:cut], [])])
+            got = eng.step([StepEntry(s, toks[cut:], [len(toks) - cut - 1])]).cpu().numpy()[0]
+            eng.free_slot(s)
+            assert (int(got.argmax()) == 1) == seen, f"marker at {at}, cut {cut}: window edge is off"
+            close(got[None], ref[None], dtype, f"window edge, marker at {at}, cut {cut}")
