@@ -58,6 +58,10 @@ class Engine:
         self.rt = rt
         self.device = rt.device
         self.ws = Workspace(rt.device)
+        if max_seq_len is None:
+            # the block tables are [slots, pages of the longest sequence]: bound the longest
+            # sequence by the model's positions (at least 32k) rather than by the whole cache
+            max_seq_len = min(max(int(max_tokens), 64), max(int(model.spec.max_position_embeddings), 32768))
         self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens=max_tokens,
                                    max_seq_len=max_seq_len, n_slots=n_slots, dtype=rt.dtype, device=rt.device)
         self.vocab_size = self.spec.vocab_size
