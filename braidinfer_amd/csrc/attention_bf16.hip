@@ -16,6 +16,11 @@
 #include "common.h"
 
 #define PAGE 64
+#define LOG2E 1.4426950408889634f
+
+// 2^x by the hardware's v_exp_f32 (2^-inf = 0).  The softmax of these kernels runs in
+// base 2: scores are scaled by scale * log2(e) once, and exp(s - m) becomes 2^(s' - m').
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
@@ -91,6 +96,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
+    const float scale2 = scale * LOG2E;
 
     const int* bt = block_table + (size_t)slot * table_stride;
     const size_t page_elems = (size_t)2 * nkv * PAGE * hd;
@@ -117,18 +123,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         for (int r = 0; r < 16; ++r) {
             const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
             const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
-            sv[r] = ok ? s_acc[r] * scale : -INFINITY;
+            sv[r] = ok ? s_acc[r] * scale2 : -INFINITY;
             mx = fmaxf(mx, sv[r]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = expf(m - m_use);
+        const float corr = fast_exp2(m - m_use);
         float psum = 0.f;
         bf16x8 p1, p2;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float p = expf(sv[r] - m_use);
+            const float p = fast_exp2(sv[r] - m_use);
             psum += p;
             if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
         }
@@ -226,6 +232,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
+    const float scale2 = scale * LOG2E;
 
     const int* bt = block_table + (size_t)slot * table_stride;
     const size_t page_elems = (size_t)2 * nkv * PAGE * hd;
@@ -295,31 +302,47 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
             }
             float sv[16];
             float mx = -INFINITY;
+            // a block every row of the wave sees whole (below the diagonal, inside the window)
+            // needs no mask
+            const bool whole = row0 + 31 < rows_total && kb + 31 <= pq_min_w &&
+                               (window <= 0 || kb > pq_max_w - window);
+            if (whole) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
-                const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
-                sv[r] = ok ? s_acc[r] * scale : -INFINITY;
-                mx = fmaxf(mx, sv[r]);
+                for (int r = 0; r < 16; ++r) { sv[r] = s_acc[r] * scale2; mx = fmaxf(mx, sv[r]); }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
+                    const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
+                    sv[r] = ok ? s_acc[r] * scale2 : -INFINITY;
+                    mx = fmaxf(mx, sv[r]);
+                }
             }
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m, mx);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float corr = expf(m - m_use);
+            // the accumulators are rescaled only when some row's maximum moved
+            const bool moved = __any(m_new > m);
+            if (moved) {
+                const float corr = fast_exp2(m - m_use);
+                lsum *= corr;
+#pragma unroll
+                for (int i = 0; i < NB; ++i)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
+            }
             float psum = 0.f;
             bf16x8 p1, p2;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float p = expf(sv[r] - m_use);
+                const float p = fast_exp2(sv[r] - m_use);
                 psum += p;
                 if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
             }
-            lsum = lsum * corr + psum;
+            lsum += psum;
             m = m_new;
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
                 const bf16* vrow = vs + (i * 32 + c) * VLD + kl + 4 * g;   // rows at or beyond hd hold zeros or stale
                 bf16x8 v1 = zero8(), v2 = zero8();
                 if (i * 32 + c < hd) {
@@ -393,6 +416,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc_o[i][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
+    const float scale2 = scale * LOG2E;
     const int* bt = block_table + (size_t)(slot < 0 ? 0 : slot) * table_stride;
     const size_t page_elems = (size_t)2 * nkv * PAGE * hd;
     const size_t k_off = (size_t)kvh * PAGE * hd, v_off = ((size_t)nkv + kvh) * PAGE * hd;
@@ -442,18 +466,18 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
             for (int e = 0; e < 8; ++e) {
                 const int key = kb + 16 * (e >> 2) + 4 * g + (e & 3);
                 const bool ok = key >= lo && key < ctx;
-                sv[e] = ok ? s_acc[e >> 2][e & 3] * scale : -INFINITY;
+                sv[e] = ok ? s_acc[e >> 2][e & 3] * scale2 : -INFINITY;
                 mx = fmaxf(mx, sv[e]);
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m, mx);           // finite: the block holds at least one visible key
-            const float corr = expf(m - m_new);
+            const float corr = fast_exp2(m - m_new);
             float psum = 0.f;
             bf16x8 pf;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = expf(sv[e] - m_new);
+                const float p = fast_exp2(sv[e] - m_new);
                 psum += p;
                 pf[e] = (bf16)p;
             }
@@ -490,7 +514,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         if (M > -INFINITY) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const float f = expf(lds[w * wstride + 16 * hd + h] - M);
+                const float f = fast_exp2(lds[w * wstride + 16 * hd + h] - M);
                 L += lds[w * wstride + 16 * hd + 16 + h] * f;
                 O += lds[w * wstride + h * hd + d] * f;
             }
@@ -516,11 +540,11 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(const float* __
     for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
     float L = 0.f;
     if (M > -INFINITY)
-        for (int s = 0; s < nsplit; ++s) L += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - M);
+        for (int s = 0; s < nsplit; ++s) L += part_ml[(base + s) * 2 + 1] * fast_exp2(part_ml[(base + s) * 2] - M);
     for (int d = threadIdx.x; d < hd; d += 64) {
         float O = 0.f;
         if (M > -INFINITY)
-            for (int s = 0; s < nsplit; ++s) O += part_o[(base + s) * hd + d] * expf(part_ml[(base + s) * 2] - M);
+            for (int s = 0; s < nsplit; ++s) O += part_o[(base + s) * hd + d] * fast_exp2(part_ml[(base + s) * 2] - M);
         out[((size_t)b * nq + head) * hd + d] = (bf16)(L > 0.f ? O / L : 0.f);
     }
 }
