@@ -29,6 +29,8 @@ def main() -> int:
     ap.add_argument("--preset", default="mistral-7b-v0.3")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prompt-min", type=int, default=128)
+    ap.add_argument("--prompt-max", type=int, default=2048)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
@@ -47,7 +49,7 @@ def main() -> int:
     layers = args.layers or full.num_hidden_layers
     cfg = B.preset(args.preset, num_hidden_layers=layers)
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
-    room = max(max(batches) * (-(-(2048 + args.steps + args.warmup + 1) // 64) * 64),
+    room = max(max(batches) * (-(-(args.prompt_max + args.steps + args.warmup + 1) // 64) * 64),
                -(-args.prefill_tokens // 64) * 64)
     t0 = time.time()
     eng = B.Engine.random(cfg, seed=0, dtype=args.dtype, max_tokens=room, max_seq_len=args.context)
@@ -83,7 +85,7 @@ def main() -> int:
 
     def decode(batch, steps, warmup, seed):
         rng = np.random.default_rng(seed)
-        lens = [int(n) for n in rng.integers(128, 2049, batch)]
+        lens = [int(n) for n in rng.integers(args.prompt_min, args.prompt_max + 1, batch)]
         prompts = [[int(t) for t in rng.integers(0, V, n)] for n in lens]
         slots = [eng.alloc_slot() for _ in range(batch)]
         # prompts in chunks of at most 16k tokens a step, to bound the activations
@@ -106,13 +108,17 @@ def main() -> int:
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()
-        ctx0 = sum(eng.length(s) for s in slots)
+        # keys a step has to read: the whole context, or the window where the model has one
+        W = cfg.sliding_window
+        seen = lambda n: n if W is None else min(n, W)
+        ctx0 = sum(seen(eng.length(s)) for s in slots)
+        ctx1 = sum(seen(eng.length(s) + steps) for s in slots)
         t = time.perf_counter()
         for _ in range(steps):
             one()
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t) / steps
-        mean_ctx_total = ctx0 + batch * (steps + 1) / 2.0
+        mean_ctx_total = (ctx0 + ctx1) / 2.0
         for s in slots:
             eng.free_slot(s)
         return dt, weight_bytes + mean_ctx_total * kv_bytes_per_token, float(np.mean(lens))
@@ -120,7 +126,8 @@ def main() -> int:
     dt, nbytes, mean_len = decode(args.batch, args.steps, args.warmup, seed=1)
     value = args.batch / dt
     line = {
-        "metric": "decode tok/s (batch 8, Mistral-7B-v0.3 shape, bf16, prompts uniform in [128, 2048])",
+        "metric": f"decode tok/s (batch {args.batch}, {args.preset} shape, {args.dtype}, prompts uniform in "
+                  f"[{args.prompt_min}, {args.prompt_max}])",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
@@ -128,7 +135,7 @@ def main() -> int:
                    "hidden": H, "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
                    "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
                    "sliding_window": cfg.sliding_window, "global_batch": args.batch, "seq_len": args.context,
-                   "prompt_lens": "uniform[128,2048]", "mean_prompt_len": round(mean_len, 1),
+                   "prompt_lens": f"uniform[{args.prompt_min},{args.prompt_max}]", "mean_prompt_len": round(mean_len, 1),
                    "weights": "random N(0,0.02) bf16", "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(nbytes / dt / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(nbytes / dt / PEAK_HBM, 4)},
