@@ -11,8 +11,9 @@
 // accumulator of the first product (a lane holds one query column and several keys) is,
 // after exp and rounding to bf16, exactly the B operand of the second, O^T = V^T P^T,
 // with V^T rows read as the A operand: no shuffle and no LDS between the two products.
-// The k-slots of the second product are a fixed permutation of the keys (a lane's slots
-// are the keys its accumulator registers hold); V^T is read with the same permutation.
+// For that, the rows of the first product are a fixed permutation of a block's keys, chosen
+// so that the accumulator registers of a lane hold 8 consecutive keys: then the k-slots of
+// the second product are in key order and V^T is read 16 contiguous bytes at a time.
 #include "common.h"
 
 #define PAGE 64
@@ -28,27 +29,18 @@ __device__ __forceinline__ bf16x8 zero8() {
     for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
     return z;
 }
-__device__ __forceinline__ bf16x8 join4(bf16x4 a, bf16x4 b) {
-    bf16x8 v;
+// 8 values V^T[dim][k .. k+7] of a page; keys at or beyond `limit` read as zero
+__device__ __forceinline__ bf16x8 load_vt8(const bf16* __restrict__ vrow, int k, int limit_local) {
+    bf16x8 v = *(const bf16x8*)(vrow + k);
+    if (k + 8 > limit_local) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
-    return v;
-}
-__device__ __forceinline__ bf16x4 zero4() {
-    bf16x4 z;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) z[i] = (bf16)0.f;
-    return z;
-}
-// 4 values V^T[dim][k .. k+3] of a page; keys at or beyond `limit` read as zero
-__device__ __forceinline__ bf16x4 load_vt4(const bf16* __restrict__ vrow, int k, int limit_local) {
-    bf16x4 v = *(const bf16x4*)(vrow + k);
-    if (k + 4 > limit_local) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) if (k + i >= limit_local) v[i] = (bf16)0.f;
+        for (int i = 0; i < 8; ++i) if (k + i >= limit_local) v[i] = (bf16)0.f;
     }
     return v;
 }
+// Row c (0..31) of a 32-key score block stands for this key of the block; lane (column, g)
+// then holds in acc[r] the key 16 (r / 8) + 8 g + r % 8.
+__device__ __forceinline__ int key_of_row32(int c) { return 16 * (c >> 4) + 8 * ((c >> 2) & 1) + 4 * ((c >> 3) & 1) + (c & 3); }
 
 // --------------------------------------------------------------------- prefill ------
 // grid = (row tiles of 128, nkv, sequences), block = 256.  A row is a (token, q head of
@@ -106,7 +98,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int kb = (lo / 32) * 32; kb <= pq_max; kb += 32) {
         const bf16* pg = cache + (size_t)bt[kb / PAGE] * page_elems;
         const int kl = kb % PAGE;                       // 0 or 32: the block's place in its page
-        const bf16* krow = pg + k_off + (size_t)(kl + c) * hd;
+        const bf16* krow = pg + k_off + (size_t)(kl + key_of_row32(c)) * hd;
         f32x16 s_acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
@@ -116,12 +108,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             const bf16x8 kf = (d < hd) ? *(const bf16x8*)(krow + d) : zero8();
             s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
         }
-        // s_acc[r]: key kb + 8 (r / 4) + 4 g + r % 4, query row = this lane's column
+        // s_acc[r]: key kb + 16 (r / 8) + 8 g + r % 8, query row = this lane's column
         float sv[16];
         float mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
+            const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
             const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
             sv[r] = ok ? s_acc[r] * scale2 : -INFINITY;
             mx = fmaxf(mx, sv[r]);
@@ -149,8 +141,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             bf16x8 v1 = zero8(), v2 = zero8();
             if (dim < hd) {
                 const bf16* vrow = pg + v_off + (size_t)dim * PAGE;
-                v1 = join4(load_vt4(vrow, kl + 4 * g, limit_local), load_vt4(vrow, kl + 8 + 4 * g, limit_local));
-                v2 = join4(load_vt4(vrow, kl + 16 + 4 * g, limit_local), load_vt4(vrow, kl + 24 + 4 * g, limit_local));
+                v1 = load_vt8(vrow, kl + 8 * g, limit_local);
+                v2 = load_vt8(vrow, kl + 16 + 8 * g, limit_local);
             }
             acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i], 0, 0, 0);
             acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i], 0, 0, 0);
@@ -290,7 +282,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
             const int kl = half * 32, kb = pi * PAGE + kl;
             // blocks no row of this wave can see are skipped
             if (!wave_ok || kb > pq_max_w || (window > 0 && kb + 31 <= pq_min_w - window)) continue;
-            const bf16* krow = ks + (kl + c) * kld;
+            const bf16* krow = ks + (kl + key_of_row32(c)) * kld;
             f32x16 s_acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
@@ -312,7 +304,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int key = kb + 8 * (r >> 2) + 4 * g + (r & 3);
+                    const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
                     const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
                     sv[r] = ok ? s_acc[r] * scale2 : -INFINITY;
                     mx = fmaxf(mx, sv[r]);
@@ -343,11 +335,11 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
             m = m_new;
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-                const bf16* vrow = vs + (i * 32 + c) * VLD + kl + 4 * g;   // rows at or beyond hd hold zeros or stale
+                const bf16* vrow = vs + (i * 32 + c) * VLD + kl + 8 * g;   // rows at or beyond hd are never filled
                 bf16x8 v1 = zero8(), v2 = zero8();
                 if (i * 32 + c < hd) {
-                    v1 = join4(*(const bf16x4*)(vrow), *(const bf16x4*)(vrow + 8));
-                    v2 = join4(*(const bf16x4*)(vrow + 16), *(const bf16x4*)(vrow + 24));
+                    v1 = *(const bf16x8*)(vrow);
+                    v2 = *(const bf16x8*)(vrow + 16);
                 }
                 acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i], 0, 0, 0);
                 acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i], 0, 0, 0);
@@ -434,7 +426,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
             bf16x8 kf[2][NB], vf[2 * NB];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const bf16* krow = pg + k_off + (size_t)(kl + 16 * j + c) * hd;
+                // row c of score block j stands for key 8 (c / 4) + 4 j + c % 4 of the 32
+                const bf16* krow = pg + k_off + (size_t)(kl + 8 * (c >> 2) + 4 * j + (c & 3)) * hd;
 #pragma unroll
                 for (int s = 0; s < NB; ++s) {
                     const int d = s * 32 + 8 * g;
@@ -447,7 +440,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
                 vf[i] = zero8();
                 if (dim < hd) {
                     const bf16* vrow = pg + v_off + (size_t)dim * PAGE;
-                    vf[i] = join4(load_vt4(vrow, kl + 4 * g, limit_local), load_vt4(vrow, kl + 16 + 4 * g, limit_local));
+                    vf[i] = load_vt8(vrow, kl + 8 * g, limit_local);
                 }
             }
             f32x4 s_acc[2];
@@ -459,12 +452,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
                 for (int s = 0; s < NB; ++s)
                     s_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j][s], qf[s], s_acc[j], 0, 0, 0);
             }
-            // s_acc[j][r]: key kb + 16 j + 4 g + r, head = this lane's column
+            // s_acc[j][r]: key kb + 8 g + 4 j + r, head = this lane's column
             float sv[8];
             float mx = -INFINITY;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int key = kb + 16 * (e >> 2) + 4 * g + (e & 3);
+                const int key = kb + 8 * g + e;
                 const bool ok = key >= lo && key < ctx;
                 sv[e] = ok ? s_acc[e >> 2][e & 3] * scale2 : -INFINITY;
                 mx = fmaxf(mx, sv[e]);
