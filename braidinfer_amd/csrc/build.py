@@ -73,15 +73,26 @@ def _build_dirs() -> List[str]:
     return dirs
 
 
+def _file_digest(path: str) -> str:
+    h = hashlib.sha256()
+    with open(path, "rb") as f:
+        for chunk in iter(lambda: f.read(1 << 20), b""):
+            h.update(chunk)
+    return h.hexdigest()
+
+
 def _find_built(name: str, digest: str) -> Optional[str]:
+    """A library counts as built when its tag names both the sources it was made from and
+    the library file itself (a tag restored or copied without its library does not)."""
     for d in _build_dirs():
         so = os.path.join(d, f"br_{name}.so")
-        tag = so + ".sha256"
+        tag = so + ".tag"
         if os.path.isfile(so) and os.path.isfile(tag):
             try:
                 with open(tag) as f:
-                    if f.read().strip() == digest:
-                        return so
+                    parts = f.read().split()
+                if len(parts) == 2 and parts[0] == digest and parts[1] == _file_digest(so):
+                    return so
             except OSError:
                 pass
     return None
@@ -145,8 +156,8 @@ def compile_module(name: str, force: bool = False) -> str:
             pass
         raise KernelError(f"hipcc failed for {name} (exit {proc.returncode}):\n{text}")
     os.replace(tmp, so)
-    with open(so + ".sha256", "w") as f:
-        f.write(digest)
+    with open(so + ".tag", "w") as f:
+        f.write(f"{digest} {_file_digest(so)}\n")
     _log(f"built {name} in {time.time() - t0:.1f} s -> {so}")
     return so
 

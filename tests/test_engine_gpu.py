@@ -306,3 +306,40 @@ def test_the_windows_edge_is_exact(tmp_path, dtype):
             eng.free_slot(s)
             assert (int(got.argmax()) == 1) == seen, f"marker at {at}, cut {cut}: window edge is off"
             close(got[None], ref[None], dtype, f"window edge, marker at {at}, cut {cut}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["b", "c"])
+def test_random_schedules_of_cuts_and_batches(engines, tiny_folders, name, dtype):
+    """Requests arrive at random steps, bring chunks of random sizes (1, a few, a page and
+    more), leave when they are done; every position's logits are compared with the plain
+    implementation, whatever the step it fell into."""
+    _, cfg, w = tiny_folders[name]
+    eng = engines(name, dtype)
+    rng = np.random.default_rng(7 if name == "b" else 8)
+    free_before = [g.pool.free_count for g in eng.cache.groups]
+    seqs = [tokens(cfg, int(n), 200 + i) for i, n in enumerate(rng.integers(1, 260, 9))]
+    refs = [P.forward(cfg, w, s) for s in seqs]
+    waiting = list(range(len(seqs)))
+    live, pos, got = {}, {}, {i: [] for i in range(len(seqs))}
+    while waiting or live:
+        for i in list(waiting):
+            if len(live) < 4 and rng.random() < 0.5:
+                waiting.remove(i); live[i] = eng.alloc_slot(); pos[i] = 0
+        if not live:
+            continue
+        chosen = [i for i in live if rng.random() < 0.8] or list(live)[:1]
+        entries, takes = [], []
+        for i in chosen:
+            n = min(int(rng.choice([1, 1, 2, 7, 64, 65, 130])), len(seqs[i]) - pos[i])
+            entries.append(StepEntry(live[i], seqs[i][pos[i]:pos[i] + n], list(range(n))))
+            takes.append(n)
+        out = eng.step(entries).cpu().numpy()
+        o = 0
+        for i, n in zip(chosen, takes):
+            got[i].append(out[o:o + n]); o += n; pos[i] += n
+            if pos[i] == len(seqs[i]):
+                eng.free_slot(live.pop(i))
+    for i in range(len(seqs)):
+        close(np.concatenate(got[i]), refs[i], dtype, f"{name} request {i} of {len(seqs[i])} tokens")
+    assert [g.pool.free_count for g in eng.cache.groups] == free_before
