@@ -124,7 +124,8 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the given tokens of each entry's sequence as one batch, from the cache
         earlier steps left; return float32 logits `[number of wanted places, vocab]` on the
-        device, in the order of the entries and of each entry's `want`.
+        device, in the order of the entries and of each entry's `want`, in a tensor of
+        their own (later steps do not touch it).
 
         Nothing is changed if the step cannot be run (bad entry, no room in the cache)."""
         if not entries:
@@ -146,9 +147,9 @@ class Engine:
                             or not 0 <= t < V), None)
                 raise StepError(f"slot {e.slot}: token {bad!r} is outside the vocabulary of {V}")
             for w in e.want:
-                if not isinstance(w, int) or not 0 <= w < len(tl):
+                if not isinstance(w, (int, np.integer)) or isinstance(w, bool) or not 0 <= w < len(tl):
                     raise StepError(f"slot {e.slot}: wanted place {w!r} is outside its {len(tl)} tokens")
-                rows.append(base + w)
+                rows.append(base + int(w))
             base += len(tl)
         new = [len(tl) for tl in token_lists]
         self.cache.reserve(slots, new)          # all or nothing

@@ -49,7 +49,8 @@ class DecodeGraph:
             is_decode=True, max_new=1, max_ctx=cache.max_seq_len,
             max_ctx_bound=cache.max_seq_len, ws=self.ws)
         # once eagerly with padding only: loads the kernels, sizes the workspace, stores nothing
-        model.forward(self.step, cache, self.want_rows, B)
+        self.logits = torch.empty((B, model.spec.vocab_size), dtype=torch.float32, device=dev)
+        model.forward(self.step, cache, self.want_rows, B, self.logits)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
         # no garbage collection while the stream is capturing: a collected tensor or graph
@@ -58,7 +59,7 @@ class DecodeGraph:
         gc.disable()
         try:
             with torch.cuda.graph(self.graph):
-                self.logits = model.forward(self.step, cache, self.want_rows, B)
+                model.forward(self.step, cache, self.want_rows, B, self.logits)
         finally:
             if gc_was_on:
                 gc.enable()

@@ -131,9 +131,11 @@ class DecoderModel:
         return out
 
     # ---- one step ----------------------------------------------------------------------
-    def forward(self, step: StepBatch, cache: SequenceCache, want_rows: torch.Tensor, n_want: int) -> torch.Tensor:
+    def forward(self, step: StepBatch, cache: SequenceCache, want_rows: torch.Tensor, n_want: int,
+                logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run the step's tokens through every scheduled layer; return float32 logits
-        `[n_want, vocab]` of the rows `want_rows` (indices into the packed tokens)."""
+        `[n_want, vocab]` of the rows `want_rows` (indices into the packed tokens), in
+        `logits_out` when given, else in a tensor of their own."""
         rt = self.rt
         T, H = step.n_tokens, self.spec.hidden_size
         ws = step.ws
@@ -152,7 +154,10 @@ class DecoderModel:
                     ctx.storage, ctx.block_table, ctx.page_tokens = g.storage[e.cache], g.table_dev, g.page_tokens
                 ctx.state = cache.state(("entry", i))
             layer.run(layer, x, step, ctx)
-        logits = ws.get("logits", (max(n_want, 1), self.spec.vocab_size), torch.float32)[:n_want]
+        if logits_out is None:
+            logits = torch.empty((n_want, self.spec.vocab_size), dtype=torch.float32, device=rt.device)
+        else:
+            logits = logits_out[:n_want]
         if n_want == 0:
             return logits
         hn = ws.get("final_h", (n_want, H), rt.dtype)
