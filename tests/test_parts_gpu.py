@@ -329,3 +329,139 @@ def test_a_schedule_that_reads_an_unwritten_cache_is_refused():
             B.DecoderModel(bad)
     finally:
         unregister_architecture("ToyLoopForCausalLM")
+
+
+# ---------------------------------- a toy routed feed-forward and a toy position encoding ----
+from braidinfer_amd.parts import FeedForward, PositionEncoding   # noqa: E402
+
+
+class Top1Experts(FeedForward):
+    """Two small experts and a router; each token goes to the expert with the larger router
+    logit (computed in float), weighted by the softmax of the two.  torch operations: a
+    test's toy."""
+
+    def __init__(self, hidden_size, expert_size, num_experts=2):
+        self.H, self.E, self.n = hidden_size, expert_size, num_experts
+
+    def weight_specs(self, prefix):
+        specs = [TensorSpec(prefix + "router.weight", (self.n, self.H))]
+        for e in range(self.n):
+            specs += [TensorSpec(prefix + f"experts.{e}.up.weight", (self.E, self.H)),
+                      TensorSpec(prefix + f"experts.{e}.down.weight", (self.H, self.E))]
+        return specs
+
+    def load(self, tensors, prefix, rt):
+        self.rt = rt
+        self.router = tensors[prefix + "router.weight"].float()
+        self.up = [tensors[prefix + f"experts.{e}.up.weight"].float() for e in range(self.n)]
+        self.down = [tensors[prefix + f"experts.{e}.down.weight"].float() for e in range(self.n)]
+
+    def forward(self, h, x, step):
+        hf = h.float()
+        logits = hf @ self.router.T
+        gate = torch.softmax(logits, -1)
+        pick = logits.argmax(-1)
+        for e in range(self.n):
+            m = pick == e
+            if m.any():
+                y = torch.relu(hf[m] @ self.up[e].T) @ self.down[e].T
+                x[m] += y * gate[m, e:e + 1]
+
+
+class LearnedPositions(PositionEncoding):
+    """A table of position vectors added to the embeddings (no rotation anywhere)."""
+
+    def __init__(self, max_positions, hidden_size):
+        self.P, self.H = max_positions, hidden_size
+
+    def weight_specs(self, prefix):
+        return [TensorSpec(prefix + "weight", (self.P, self.H))]
+
+    def load(self, tensors, prefix, rt):
+        self.rt = rt
+        self.table = tensors[prefix + "weight"].float()
+
+    def add_to_embedding(self, x, step):
+        x += self.table[step.positions.long()]
+
+
+@dataclass(frozen=True)
+class RoutedConfig:
+    architecture = "ToyRoutedForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls()
+
+    def to_dict(self):
+        return {"architectures": [self.architecture]}
+
+
+def routed_spec(cfg):
+    H = 48
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 3, "head_dim": 16,
+                                      "window": None, "position": None})          # attention without rotation
+    layers = [LayerSpec("r.layers.0.", attn, PartSpec("top1_experts", {"hidden_size": H, "expert_size": 24}), norm, norm),
+              LayerSpec("r.layers.1.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 64}), norm, norm)]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=60,
+                     embedding=PartSpec("embedding", {"vocab_size": 60, "hidden_size": H}), layers=layers,
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1)], final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": 60, "hidden_size": H, "tied_to": None}),
+                     positions={"learned": PartSpec("learned_positions", {"max_positions": 128, "hidden_size": H})},
+                     max_position_embeddings=128, embedding_prefix="r.embed.", final_norm_prefix="r.norm.",
+                     lm_head_prefix="r.head.")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_learned_positions(tmp_path, dtype):
+    """Different feed-forwards in different layers, a position encoding that acts on the
+    embeddings, attention that rotates nothing: registered, built and stepped from outside."""
+    register_part("feed_forward", "top1_experts", Top1Experts)
+    register_part("position", "learned_positions", LearnedPositions)
+    register_architecture("ToyRoutedForCausalLM", RoutedConfig, routed_spec)
+    try:
+        folder = B.Engine.write_random_folder(str(tmp_path / "routed"), RoutedConfig(), seed=6, std=0.15)
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=256)
+        assert not eng.use_graphs                          # the toys decide on the host: no graph capture
+        _, w = P.read_folder(folder)
+
+        def plain(toks):
+            T = len(toks)
+            x = P.embedding(w["r.embed.weight"], toks) + w["position.learned.weight"][:T]
+            for l, ffn in ((0, "experts"), (1, "swiglu")):
+                p = f"r.layers.{l}."
+                n = P.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+                q, k, v = (P.linear(n, w[p + f"self_attn.{m}_proj.weight"]).reshape(T, 3, 16) for m in "qkv")
+                x = x + P.linear(P.attention(q, k, v, 3, 3).reshape(T, 48), w[p + "self_attn.o_proj.weight"])
+                n = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+                if ffn == "swiglu":
+                    x = x + P.swiglu(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+                else:
+                    logits = n @ w[p + "mlp.router.weight"].T
+                    gate = np.exp(logits - logits.max(-1, keepdims=True)); gate /= gate.sum(-1, keepdims=True)
+                    for t in range(T):
+                        e = int(logits[t].argmax())
+                        y = np.maximum(n[t] @ w[p + f"mlp.experts.{e}.up.weight"].T, 0) @ w[p + f"mlp.experts.{e}.down.weight"].T
+                        x[t] = x[t] + y * gate[t, e]
+            return P.linear(P.rms_norm(x, w["r.norm.weight"], 1e-5), w["r.head.weight"])
+
+        toks = [int(t) for t in np.random.default_rng(2).integers(0, 60, 50)]
+        ref = plain(toks)
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, toks[:30], list(range(30)))]).cpu().numpy()]
+        for t in toks[30:]:
+            got.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+        eng.free_slot(s)
+        got = np.concatenate(got)
+        if dtype == "float32":
+            assert np.abs(got - ref).max() < 1e-4 * np.abs(ref).max()
+        else:
+            # bf16 may send a token whose two router logits are within rounding to the other
+            # expert, which changes that position and those after it: most positions agree
+            cos = (got * ref).sum(-1) / (np.linalg.norm(got, axis=-1) * np.linalg.norm(ref, axis=-1))
+            assert np.median(cos) > 0.999
+    finally:
+        unregister_architecture("ToyRoutedForCausalLM")
+        unregister_part("feed_forward", "top1_experts")
+        unregister_part("position", "learned_positions")
