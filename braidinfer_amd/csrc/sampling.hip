@@ -139,30 +139,188 @@ __device__ __forceinline__ int block_first_reach(int n, float target, F f, float
 }
 
 // ------------------------------------------------- top-k / min-p / top-p filter ----
-// Masks entries of work[b, :] to -inf as sampling.rs:89-151 does.  The row is sorted
-// once, descending by value with the lower index first among equals, as 64-bit keys
-// (value key << 32 | ~index) by a bitonic network in `keys` ([B, n2], n2 = V rounded up
-// to a power of two).  top-k keeps the first k of that order; min-p keeps values with
-// exp(v - max) >= min_p; top-p keeps the shortest prefix of the survivors whose
-// probabilities (softmax over the survivors) sum to >= top_p, accumulated in order.
+// Masks entries of work[b, :] to -inf as sampling.rs:89-151 does: top-k keeps the k
+// largest; min-p keeps values with exp(v - max) >= min_p; top-p keeps the shortest prefix,
+// in descending order, of the survivors whose probabilities (softmax over the survivors)
+// sum to >= top_p.  Order is by value, the lower index first among equals: every entry
+// has a 64-bit key (value key << 32 | ~index), all distinct, and "kept" is "key >= some
+// key", so the mask is one pass once that key is known.
+//
+// sample_filter_select_kernel finds it without sorting the row: a radix select over the
+// value keys picks the (at most 1024) largest entries, which are sorted in LDS; top-k,
+// min-p and top-p are then decided on that short list.  A row it cannot decide there
+// (top_k above 1024, or no top-k and a top-p that the 1024 largest do not reach) is
+// flagged in `slow` and left untouched for sample_filter_sort_kernel, which sorts the
+// whole row in global memory.
 #define FBLOCK 1024
-__global__ __launch_bounds__(FBLOCK) void sample_filter_kernel(
+#define CAND 1024
+
+__device__ __forceinline__ unsigned long long comp_key(float v, int i) {
+    return ((unsigned long long)f2key(v) << 32) | (uint32_t)(~(uint32_t)i);
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[w] = v;
+    __syncthreads();
+    float t = -INFINITY;
+    for (int i = 0; i < nw; ++i) t = fmaxf(t, scratch[i]);
+    return t;
+}
+
+__global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
+    float* __restrict__ work, int V, const int* __restrict__ top_k, const float* __restrict__ min_p,
+    const float* __restrict__ top_p, const float* __restrict__ temperature, int* __restrict__ slow) {
+    __shared__ unsigned long long ck[CAND];
+    __shared__ int hist[256];
+    __shared__ float red[16];
+    __shared__ float wsum[FBLOCK / 64];
+    __shared__ int sh_bin, sh_need, sh_ties, sh_cnt, keep_s;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int k = top_k[b];
+    const float mp = min_p[b], tp = top_p[b];
+    const bool use_k = k > 0 && k < V, use_mp = mp > 0.f, use_tp = tp < 1.f;
+    if (tid == 0) slow[b] = 0;
+    if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
+    if (use_k && k > CAND) { if (tid == 0) slow[b] = 1; return; }
+    float* w = work + (size_t)b * V;
+    float mx = -INFINITY;
+    for (int i = tid; i < V; i += FBLOCK) mx = fmaxf(mx, w[i]);
+    const float vmax = block_max(mx, red);
+    if (!use_k && !use_tp) {          // min-p alone is a threshold on the value
+        for (int i = tid; i < V; i += FBLOCK)
+            if (w[i] > -INFINITY && expf(w[i] - vmax) < mp) w[i] = -INFINITY;
+        return;
+    }
+    const int cand = use_k ? k : (V < CAND ? V : CAND);
+    // radix select: the value key T of the cand-th largest entry, 8 bits a pass
+    uint32_t prefix = 0, bits = 0;
+    int need = cand, ties = 0;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        for (int i = tid; i < V; i += FBLOCK) {
+            const uint32_t key = f2key(w[i]);
+            if ((key & bits) == prefix) atomicAdd(&hist[(key >> shift) & 255], 1);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int cum = 0, bin = 255;
+            for (; bin > 0; --bin) {
+                if (cum + hist[bin] >= need) break;
+                cum += hist[bin];
+            }
+            sh_bin = bin; sh_need = need - cum; sh_ties = hist[bin];
+        }
+        __syncthreads();
+        prefix |= (uint32_t)sh_bin << shift;
+        bits |= 255u << shift;
+        need = sh_need;
+        ties = sh_ties;
+        __syncthreads();
+    }
+    const uint32_t T = prefix;        // take every key above T and `need` of the `ties` keys equal to it
+    if (tid == 0) sh_cnt = 0;
+    __syncthreads();
+    for (int i = tid; i < V; i += FBLOCK) {
+        const float v = w[i];
+        if (f2key(v) > T) ck[atomicAdd(&sh_cnt, 1)] = comp_key(v, i);
+    }
+    __syncthreads();
+    const int ngt = sh_cnt;
+    if (ties == need) {
+        for (int i = tid; i < V; i += FBLOCK) {
+            const float v = w[i];
+            if (f2key(v) == T) ck[atomicAdd(&sh_cnt, 1)] = comp_key(v, i);
+        }
+    } else {
+        // more equal values than places: the lowest indices win, found by an ordered scan
+        const int lane = tid & 63, wv = tid >> 6;
+        int base = 0;
+        for (int i0 = 0; i0 < V && base < need; i0 += FBLOCK) {
+            const int i = i0 + tid;
+            const float v = i < V ? w[i] : 0.f;
+            const int flag = (i < V && f2key(v) == T) ? 1 : 0;
+            int sc = flag;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+            __syncthreads();
+            if (lane == 63) hist[wv] = sc;
+            __syncthreads();
+            int before = base, tot = base;
+            for (int x = 0; x < FBLOCK / 64; ++x) { if (x < wv) before += hist[x]; tot += hist[x]; }
+            const int rank = before + sc - flag;
+            if (flag && rank < need) ck[ngt + rank] = comp_key(v, i);
+            base = tot;
+            __syncthreads();
+        }
+    }
+    for (int t = cand + tid; t < CAND; t += FBLOCK) ck[t] = 0ull;
+    __syncthreads();
+    // bitonic sort of the candidates in LDS, descending
+    for (int size = 2; size <= CAND; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            if (tid < CAND / 2) {
+                const int lo = 2 * tid - (tid & (stride - 1)), hi = lo + stride;
+                const bool desc = (lo & size) == 0;
+                const unsigned long long a = ck[lo], c = ck[hi];
+                if ((a < c) == desc) { ck[lo] = c; ck[hi] = a; }
+            }
+            __syncthreads();
+        }
+    }
+    // survivors are a prefix [0, keep) of the candidates
+    int keep = cand;
+    float cnt = 0.f, part = 0.f;
+    for (int i = tid; i < cand; i += FBLOCK) {
+        const float v = key2f((uint32_t)(ck[i] >> 32));
+        if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { cnt += 1.f; part += expf(v - vmax); }
+    }
+    keep = (int)(block_sum(cnt, red) + 0.5f);
+    float sum = block_sum(part, red);
+    bool covered = true;              // do the candidates hold every survivor?
+    if (!use_k) {
+        // without top-k the survivors are all entries that pass min-p: count and add them all
+        float call = 0.f, pall = 0.f;
+        for (int i = tid; i < V; i += FBLOCK) {
+            const float v = w[i];
+            if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { call += 1.f; pall += expf(v - vmax); }
+        }
+        covered = (int)(block_sum(call, red) + 0.5f) <= keep;
+        sum = block_sum(pall, red);
+    }
+    if (use_tp) {
+        const int hit = block_first_reach(keep, tp, [&](int i) {
+            return expf(key2f((uint32_t)(ck[i] >> 32)) - vmax) / sum; }, wsum, &keep_s);
+        if (hit < keep) keep = hit + 1;
+        else if (!covered) { if (tid == 0) slow[b] = 1; return; }
+    }
+    const unsigned long long last = ck[keep - 1];
+    for (int i = tid; i < V; i += FBLOCK)
+        if (comp_key(w[i], i) < last) w[i] = -INFINITY;
+}
+
+// The general form: the whole row is sorted once as 64-bit keys by a bitonic network in
+// `keys` ([B, n2], n2 = V rounded up to a power of two).  With `slow` given, only the rows
+// it flags are treated.
+__global__ __launch_bounds__(FBLOCK) void sample_filter_sort_kernel(
     float* __restrict__ work, unsigned long long* __restrict__ keys, int V, int n2,
     const int* __restrict__ top_k, const float* __restrict__ min_p, const float* __restrict__ top_p,
-    const float* __restrict__ temperature) {
+    const float* __restrict__ temperature, const int* __restrict__ slow) {
     __shared__ float red[16];
     __shared__ float wsum[FBLOCK / 64];
     __shared__ int keep_s;
     const int b = blockIdx.x;
+    if (slow && !slow[b]) return;
     const int k = top_k[b]; const float mp = min_p[b], tp = top_p[b];
     const bool use_k = k > 0 && k < V, use_mp = mp > 0.f, use_tp = tp < 1.f;
     if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
     float* w = work + (size_t)b * V;
     unsigned long long* ks = keys + (size_t)b * n2;
-    for (int i = threadIdx.x; i < n2; i += FBLOCK)
-        ks[i] = i < V ? (((unsigned long long)f2key(w[i]) << 32) | (uint32_t)(~(uint32_t)i)) : 0ull;
+    for (int i = threadIdx.x; i < n2; i += FBLOCK) ks[i] = i < V ? comp_key(w[i], i) : 0ull;
     __syncthreads();
-    // bitonic sort, descending
     for (int size = 2; size <= n2; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             for (int i = threadIdx.x; i < n2 / 2; i += FBLOCK) {
@@ -174,44 +332,44 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_kernel(
             __syncthreads();
         }
     }
-    // survivors are a prefix [0, keep) of the sorted order
-    int keep = V;
-    if (use_k) keep = k;
+    int keep = use_k ? k : V;         // survivors are a prefix [0, keep) of the sorted order
     const float vmax = key2f((uint32_t)(ks[0] >> 32));
-    if (use_mp) {
-        // values are descending: count entries of the prefix with exp(v - max) >= min_p
-        float cnt = 0.f;
-        for (int i = threadIdx.x; i < keep; i += FBLOCK) {
-            float v = key2f((uint32_t)(ks[i] >> 32));
-            if (!(v > -INFINITY && expf(v - vmax) < mp)) cnt += 1.f;
-        }
-        keep = (int)(block_sum(cnt, red) + 0.5f);
+    float cnt = 0.f, part = 0.f;
+    for (int i = threadIdx.x; i < keep; i += FBLOCK) {
+        const float v = key2f((uint32_t)(ks[i] >> 32));
+        if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { cnt += 1.f; part += expf(v - vmax); }
     }
+    keep = (int)(block_sum(cnt, red) + 0.5f);
+    const float sum = block_sum(part, red);
     if (use_tp) {
-        float part = 0.f;
-        for (int i = threadIdx.x; i < keep; i += FBLOCK) {
-            float v = key2f((uint32_t)(ks[i] >> 32));
-            if (v > -INFINITY) part += expf(v - vmax);
-        }
-        const float sum = block_sum(part, red);
-        // survivors with a finite value are a prefix too (masked entries sort last)
-        float fin = 0.f;
-        for (int i = threadIdx.x; i < keep; i += FBLOCK)
-            if (key2f((uint32_t)(ks[i] >> 32)) > -INFINITY) fin += 1.f;
-        const int nfin = (int)(block_sum(fin, red) + 0.5f);
-        const int hit = block_first_reach(nfin, tp, [&](int i) {
+        const int hit = block_first_reach(keep, tp, [&](int i) {
             return expf(key2f((uint32_t)(ks[i] >> 32)) - vmax) / sum; }, wsum, &keep_s);
-        keep = hit < nfin ? hit + 1 : nfin;
+        if (hit < keep) keep = hit + 1;
     }
     for (int i = keep + threadIdx.x; i < V; i += FBLOCK) w[~(uint32_t)(ks[i] & 0xffffffffu)] = -INFINITY;
 }
 
+// slow: int [B] scratch.  keys: [B, n2] scratch, needed only when `with_sort` (some row may
+// take the general form: top_k above 1024, or top-p without top-k).
 extern "C" int br_sample_filter(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
-                                const float* min_p, const float* top_p, const float* temperature,
-                                hipStream_t s) {
+                                const float* min_p, const float* top_p, const float* temperature, int* slow,
+                                int with_sort, hipStream_t s) {
     if (B <= 0) return BR_OK;
-    if (V <= 0 || n2 < V || (n2 & (n2 - 1))) return BR_BAD_ARG;
-    sample_filter_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature);
+    if (V <= 0 || !slow || (with_sort && (!keys || n2 < V || (n2 & (n2 - 1))))) return BR_BAD_ARG;
+    sample_filter_select_kernel<<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
+    int rc = br_check_launch();
+    if (rc != BR_OK || !with_sort) return rc;
+    sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, slow);
+    return br_check_launch();
+}
+
+// the general form alone, for every row (tests compare the two)
+extern "C" int br_sample_filter_sort(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
+                                     const float* min_p, const float* top_p, const float* temperature,
+                                     hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0 || !keys || n2 < V || (n2 & (n2 - 1))) return BR_BAD_ARG;
+    sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, nullptr);
     return br_check_launch();
 }
 

@@ -6,6 +6,7 @@ from __future__ import annotations
 from collections import Counter
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from .. import kernels as K
@@ -16,6 +17,7 @@ class Sampler:
     def __init__(self, device, vocab_size: int):
         self.device = torch.device(device)
         self.V = int(vocab_size)
+        self._keys = None          # scratch for whole-row sorts, made when first needed
 
     def _i32(self, v):
         return torch.tensor(v, dtype=torch.int32).to(self.device)
@@ -59,14 +61,29 @@ class Sampler:
                         cnt.append(c)
                 off.append(len(tok))
             hist_off, hist_tok, hist_cnt = self._i32(off), self._i32(tok or [0]), self._i32(cnt or [0])
-        temperature = self._f32([p.temperature for p in params])
-        penalty = self._f32([p.repetition_penalty for p in params])
+        # the per-row numbers go over in one copy: five float rows and one int row
+        host = np.empty((6, B), dtype=np.float32)
+        host[0] = [p.temperature for p in params]
+        host[1] = [p.repetition_penalty for p in params]
+        host[2] = [p.min_p for p in params]
+        host[3] = [p.top_p for p in params]
+        host[4] = list(us)
+        host[5].view(np.int32)[:] = [p.top_k for p in params]
+        dev = torch.from_numpy(host).to(self.device)
+        temperature, penalty, min_p, top_p, u = dev[0], dev[1], dev[2], dev[3], dev[4]
+        top_k = dev[5].view(torch.int32)
         K.sample_prepare(logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature)
-        if any(p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0) for p in params):
-            n2 = 1 << (V - 1).bit_length()
-            keys = torch.empty((B, n2), dtype=torch.int64, device=self.device)
-            K.sample_filter(work, keys, self._i32([p.top_k for p in params]), self._f32([p.min_p for p in params]),
-                            self._f32([p.top_p for p in params]), temperature)
+        filtered = [p for p in params if p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)]
+        if filtered:
+            # rows that the short-list kernel may hand on need room for a sort of the whole row
+            keys = None
+            if any(p.top_k > K.FILTER_CANDIDATES or (not 0 < p.top_k < V and p.top_p < 1.0) for p in filtered):
+                n2 = 1 << (V - 1).bit_length()
+                if self._keys is None or self._keys.shape[0] < B:
+                    self._keys = torch.empty((B, n2), dtype=torch.int64, device=self.device)
+                keys = self._keys
+            slow = torch.empty(B, dtype=torch.int32, device=self.device)
+            K.sample_filter(work, top_k, min_p, top_p, temperature, slow, keys)
         out = torch.empty(B, dtype=torch.int32, device=self.device)
-        K.sample_draw(work, out, temperature, self._f32(list(us)))
+        K.sample_draw(work, out, temperature, u)
         return out.tolist()

@@ -200,23 +200,11 @@ def argmax_lowest(v):
     return int(np.argmax(np.asarray(v)))
 
 
-def sample(logits, u, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, repetition_penalty=1.0,
-           history=(), logit_bias=None):
-    """The reference's sampler in its order (sampling.rs:49-171), with the uniform draw
-    `u` given.  Sorting is stable by (value descending, index ascending)."""
-    l = np.array(logits, dtype=F)
+def filter_logits(l, top_k=0, top_p=1.0, min_p=0.0):
+    """Top-k, then min-p, then top-p (sampling.rs:89-151): the logits with what is cut set
+    to -inf.  Sorting is stable by (value descending, index ascending)."""
+    l = np.array(l, dtype=F)
     n = l.shape[0]
-    if logit_bias:
-        for tok, d in logit_bias:
-            if 0 <= tok < n:
-                l[tok] = F(l[tok] + F(d))
-    if repetition_penalty != 1.0:
-        for tok in history:
-            if 0 <= tok < n:
-                l[tok] = F(l[tok] / F(repetition_penalty)) if l[tok] > 0 else F(l[tok] * F(repetition_penalty))
-    if temperature == 0.0:
-        return argmax_lowest(l)
-    l = (l / F(temperature)).astype(F)
     order = sorted(range(n), key=lambda i: (-l[i], i))
     if 0 < top_k < n:
         for i in order[top_k:]:
@@ -239,6 +227,26 @@ def sample(logits, u, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, repetition
                 break
         for i in idx[cut:]:
             l[i] = -np.inf
+    return l
+
+
+def sample(logits, u, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, repetition_penalty=1.0,
+           history=(), logit_bias=None):
+    """The reference's sampler in its order (sampling.rs:49-171), with the uniform draw
+    `u` given.  Sorting is stable by (value descending, index ascending)."""
+    l = np.array(logits, dtype=F)
+    n = l.shape[0]
+    if logit_bias:
+        for tok, d in logit_bias:
+            if 0 <= tok < n:
+                l[tok] = F(l[tok] + F(d))
+    if repetition_penalty != 1.0:
+        for tok in history:
+            if 0 <= tok < n:
+                l[tok] = F(l[tok] / F(repetition_penalty)) if l[tok] > 0 else F(l[tok] * F(repetition_penalty))
+    if temperature == 0.0:
+        return argmax_lowest(l)
+    l = filter_logits((l / F(temperature)).astype(F), top_k, top_p, min_p)
     mx = l.max()
     pr = np.exp((l - mx).astype(F), dtype=F)
     pr = pr / pr.sum(dtype=F)

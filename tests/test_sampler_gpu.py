@@ -77,3 +77,73 @@ def test_distribution_follows_the_probabilities():
     got = run(np.tile(logits, (n, 1)), SamplingParams(temperature=1.0, top_k=0), us=us)
     freq = np.bincount(got, minlength=5) / n
     assert np.abs(freq - want).max() < 2e-3
+
+
+# ---- the filter kernels alone -------------------------------------------------------------
+def _filter_gpu(rows, top_k, min_p, top_p, general):
+    from braidinfer_amd import kernels as K
+    B, V = rows.shape
+    work = torch.tensor(rows).to(DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32).to(DEV)
+    f32 = lambda v: torch.tensor(v, dtype=torch.float32).to(DEV)
+    keys = torch.empty((B, 1 << (V - 1).bit_length()), dtype=torch.int64, device=DEV)
+    temp = f32([1.0] * B)
+    if general:
+        K.sample_filter_sort(work, keys, i32(top_k), f32(min_p), f32(top_p), temp)
+        return work.cpu().numpy(), None
+    slow = torch.full((B,), -1, dtype=torch.int32, device=DEV)
+    K.sample_filter(work, i32(top_k), f32(min_p), f32(top_p), temp, slow, keys)
+    return work.cpu().numpy(), slow.cpu().numpy()
+
+
+def _check_row(row, got, k, mp, tp, label):
+    """`got` keeps a prefix of the (value descending, index ascending) order whose length is
+    the plain filter's, or, where a float sum in another order moves the top-p cut by
+    rounding, the plain filter's at a top_p within that rounding."""
+    V = row.shape[0]
+    order = sorted(range(V), key=lambda i: (-row[i], i))
+    kept = [i for i in range(V) if got[i] > -np.inf]
+    assert all(got[i] == row[i] for i in kept), label
+    assert sorted(kept) == sorted(order[:len(kept)]), f"{label}: kept entries are not the first of the order"
+    count = lambda t: int((P.filter_logits(row, k, min(max(t, 0.0), 1.0), mp) > -np.inf).sum())
+    counts = {count(tp)}
+    if tp < 1.0:
+        # a running float32 sum of n probabilities is off by at most n * 2^-24
+        eps = max(counts) * 2.0 ** -24
+        counts |= {count(tp - eps), count(tp + eps)}
+    assert min(counts) <= len(kept) <= max(counts), f"{label}: kept {len(kept)}, plain {sorted(counts)}"
+
+
+@pytest.mark.parametrize("V", [257, 3000, 32768 + 5])
+def test_filter_short_list_and_whole_row_sort_agree_with_the_plain_filter(V):
+    rng = np.random.default_rng(V)
+    smooth = (rng.normal(size=V) * 3).astype(np.float32)
+    peaked = smooth.copy(); peaked[rng.integers(0, V, 5)] += 12.0
+    tied = np.round(rng.normal(size=V) * 2).astype(np.float32)           # many equal values
+    flat = np.zeros(V, np.float32)                                        # all equal
+    holes = smooth.copy(); holes[rng.integers(0, V, V // 3)] = -np.inf    # already masked entries
+    cases = []
+    for name, row in (("smooth", smooth), ("peaked", peaked), ("tied", tied), ("flat", flat), ("holes", holes)):
+        for k, mp, tp in ((1, 0.0, 1.0), (5, 0.0, 1.0), (50, 0.0, 1.0), (50, 0.05, 0.9), (200, 0.0, 0.5),
+                          (1024, 0.0, 1.0), (1025, 0.0, 0.95), (0, 0.1, 1.0), (0, 0.0, 0.9), (0, 0.02, 0.999),
+                          (0, 0.0, 0.3), (V, 0.0, 0.7), (V - 1, 0.0, 1.0)):
+            cases.append((f"{name} k={k} min_p={mp} top_p={tp}", row, k, mp, tp))
+    rows = np.stack([c[1] for c in cases])
+    ks, mps, tps = [c[2] for c in cases], [c[3] for c in cases], [c[4] for c in cases]
+    fast, slow = _filter_gpu(rows, ks, mps, tps, general=False)
+    whole, _ = _filter_gpu(rows, ks, mps, tps, general=True)
+    assert set(np.unique(slow)) <= {0, 1}
+    for b, (label, row, k, mp, tp) in enumerate(cases):
+        if V > 1100:
+            # a top_k within the short list never needs the whole row; one above it always does
+            if 0 < k <= 1024:
+                assert slow[b] == 0, label
+            if 1024 < k < V:
+                assert slow[b] == 1, label
+        _check_row(row, fast[b], k, mp, tp, "short list, " + label)
+        _check_row(row, whole[b], k, mp, tp, "whole row, " + label)
+    if V > 1100:
+        flat_top_p = [b for b, c in enumerate(cases) if c[0].startswith("flat k=0 min_p=0.0 top_p=0.9")]
+        assert slow[flat_top_p[0]] == 1       # 1024 equal entries of 32773 do not reach 0.9
+        peaked_top_p = [b for b, c in enumerate(cases) if c[0].startswith("peaked k=0 min_p=0.0 top_p=0.3")]
+        assert slow[peaked_top_p[0]] == 0
