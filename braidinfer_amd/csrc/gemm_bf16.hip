@@ -2,7 +2,10 @@
 // bf16 inputs, float accumulation, and a bf16 or float output.  W is a weight matrix as
 // checkpoints store it ([out, in], row-major), so both operands are read along k.
 //
-// Two kernels:
+// Kernels:
+//  * gemm_stream: M <= 16 rows (decode): weight streaming by one resident workgroup per
+//    compute unit, weights and activations brought into per-wave LDS rings by direct
+//    global-to-LDS loads (described at the kernel).
 //  * gemm_tile: LDS-staged tiles for many rows (prompts): 4 waves, each a TM x TN grid of
 //    v_mfma_f32_32x32x16_bf16 blocks; global loads of the next k-tile are issued before the
 //    current one is multiplied and written to the other LDS buffer after it.
@@ -659,9 +662,197 @@ static int launch_skinny_lds(const bf16* A, const bf16* W, void* C, int M, int N
     return br_check_launch();
 }
 
+// ------------------------------------------------------------------ gemm_stream ------
+// M <= 16, K in steps of 128: weight streaming by workgroups that stay.  One workgroup per
+// compute unit walks over tiles of 16 weight rows (tile t of workgroup b is b + t * grid);
+// its 8 waves take the tile's 128-wide k-chunks in turn.  A wave brings a chunk of the
+// tile (16 rows x 256 bytes) and the same chunk of the activations (8 or 16 rows) into a
+// ring of LDS stages of its own with direct global-to-LDS loads: whole 256-byte row
+// pieces per request, no registers, and the loads of the next chunk (of the next tile,
+// at a tile's end) are in flight while this one is multiplied.  No wave waits for another
+// inside a tile; at a tile's end the waves' sums meet in LDS (one barrier, two buffers)
+// and are added in wave order.  The 16-byte columns of a row are XOR-swizzled by the row
+// number through the choice of the global column a lane fetches.
+template <int RT, int XR, int KC, int S, int NW, int MODE>
+__global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                              void* __restrict__ C, int M, int N, int K, size_t lda,
+                                                              size_t ldc, int ntiles) {
+    constexpr int STEPS = KC / 32;
+    constexpr int ROWB = KC * 2;
+    constexpr int STAGE = (RT + XR) * ROWB;
+    constexpr int WDMA = RT * ROWB / 1024;
+    constexpr int NDMA = STAGE / 1024;
+    constexpr int CPL = ROWB / 16;          // 16-byte columns per row
+    constexpr int RPI = 64 / CPL;           // rows per DMA instruction
+    constexpr int LPI = NDMA;
+    constexpr int D = S - 1;
+    static_assert(RPI >= 1 && (D - 1) * LPI <= 63, "wait count");
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    float* red = (float*)(smem + NW * S * STAGE);       // [2][NW][16][17]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    unsigned char* ring = smem + wave * (S * STAGE);
+    const unsigned ring_lds = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)ring);
+
+    const int nch = K / KC;
+    const int ncw = (nch - wave + NW - 1) / NW;
+    const int my_tiles = (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int nitems = my_tiles * ncw;
+
+    // DMA lane mapping
+    const int drow = lane / CPL, dcol = lane % CPL;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+
+    int is_t = 0, is_c = 0;      // issue cursor: local tile index, local chunk index
+    int cp_t = 0, cp_c = 0;      // compute cursor
+    int buf = 0;
+
+#define ISSUE(J)                                                                                         \
+    do {                                                                                                 \
+        const int chunk_ = wave + is_c * NW;                                                             \
+        const int n0_ = ((int)blockIdx.x + is_t * (int)gridDim.x) * RT;                                  \
+        _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                            \
+            const int row_ = q_ * RPI + drow;                                                            \
+            const bf16* gp_;                                                                             \
+            if (q_ < WDMA) {                                                                             \
+                int nrow_ = n0_ + row_;                                                                  \
+                if (nrow_ > N - 1) nrow_ = N - 1;                                                        \
+                gp_ = W + (size_t)nrow_ * K + (size_t)chunk_ * KC + ((dcol ^ (row_ & 7)) * 8);           \
+            } else {                                                                                     \
+                int m_ = row_ - RT;                                                                      \
+                if (m_ > M - 1) m_ = M - 1;                                                              \
+                gp_ = A + (size_t)m_ * lda + (size_t)chunk_ * KC + ((dcol ^ (row_ & 7)) * 8);            \
+            }                                                                                            \
+            const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + (J) * STAGE + q_ * 1024);    \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
+        }                                                                                                \
+        if (++is_c == ncw) { is_c = 0; ++is_t; }                                                         \
+    } while (0)
+
+    // prologue
+#pragma unroll
+    for (int j = 0; j < D; ++j)
+        if (j < nitems) ISSUE(j);
+
+    for (int base = 0; base < nitems; base += S) {
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            const int it = base + j;
+            if (it < nitems) {
+                // wait for item `it`
+                if (it + D - 1 < nitems) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D - 1) * LPI) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                if (it + D < nitems) ISSUE((j + D) % S);
+                // compute
+                const unsigned char* st = ring + j * STAGE;
+                const int rr = RT == 8 ? (r16 & 7) : r16;
+                const int xr = XR == 8 ? (r16 & 7) : r16;
+                bf16x8 wf[STEPS], xv[STEPS];
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    wf[s] = *(const bf16x8*)(st + rr * ROWB + (((4 * s + g) ^ (rr & 7)) * 16));
+                    xv[s] = *(const bf16x8*)(st + (RT + xr) * ROWB + (((4 * s + g) ^ (xr & 7)) * 16));
+                }
+#pragma unroll
+                for (int s = 0; s < STEPS; s += 2) {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], xv[s], acc, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s + 1], xv[s + 1], acc1, 0, 0, 0);
+                }
+                if (++cp_c == ncw) {
+                    cp_c = 0;
+                    const int n0 = ((int)blockIdx.x + cp_t * (int)gridDim.x) * RT;
+                    ++cp_t;
+                    float* rb = red + buf * (NW * 16 * 17);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) rb[(wave * 16 + 4 * g + r) * 17 + r16] = acc[r] + acc1[r];
+                    acc = {0.f, 0.f, 0.f, 0.f};
+                    acc1 = {0.f, 0.f, 0.f, 0.f};
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (MODE == OUT_SWIGLU) {
+                        for (int e = tid; e < 8 * 16; e += NW * 64) {
+                            const int m = e >> 3, jl = e & 7;
+                            if (m < M && n0 + jl + 8 < N) {
+                                float gv = 0.f, uv = 0.f;
+#pragma unroll
+                                for (int w = 0; w < NW; ++w) { gv += rb[(w * 16 + jl) * 17 + m]; uv += rb[(w * 16 + jl + 8) * 17 + m]; }
+                                ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
+                            }
+                        }
+                    } else {
+                        for (int e = tid; e < RT * 16; e += NW * 64) {
+                            const int m = e / RT, nl = e % RT, n = n0 + nl;
+                            if (m < M && n < N) {
+                                float v = 0.f;
+#pragma unroll
+                                for (int w = 0; w < NW; ++w) v += rb[(w * 16 + nl) * 17 + m];
+                                const size_t idx = (size_t)m * ldc + n;
+                                if (MODE == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
+                                else if (MODE == OUT_F32) ((float*)C)[idx] = v;
+                                // one add per element and product, without a read that this wave would
+                                // have to wait for behind its loads in flight
+                                else unsafeAtomicAdd((float*)C + idx, v);
+                            }
+                        }
+                    }
+                    buf ^= 1;
+                }
+            }
+        }
+    }
+#undef ISSUE
+}
+
+
+static int device_cus() {
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (!cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+#define STREAM_KC 128
+#define STREAM_NW 8
+template <int XR>
+static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                         int mode, hipStream_t s) {
+    constexpr int RT = 16, KC = STREAM_KC, S = 2, NW = STREAM_NW;
+    const int cus = device_cus();
+    if (!cus) return BR_LAUNCH_FAILED;
+    const int ntiles = (N + RT - 1) / RT;
+    const int grid = ntiles < cus ? ntiles : cus;
+    constexpr size_t lds = (size_t)NW * S * (RT + XR) * KC * 2 + 2 * NW * 16 * 17 * 4;
+#define BR_STREAM(MODE_)                                                                                        \
+    do {                                                                                                        \
+        auto kern = gemm_stream_kernel<RT, XR, KC, S, NW, MODE_>;                                               \
+        static bool set = false;                                                                                \
+        if (!set) {                                                                                             \
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != \
+                hipSuccess)                                                                                     \
+                return BR_LAUNCH_FAILED;                                                                        \
+            set = true;                                                                                         \
+        }                                                                                                       \
+        kern<<<grid, NW * 64, lds, s>>>(A, W, C, M, N, K, lda, ldc, ntiles);                                    \
+    } while (0)
+    if (mode == OUT_BF16) BR_STREAM(OUT_BF16);
+    else if (mode == OUT_F32) BR_STREAM(OUT_F32);
+    else if (mode == OUT_F32_ACC) BR_STREAM(OUT_F32_ACC);
+    else BR_STREAM(OUT_SWIGLU);
+#undef BR_STREAM
+    return br_check_launch();
+}
+
 // kernel: 0 = choose, 1 = tile 128x128 through registers (any shape), 2 = the same 256x128,
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
-// of 64, aligned rows); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
+// of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
+// rows); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
 // of registers in three of the four epilogues and was no faster in the fourth.)
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
                                size_t ldc, int mode, int kernel, hipStream_t s) {
@@ -673,8 +864,12 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     const bool aligned = (K % 8 == 0) && (lda % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     if (kernel == 3 && (!aligned || M > 64)) return BR_BAD_ARG;
     const bool dma_ok = aligned && K % DMA_BK == 0;
-    if (kernel >= 4 && (!dma_ok || kernel > 6)) return BR_BAD_ARG;
-    if (kernel == 0) kernel = (aligned && M <= 64) ? 3 : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
+    const bool stream_ok = aligned && M <= 16 && K % STREAM_KC == 0 && K / STREAM_KC >= STREAM_NW;
+    if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
+    if ((kernel == 7 && !stream_ok) || kernel > 7 || kernel < 0) return BR_BAD_ARG;
+    if (kernel == 0) kernel = stream_ok ? 7 : (aligned && M <= 64) ? 3 : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
+    if (kernel == 7) return M <= 8 ? launch_stream<8>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                   : launch_stream<16>(A, W, C, M, N, K, lda, ldc, mode, s);
     if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
     if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
     if (kernel == 6) return launch_tile_dma<128, 128, 2, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s);

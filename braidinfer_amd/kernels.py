@@ -174,7 +174,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     Rows of `a` and `out` may be strided (a view of a wider buffer); w is contiguous.
     `kernel` forces one bf16 kernel (1, 2: 128x128 and 256x128 tiles staged through
     registers, any shape; 3: skinny, M <= 64; 4, 5, 6: 256x128, 128x256 and 128x128 tiles
-    loaded straight into LDS, K in steps of 64); 0 chooses by shape.
+    loaded straight into LDS, K in steps of 64; 7: streaming by workgroups that stay, M <= 16
+    and K in steps of 128 from 1024); 0 chooses by shape.
     """
     name = "gemm"
     for t in (a, w, out):

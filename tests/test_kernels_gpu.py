@@ -64,14 +64,19 @@ def test_rmsnorm_reference_vector():
 # ----------------------------------------------------------------------- GEMM ------
 SHAPES = [(1, 64, 64), (5, 100, 96), (17, 192, 320), (64, 301, 100), (33, 1000, 264), (3, 50, 44),
           (130, 514, 100), (257, 129, 72), (300, 260, 1032), (130, 514, 128), (257, 129, 192), (300, 700, 1024),
-          (65, 301, 64), (513, 260, 320)]
+          (65, 301, 64), (513, 260, 320),
+          # few rows and a long k: what the streaming kernel takes (tiles beyond one per workgroup, a chunk
+          # count that the waves do not share evenly)
+          (1, 100, 1024), (8, 301, 1152), (9, 48, 2048), (16, 4100, 1024), (3, 9000, 1280)]
 
 
 def _skip_unless_kernel_takes(kernel, M, Kd):
     if kernel == 3 and (Kd % 8 or M > 64):
         pytest.skip("the skinny kernels take M <= 64 and K in steps of 8")
-    if kernel >= 4 and Kd % 64:
+    if 4 <= kernel <= 6 and Kd % 64:
         pytest.skip("the direct-to-LDS tile kernels take K in steps of 64")
+    if kernel == 7 and (M > 16 or Kd % 128 or Kd < 1024):
+        pytest.skip("the streaming kernel takes M <= 16 and K in steps of 128 from 1024")
 
 
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
@@ -96,7 +101,7 @@ def test_gemm_f32_rows_do_not_depend_on_the_batch():
     assert torch.equal(one[0], full[33])
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
 def test_gemm_bf16(M, N, Kd, kernel):
     _skip_unless_kernel_takes(kernel, M, Kd)
@@ -112,6 +117,28 @@ def test_gemm_bf16(M, N, Kd, kernel):
     acc = base.clone()
     K.gemm(a, w, acc, accumulate=True, kernel=kernel)
     assert (acc.double() - (base.double() + want)).abs().max() < 1e-4 * want.abs().max()
+
+
+def test_gemm_streaming_kernel_rows_and_strides():
+    # a row's result does not depend on the rows beside it, nor on the row stride of a or out
+    Kd, N = 2048, 530
+    a, w = rnd(16, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
+    full = torch.empty(16, N, device=DEV)
+    K.gemm(a, w, full, kernel=7)
+    for rows in (slice(0, 1), slice(5, 6), slice(3, 11), slice(15, 16)):
+        part = torch.empty(rows.stop - rows.start, N, device=DEV)
+        K.gemm(a[rows].contiguous(), w, part, kernel=7)
+        assert torch.equal(part, full[rows])
+    wide_a = torch.zeros(7, Kd + 64, device=DEV, dtype=torch.bfloat16)
+    wide_a[:, 8:8 + Kd] = a[:7]
+    wide_o = torch.full((7, N + 10), 7.0, device=DEV)
+    K.gemm(wide_a[:, 8:8 + Kd], w, wide_o[:, 3:3 + N], kernel=7)
+    assert torch.equal(wide_o[:, 3:3 + N], full[:7])
+    assert bool((wide_o[:, :3] == 7.0).all()) and bool((wide_o[:, 3 + N:] == 7.0).all())
+    with pytest.raises(KernelError):
+        K.gemm(rnd(17, Kd, dtype=torch.bfloat16), w, torch.empty(17, N, device=DEV), kernel=7)
+    with pytest.raises(KernelError):
+        K.gemm(rnd(4, 960, dtype=torch.bfloat16), rnd(N, 960, dtype=torch.bfloat16), torch.empty(4, N, device=DEV), kernel=7)
 
 
 def test_gemm_reference_vectors():
@@ -399,9 +426,9 @@ def test_attention_kernels_refuse_what_they_do_not_take():
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("M,I,Kd", [(1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
-                                    (300, 512, 1024), (129, 200, 192)])
+                                    (300, 512, 1024), (129, 200, 192), (1, 2056, 1024), (8, 328, 1152), (13, 4400, 1280)])
 def test_gemm_with_swiglu_epilogue(M, I, Kd, kernel):
     _skip_unless_kernel_takes(kernel, M, Kd)
     a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
