@@ -182,12 +182,132 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
     }
 }
 
+// The same for many tokens (prompts), bf16, head sizes and rotary sizes in steps of 16:
+// a workgroup takes 64 consecutive tokens of one head.  Rotation works on 16-byte vectors
+// (8 low elements and their 8 partners at once); values go through an LDS tile so that a
+// wave writes one element row of the transposed page for 64 tokens, contiguous wherever
+// the tokens are neighbours in a page, instead of 2-byte stores 128 bytes apart.
+// grid = (ceil(T / 64), nq + 2 nkv), block = 256.
+#define RKV_TOK 64
+__global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
+    bf16* __restrict__ qkv, const float* __restrict__ cs, const float* __restrict__ sn, const int* __restrict__ pos,
+    const int* __restrict__ seq_of_token, const int* __restrict__ slots, const int* __restrict__ block_table,
+    int table_stride, bf16* __restrict__ cache, int T, int nq, int nkv, int hd, int rd, int adjacent,
+    int write_cache) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char rkv_smem[];
+    __shared__ int tok_page[RKV_TOK];      // page of the token's position, -1 if nothing is stored
+    __shared__ int tok_off[RKV_TOK];       // its place in the page
+    const int t0 = blockIdx.x * RKV_TOK, h = blockIdx.y, tid = threadIdx.x;
+    const int nt = T - t0 < RKV_TOK ? T - t0 : RKV_TOK;
+    const int width = (nq + 2 * nkv) * hd;
+    const bool is_q = h < nq, is_k = !is_q && h < nq + nkv;
+    if (!is_q && !write_cache) return;
+    if (!is_q) {
+        if (tid < RKV_TOK) {
+            int pg = -1, off = 0;
+            if (tid < nt) {
+                const int slot = slots[seq_of_token[t0 + tid]];
+                if (slot >= 0) {
+                    const int p = pos[t0 + tid];
+                    pg = block_table[(size_t)slot * table_stride + p / RKV_TOK];
+                    off = p % RKV_TOK;
+                }
+            }
+            tok_page[tid] = pg;
+            tok_off[tid] = off;
+        }
+        __syncthreads();
+    }
+    const size_t unit = (size_t)RKV_TOK * hd;                  // elements of one head's keys (or values) in a page
+    if (is_q || is_k) {
+        const int kvh = h - nq;
+        const int P = rd / 2;
+        // work items of a token row: rotations of 8 pairs, then copies of 8 elements beyond rd
+        const int nrot = adjacent ? rd / 8 : P / 8, ncopy = is_k ? (hd - rd) / 8 : 0, per = nrot + ncopy;
+        for (int e = tid; e < nt * per; e += 256) {
+            const int tl = e / per, w = e - tl * per, t = t0 + tl;
+            const bf16* src = qkv + (size_t)t * width + (size_t)h * hd;
+            bf16* dst;
+            if (is_q) dst = qkv + (size_t)t * width + (size_t)h * hd;
+            else {
+                if (tok_page[tl] < 0) continue;
+                dst = cache + ((size_t)tok_page[tl] * 2 * nkv + kvh) * unit + (size_t)tok_off[tl] * hd;
+            }
+            if (w >= nrot) {
+                const int d = rd + (w - nrot) * 8;
+                *(bf16x8*)(dst + d) = *(const bf16x8*)(src + d);
+                continue;
+            }
+            if (adjacent) {
+                const int d = w * 8;                            // pairs d / 2 .. d / 2 + 3
+                const bf16x8 v = *(const bf16x8*)(src + d);
+                const f32x4 c = cs ? *(const f32x4*)(cs + (size_t)t * P + d / 2) : f32x4{1.f, 1.f, 1.f, 1.f};
+                const f32x4 sgn = sn ? *(const f32x4*)(sn + (size_t)t * P + d / 2) : f32x4{0.f, 0.f, 0.f, 0.f};
+                bf16x8 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float a = (float)v[2 * i], b = (float)v[2 * i + 1];
+                    o[2 * i] = (bf16)(a * c[i] - b * sgn[i]);
+                    o[2 * i + 1] = (bf16)(a * sgn[i] + b * c[i]);
+                }
+                *(bf16x8*)(dst + d) = o;
+            } else {
+                const int d = w * 8;                            // pairs d .. d + 7 with partners at d + P
+                const bf16x8 lo = *(const bf16x8*)(src + d), hi = *(const bf16x8*)(src + d + P);
+                bf16x8 olo, ohi;
+#pragma unroll
+                for (int v4 = 0; v4 < 2; ++v4) {
+                    const f32x4 c = cs ? *(const f32x4*)(cs + (size_t)t * P + d + 4 * v4) : f32x4{1.f, 1.f, 1.f, 1.f};
+                    const f32x4 sgn = sn ? *(const f32x4*)(sn + (size_t)t * P + d + 4 * v4) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float a = (float)lo[4 * v4 + i], b = (float)hi[4 * v4 + i];
+                        olo[4 * v4 + i] = (bf16)(a * c[i] - b * sgn[i]);
+                        ohi[4 * v4 + i] = (bf16)(a * sgn[i] + b * c[i]);
+                    }
+                }
+                *(bf16x8*)(dst + d) = olo;
+                *(bf16x8*)(dst + d + P) = ohi;
+            }
+        }
+        return;
+    }
+    // values: [token][hd] rows into LDS (rows padded by one word against bank conflicts), then element rows out
+    const int kvh = h - nq - nkv;
+    const int ld = hd + 2;
+    bf16* tile = (bf16*)rkv_smem;
+    const int vec = hd / 8;
+    for (int e = tid; e < nt * vec; e += 256) {
+        const int tl = e / vec, c = e - tl * vec;
+        const bf16x8 v = *(const bf16x8*)(qkv + (size_t)(t0 + tl) * width + (size_t)h * hd + c * 8);
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) *(bf16x2*)(tile + tl * ld + c * 8 + i) = bf16x2{v[i], v[i + 1]};
+    }
+    __syncthreads();
+    const int lane = tid & 63, wave = tid >> 6;
+    if (lane < nt && tok_page[lane] >= 0) {
+        bf16* col = cache + (((size_t)tok_page[lane] * 2 + 1) * nkv + kvh) * unit + tok_off[lane];
+        for (int d = wave; d < hd; d += 4) col[(size_t)d * RKV_TOK] = tile[lane * ld + d];
+    }
+}
+
 extern "C" int br_rope_kv_write(void* qkv, int is_bf16, const float* cs, const float* sn, const int* pos,
                                 const int* seq_of_token, const int* slots, const int* block_table,
                                 int table_stride, void* cache, int T, int nq, int nkv, int hd, int rd,
                                 int adjacent, int page, int write_cache, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || hd <= 0 || rd < 0 || rd > hd || (rd & 1) || page <= 0) return BR_BAD_ARG;
+    if (nq + 2 * nkv > 65535) return BR_BAD_ARG;
+    const bool vectors = is_bf16 && page == RKV_TOK && hd % 16 == 0 && rd % 16 == 0 &&
+                         ((uintptr_t)qkv | (uintptr_t)cache | (uintptr_t)cs | (uintptr_t)sn) % 16 == 0;
+    if (vectors && T >= 32) {
+        dim3 grid((T + RKV_TOK - 1) / RKV_TOK, nq + 2 * nkv);
+        const size_t lds = (size_t)RKV_TOK * (hd + 2) * sizeof(bf16);
+        rope_kv_write_tile_kernel<<<grid, 256, lds, s>>>((bf16*)qkv, cs, sn, pos, seq_of_token, slots, block_table,
+                                                        table_stride, (bf16*)cache, T, nq, nkv, hd, rd, adjacent,
+                                                        write_cache);
+        return br_check_launch();
+    }
     dim3 grid(T, nq + 2 * nkv);
     if (is_bf16)
         rope_kv_write_kernel<bf16><<<grid, 64, 0, s>>>((bf16*)qkv, cs, sn, pos, seq_of_token, slots,

@@ -183,12 +183,14 @@ def _rope_ref(x, pos, inv, adjacent):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("adjacent", [False, True])
-@pytest.mark.parametrize("nq,nkv,hd,rd", [(8, 2, 256, 64), (5, 5, 48, 48), (4, 1, 80, 80)])
-def test_rope_and_paged_write(dtype, adjacent, nq, nkv, hd, rd):
+@pytest.mark.parametrize("nq,nkv,hd,rd", [(8, 2, 256, 64), (5, 5, 48, 48), (4, 1, 80, 80), (3, 1, 40, 20)])
+@pytest.mark.parametrize("lens,starts", [([8, 128, 64], [0, 0, 32]), ([3, 17, 5], [0, 60, 32])])
+def test_rope_and_paged_write(dtype, adjacent, nq, nkv, hd, rd, lens, starts):
     # sizes of tests/mrope_test.rs:5-13 (nq 8, nkv 2, hd 256, rotary 64, theta 1e7) among them;
-    # page/offset cases of tests/op_kv_write_paged_batch_test.rs:196-198: starts 0 and 32, across pages
+    # page/offset cases of tests/op_kv_write_paged_batch_test.rs:196-198: starts 0 and 32, across pages.
+    # Many tokens in bf16 with sizes in steps of 16 take the kernel that works on 64 tokens at a time,
+    # everything else the one that takes a token at a time.
     page, theta = 64, 1e7
-    lens, starts = [8, 128, 64], [0, 0, 32]
     T = sum(lens)
     pos = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int().to(DEV)
     sot = torch.cat([torch.full((n,), b) for b, n in enumerate(lens)]).int().to(DEV)
