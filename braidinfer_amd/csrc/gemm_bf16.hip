@@ -560,8 +560,9 @@ static int launch_skinny(const bf16* A, const bf16* W, void* C, int M, int N, in
 #define SLAB_K 512
 template <int MB, int RB, int MODE>
 __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
-                                                              void* __restrict__ C, int M, int N, int K,
-                                                              size_t lda, size_t ldc) {
+                                                              void* __restrict__ C_, int M, int N, int K,
+                                                              size_t lda, size_t ldc, int slabs_per_part,
+                                                              size_t part_stride) {
     constexpr int ROWS = 16 * RB, COLS = 16 * MB;
     constexpr int SLAB_BYTES = COLS * SLAB_K * 2;
     constexpr int RED_BYTES = 4 * ROWS * (COLS + 1) * 4;
@@ -583,8 +584,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const bf16* __rest
         if (row > N - 1) row = N - 1;
         wp[i] = W + (size_t)row * K + wave * 128 + g * 8;
     }
+    // blockIdx.y: which run of k-slabs this workgroup sums (one run, or the parts of a split
+    // product, each into its own float matrix `part_stride` elements on)
     const int nslab = (K + SLAB_K - 1) / SLAB_K;
-    for (int sl = 0; sl < nslab; ++sl) {
+    const int sl0 = blockIdx.y * slabs_per_part;
+    const int sl1 = sl0 + slabs_per_part < nslab ? sl0 + slabs_per_part : nslab;
+    void* C = MODE == OUT_F32 ? (void*)((float*)C_ + blockIdx.y * part_stride) : C_;
+    for (int sl = sl0; sl < sl1; ++sl) {
         const int k0 = sl * SLAB_K;
         bf16x8 fw[RB][4];                                  // this wave's weight fragments of the slab
 #pragma unroll
@@ -655,11 +661,61 @@ template <int MB, int RB>
 static int launch_skinny_lds(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                              int mode, hipStream_t s) {
     const unsigned grid = (unsigned)((N + 16 * RB - 1) / (16 * RB));
-    if (mode == OUT_BF16) gemm_skinny_lds_kernel<MB, RB, OUT_BF16><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
-    else if (mode == OUT_F32) gemm_skinny_lds_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
-    else if (mode == OUT_F32_ACC) gemm_skinny_lds_kernel<MB, RB, OUT_F32_ACC><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
-    else gemm_skinny_lds_kernel<MB, RB, OUT_SWIGLU><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc);
+    const int nslab = (K + SLAB_K - 1) / SLAB_K;
+    if (mode == OUT_BF16) gemm_skinny_lds_kernel<MB, RB, OUT_BF16><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, nslab, 0);
+    else if (mode == OUT_F32) gemm_skinny_lds_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, nslab, 0);
+    else if (mode == OUT_F32_ACC) gemm_skinny_lds_kernel<MB, RB, OUT_F32_ACC><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, nslab, 0);
+    else gemm_skinny_lds_kernel<MB, RB, OUT_SWIGLU><<<grid, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, nslab, 0);
     return br_check_launch();
+}
+
+// ---------------------------------------------------------------- split product ------
+// 16 < M <= 64 and so few weight rows that 64-row workgroups would leave most of the chip
+// idle (N = 4096: 64 of them): the k-slabs are cut into `parts` runs, every (tile, run)
+// workgroup writes its sums to a float matrix of its own in `scratch`, and a second kernel
+// adds the runs in run order and applies the epilogue.  Nothing is added atomically: the
+// result does not depend on which workgroup finishes first.
+template <int MODE>
+__global__ void gemm_split_sum_kernel(const float* __restrict__ part, int parts, size_t part_stride, void* __restrict__ C,
+                                      int M, int N, size_t ldc) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)M * N) return;
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += part[p * part_stride + i];
+    const size_t m = i / N, n = i - m * N;
+    store_out<MODE>(C, m * ldc + n, v);
+}
+
+template <int MB>
+static int launch_split(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc, int mode,
+                        int parts, float* scratch, hipStream_t s) {
+    constexpr int RB = 4;
+    const int nslab = (K + SLAB_K - 1) / SLAB_K;
+    const int spp = (nslab + parts - 1) / parts;
+    parts = (nslab + spp - 1) / spp;                                   // no empty run
+    const size_t stride = (size_t)M * N;
+    dim3 grid((unsigned)((N + 16 * RB - 1) / (16 * RB)), (unsigned)parts);
+    gemm_skinny_lds_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, spp, stride);
+    int rc = br_check_launch();
+    if (rc != BR_OK) return rc;
+    const unsigned blocks = (unsigned)((stride + 255) / 256);
+    if (mode == OUT_BF16) gemm_split_sum_kernel<OUT_BF16><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    else if (mode == OUT_F32) gemm_split_sum_kernel<OUT_F32><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    else gemm_split_sum_kernel<OUT_F32_ACC><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    return br_check_launch();
+}
+
+// How many runs of k-slabs a product of 16 < M <= 64 rows is cut into when the caller gives
+// scratch memory: enough (tile, run) workgroups of 64 weight rows for the chip, at least two
+// slabs a run; 1 = not split.
+static int split_parts(int M, int N, int K, int mode, size_t scratch_bytes) {
+    if (M <= 16 || M > 64 || mode == OUT_SWIGLU) return 1;
+    const int tiles = (N + 63) / 64, nslab = (K + SLAB_K - 1) / SLAB_K;
+    int parts = 256 / tiles;
+    if (parts > nslab / 2) parts = nslab / 2;
+    if (parts > 8) parts = 8;
+    if (parts < 2 || (size_t)parts * M * N * sizeof(float) > scratch_bytes) return 1;
+    return parts;
 }
 
 // ------------------------------------------------------------------ gemm_stream ------
@@ -854,8 +910,10 @@ static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, in
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
 // rows); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
 // of registers in three of the four epilogues and was no faster in the fourth.)
+// `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
+// weight rows be split along k (see gemm_split_sum_kernel); BR_GEMM_SCRATCH_BYTES always suffices.
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
-                               size_t ldc, int mode, int kernel, hipStream_t s) {
+                               size_t ldc, int mode, int kernel, void* scratch, size_t scratch_bytes, hipStream_t s) {
     if (M <= 0 || N <= 0) return BR_OK;
     if (K <= 0 || lda < (size_t)K || mode < 0 || mode > 3) return BR_BAD_ARG;
     if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
@@ -878,9 +936,14 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
         const bool wide = N >= 16384;
         if (M <= 16) return (wide && M > 4) ? launch_skinny<1, 1, 2, 8>(A, W, C, M, N, K, lda, ldc, mode, s)
                                             : launch_skinny<1, 1, 4, 8>(A, W, C, M, N, K, lda, ldc, mode, s);
+        const int parts = (scratch && (uintptr_t)scratch % 16 == 0) ? split_parts(M, N, K, mode, scratch_bytes) : 1;
+        if (parts > 1)
+            return M <= 32 ? launch_split<2>(A, W, C, M, N, K, lda, ldc, mode, parts, (float*)scratch, s)
+                           : launch_split<4>(A, W, C, M, N, K, lda, ldc, mode, parts, (float*)scratch, s);
         if (M <= 32) return wide ? launch_skinny_lds<2, 4>(A, W, C, M, N, K, lda, ldc, mode, s)
                                  : launch_skinny_lds<2, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
-        if (wide) return launch_skinny_lds<4, 4>(A, W, C, M, N, K, lda, ldc, mode, s);
+        if (wide) return dma_ok ? launch_tile_dma<64, 128, 1, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                : launch_skinny_lds<4, 4>(A, W, C, M, N, K, lda, ldc, mode, s);
         return (N >= 6144) ? launch_skinny_lds<4, 2>(A, W, C, M, N, K, lda, ldc, mode, s)
                            : launch_skinny_lds<4, 1>(A, W, C, M, N, K, lda, ldc, mode, s);
     }
@@ -890,5 +953,5 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
 
 extern "C" int br_gemm_bf16(const void* A, const void* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                             int mode, hipStream_t s) {
-    return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, s);
+    return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, nullptr, 0, s);
 }

@@ -165,7 +165,11 @@ def convert(a: torch.Tensor, out: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------------ GEMM ------
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, kernel: int = 0) -> None:
+GEMM_SCRATCH_FLOATS = 8 * 64 * 8192      # room for every product that the bf16 kernels split along k
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, kernel: int = 0,
+         scratch: Optional[torch.Tensor] = None) -> None:
     """out[M, N] (+)= a[M, K] @ w[N, K]^T.
 
     float32 a and w: the true 32-bit kernel (out float32).  bfloat16 a and w: the
@@ -176,6 +180,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     registers, any shape; 3: skinny, M <= 64; 4, 5, 6: 256x128, 128x256 and 128x128 tiles
     loaded straight into LDS, K in steps of 64; 7: streaming by workgroups that stay, M <= 16
     and K in steps of 128 from 1024); 0 chooses by shape.
+    `scratch` (float32, on the device): with it, a bf16 product of 17 to 64 rows with few
+    weight rows is cut along k into runs that are summed in a fixed order by a second kernel.
     """
     name = "gemm"
     for t in (a, w, out):
@@ -199,8 +205,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             mode = 2 if accumulate else 1
         else:
             raise KernelError(f"gemm: output dtype {out.dtype}")
-        f = _fn("gemm_bf16", "br_gemm_bf16_ex", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P])
-        _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, mode, kernel, _stream()), name)
+        if scratch is not None:
+            _req(scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous(), "gemm: scratch must be float32 on the device")
+        f = _fn("gemm_bf16", "br_gemm_bf16_ex",
+                [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, _P])
+        _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, mode, kernel, _ptr(scratch),
+                 0 if scratch is None else scratch.numel() * 4, _stream()), name)
     else:
         raise KernelError(f"gemm: a is {a.dtype} and w is {w.dtype}; both float32 or both bfloat16")
 
@@ -217,8 +227,9 @@ def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: 
     _req(N % 16 == 0 and w_gu.shape[1] == K and out.shape == (M, N // 2), "gemm_swiglu: shapes")
     _req(w_gu.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1, "gemm_swiglu: rows must be dense")
     lda, ldc = (a.stride(0) if M > 1 else K), (out.stride(0) if M > 1 else N // 2)
-    f = _fn("gemm_bf16", "br_gemm_bf16_ex", [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P])
-    _check(f(_ptr(a), _ptr(w_gu), _ptr(out), M, N, K, lda, ldc, 3, kernel, _stream()), "gemm_swiglu")
+    f = _fn("gemm_bf16", "br_gemm_bf16_ex",
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, _P])
+    _check(f(_ptr(a), _ptr(w_gu), _ptr(out), M, N, K, lda, ldc, 3, kernel, None, 0, _stream()), "gemm_swiglu")
 
 
 def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:

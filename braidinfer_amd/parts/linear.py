@@ -19,7 +19,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, ws, accumulate: 
                 K.gemm(a, w, tmp)
                 K.convert(tmp, out)
                 return
-            K.gemm(a, w, out, accumulate)
+            scratch = None
+            if a.dtype == torch.bfloat16 and 16 < a.shape[0] <= 64:
+                scratch = ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32)
+            K.gemm(a, w, out, accumulate, scratch=scratch)
             return
     if w.dtype == torch.float32 and a.dtype == torch.bfloat16:
         a32 = ws.get("linear_in32", a.shape, torch.float32)

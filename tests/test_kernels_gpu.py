@@ -141,6 +141,31 @@ def test_gemm_streaming_kernel_rows_and_strides():
         K.gemm(rnd(4, 960, dtype=torch.bfloat16), rnd(N, 960, dtype=torch.bfloat16), torch.empty(4, N, device=DEV), kernel=7)
 
 
+@pytest.mark.parametrize("M,N,Kd", [(17, 520, 1536), (40, 300, 4096), (64, 4096, 2048), (33, 1000, 1032), (64, 96, 8192)])
+def test_gemm_split_along_k_with_scratch(M, N, Kd):
+    a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
+    want = a.double() @ w.double().T
+    scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
+    o32 = torch.empty(M, N, device=DEV)
+    K.gemm(a, w, o32, scratch=scratch)
+    assert (o32.double() - want).abs().max() < 1e-4 * want.abs().max()
+    again = torch.empty(M, N, device=DEV)
+    K.gemm(a, w, again, scratch=scratch)
+    assert torch.equal(again, o32)                                   # the runs are added in a fixed order
+    o16 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    K.gemm(a, w, o16, scratch=scratch)
+    assert (o16.double() - want).abs().max() < 1e-2 * want.abs().max()
+    base = rnd(M, N + 6, seed=3)
+    acc = base.clone()
+    K.gemm(a, w, acc[:, 3:3 + N], accumulate=True, scratch=scratch)
+    assert (acc[:, 3:3 + N].double() - (base[:, 3:3 + N].double() + want)).abs().max() < 1e-4 * want.abs().max()
+    assert torch.equal(acc[:, :3], base[:, :3]) and torch.equal(acc[:, 3 + N:], base[:, 3 + N:])
+    # too little scratch: the product is not split, and is right all the same
+    small = torch.empty(16, device=DEV)
+    K.gemm(a, w, again, scratch=small)
+    assert (again.double() - want).abs().max() < 1e-4 * want.abs().max()
+
+
 def test_gemm_reference_vectors():
     # tests/wmma_gemm_test.rs:27-69,72-114: sin/cos ramps times 0.5 / 0.3, tol 1e-3
     for M, N, Kd in ((32, 32, 64), (256, 256, 1024)):
