@@ -372,7 +372,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
 // workgroup writes the output; otherwise it writes (m, l, unnormalised O) for its split
 // and attn_decode_combine_kernel adds the splits in split order.  NB = ceil(hd / 32).
 template <int NB>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NB <= 4 ? 3 : 1, NB <= 4 ? 3 : 2))) void attn_decode_kernel(
     const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ slots,
     const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
     const bf16* __restrict__ cache, int nq, int nkv, int hd, int window, float scale, int nsplit,
