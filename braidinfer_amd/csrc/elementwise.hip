@@ -300,7 +300,7 @@ extern "C" int br_rope_kv_write(void* qkv, int is_bf16, const float* cs, const f
     if (nq + 2 * nkv > 65535) return BR_BAD_ARG;
     const bool vectors = is_bf16 && page == RKV_TOK && hd % 16 == 0 && rd % 16 == 0 &&
                          ((uintptr_t)qkv | (uintptr_t)cache | (uintptr_t)cs | (uintptr_t)sn) % 16 == 0;
-    if (vectors && T >= 32) {
+    if (vectors && T >= 256) {             // fewer tokens: one workgroup per token and head fills the chip better
         dim3 grid((T + RKV_TOK - 1) / RKV_TOK, nq + 2 * nkv);
         const size_t lds = (size_t)RKV_TOK * (hd + 2) * sizeof(bf16);
         rope_kv_write_tile_kernel<<<grid, 256, lds, s>>>((bf16*)qkv, cs, sn, pos, seq_of_token, slots, block_table,

@@ -209,7 +209,7 @@ def _rope_ref(x, pos, inv, adjacent):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("adjacent", [False, True])
 @pytest.mark.parametrize("nq,nkv,hd,rd", [(8, 2, 256, 64), (5, 5, 48, 48), (4, 1, 80, 80), (3, 1, 40, 20)])
-@pytest.mark.parametrize("lens,starts", [([8, 128, 64], [0, 0, 32]), ([3, 17, 5], [0, 60, 32])])
+@pytest.mark.parametrize("lens,starts", [([8, 128, 64], [0, 0, 32]), ([70, 128, 100], [0, 0, 32]), ([3, 17, 5], [0, 60, 32])])
 def test_rope_and_paged_write(dtype, adjacent, nq, nkv, hd, rd, lens, starts):
     # sizes of tests/mrope_test.rs:5-13 (nq 8, nkv 2, hd 256, rotary 64, theta 1e7) among them;
     # page/offset cases of tests/op_kv_write_paged_batch_test.rs:196-198: starts 0 and 32, across pages.
@@ -222,6 +222,7 @@ def test_rope_and_paged_write(dtype, adjacent, nq, nkv, hd, rd, lens, starts):
     slots = i32([2, 0, 3])
     table = torch.full((4, 4), -1, dtype=torch.int32)
     table[2, 0], table[0, 0], table[0, 1], table[3, 0], table[3, 1] = 5, 1, 6, 0, 3
+    table[2, 1], table[3, 2] = 2, 4
     table = table.to(DEV)
     inv = (1.0 / theta ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd)).to(DEV)
     cs, sn = torch.empty(T, rd // 2, device=DEV), torch.empty(T, rd // 2, device=DEV)
