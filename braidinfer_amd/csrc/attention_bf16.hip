@@ -523,6 +523,199 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NB <= 4 ? 3
     }
 }
 
+// The same through LDS, for head sizes 64 and 128.  The workgroup brings whole pages of its
+// kv head (keys 64 x hd, values hd x 64: two contiguous blocks) into a ring of S stages
+// with direct global-to-LDS loads, 1 KB per wave-load, the next pages in flight while one
+// is multiplied; one barrier per page.  The 4 waves share a page as (key half, dim half):
+// a wave computes the scores of its 32 keys (both waves of a key half do, and get the same
+// m and l) and the output of its hd / 2 dims; the two key halves of a dim half are merged
+// in LDS at the end, first half first.  16-byte columns are XOR-swizzled by the row so that
+// operand reads spread over the banks; the swizzle is applied by the choice of the global
+// column a lane fetches.
+__device__ __forceinline__ int kswz(int row, int cols) {      // the 16 key rows of a score block differ in bits 0,1,3,4
+    return cols == 16 ? (((row >> 3) & 3) * 4 + (row & 3)) : (((row >> 3) & 1) * 4 + (row & 3));
+}
+
+#define DEC_MAX_RUN 1024      // pages of one workgroup's run whose numbers are kept in LDS
+
+template <int HD, int S>
+__global__ __launch_bounds__(256) void attn_decode_lds_kernel(
+    const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ slots,
+    const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
+    const bf16* __restrict__ cache, int nq, int nkv, int window, float scale, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    constexpr int NB = HD / 32;                      // 32-wide k-steps of the score product
+    constexpr int KROWB = HD * 2, KCOLS = KROWB / 16; // a key row in bytes, in 16-byte columns
+    constexpr int KB = PAGE * KROWB, STAGE = 2 * KB;  // keys, then values [HD][128 bytes]
+    constexpr int KINSTR = KB / 1024, NDMA = STAGE / 1024 / 4;   // wave-loads: of the keys; per wave and page
+    constexpr int KROWS = 1024 / KROWB;              // key rows per wave-load
+    constexpr int OB = HD / 2 / 16;                  // 16-dim output blocks of a wave
+    constexpr int D = S - 1;
+    static_assert(S >= 2 && S <= 4 && (D - 1) * NDMA <= 63, "ring");
+    extern __shared__ __attribute__((aligned(1024))) unsigned char dsm[];
+    int* bts = (int*)(dsm + S * STAGE);
+    const int G = nq / nkv, nhb = (G + 15) / 16;
+    const int split = blockIdx.x, kvh = blockIdx.y / nhb, hb = blockIdx.y % nhb, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int kh = wave & 1, dh = wave >> 1;
+    const int nheads = (G - hb * 16 < 16) ? G - hb * 16 : 16;
+    const int head0 = kvh * G + hb * 16;
+    const int slot = slots[b];
+    const int ctx = slot < 0 ? 0 : ctx_lens[b];
+    int lo = 0;
+    if (window > 0 && ctx - window > 0) lo = ctx - window;
+    const int pg_lo = lo / PAGE, npg = ctx > 0 ? (ctx - 1) / PAGE - pg_lo + 1 : 0;
+    const int pps = (npg + nsplit - 1) / nsplit;
+    const int pg_begin = pg_lo + split * pps;
+    int pg_end = pg_begin + pps;
+    if (pg_end > pg_lo + npg) pg_end = pg_lo + npg;
+    const int n_run = pg_end > pg_begin ? pg_end - pg_begin : 0;          // at most DEC_MAX_RUN (the launcher checks)
+
+    const int* bt = block_table + (size_t)(slot < 0 ? 0 : slot) * table_stride;
+    for (int i = tid; i < n_run; i += 256) bts[i] = bt[pg_begin + i];
+    const bool head_ok = c < nheads;
+    const bf16* qrow = q + (size_t)b * q_stride + (size_t)(head0 + (head_ok ? c : 0)) * HD;
+    bf16x8 qf[NB];
+#pragma unroll
+    for (int s = 0; s < NB; ++s) qf[s] = head_ok ? *(const bf16x8*)(qrow + s * 32 + 8 * g) : zero8();
+    // the query has arrived before the loop: a wait for it inside would also wait for the pages in flight
+#pragma unroll
+    for (int s = 0; s < NB; ++s) asm volatile("" ::"v"(qf[s]));
+    __syncthreads();
+
+    const size_t page_elems = (size_t)2 * nkv * PAGE * HD;
+    const size_t k_off = (size_t)kvh * PAGE * HD, v_off = ((size_t)nkv + kvh) * PAGE * HD;
+    const unsigned ring_lds = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)dsm);
+#define DEC_ISSUE(I)                                                                                         \
+    do {                                                                                                     \
+        const bf16* pg_ = cache + (size_t)bts[I] * page_elems;                                               \
+        _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                \
+            const int in_ = wave * NDMA + q_;                                                                \
+            const bf16* gp_;                                                                                 \
+            if (in_ < KINSTR) {                                                                              \
+                const int row_ = in_ * KROWS + lane / KCOLS;                                                 \
+                gp_ = pg_ + k_off + (size_t)row_ * HD + (((lane % KCOLS) ^ kswz(row_, KCOLS)) * 8);          \
+            } else {                                                                                         \
+                const int row_ = (in_ - KINSTR) * 8 + (lane >> 3);                                           \
+                gp_ = pg_ + v_off + (size_t)row_ * PAGE + (((lane & 7) ^ ((row_ >> 1) & 7)) * 8);            \
+            }                                                                                                \
+            const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + ((I) % S) * STAGE + in_ * 1024); \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
+        }                                                                                                    \
+    } while (0)
+
+    f32x4 acc_o[OB];
+#pragma unroll
+    for (int i = 0; i < OB; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc_o[i][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+    const float scale2 = scale * LOG2E;
+
+    for (int j = 0; j < D; ++j)
+        if (j < n_run) DEC_ISSUE(j);
+    for (int i = 0; i < n_run; ++i) {
+        // page i has landed when at most the loads of the pages after it are in flight
+        int after = n_run - 1 - i;
+        if (after > D - 1) after = D - 1;
+        if (after >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NDMA) : "memory");
+        else if (after == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                 // every wave's part of page i is there; page i - 1 is done with
+        asm volatile("" ::: "memory");
+        if (i + D < n_run) DEC_ISSUE(i + D);
+        const unsigned char* st = dsm + (i % S) * STAGE;
+        const int kb = (pg_begin + i) * PAGE + 32 * kh;        // position of this wave's first key
+        if (kb >= ctx || kb + 32 <= lo) continue;
+        f32x4 s_acc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s_acc[j][r] = 0.f;
+            // row c of score block j stands for key 8 (c / 4) + 4 j + c % 4 of the 32
+            const int row = 32 * kh + 8 * (c >> 2) + 4 * j + (c & 3);
+#pragma unroll
+            for (int s = 0; s < NB; ++s) {
+                const bf16x8 kf = *(const bf16x8*)(st + row * KROWB + (((4 * s + g) ^ kswz(row, KCOLS)) * 16));
+                s_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s_acc[j], 0, 0, 0);
+            }
+        }
+        // s_acc[j][r]: key kb + 8 g + 4 j + r, head = this lane's column
+        float sv[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int key = kb + 8 * g + e;
+            const bool ok = key >= lo && key < ctx;
+            sv[e] = ok ? s_acc[e >> 2][e & 3] * scale2 : -INFINITY;
+            mx = fmaxf(mx, sv[e]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);             // finite: the block holds at least one visible key
+        const float corr = fast_exp2(m - m_new);
+        float psum = 0.f;
+        bf16x8 pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = fast_exp2(sv[e] - m_new);
+            psum += p;
+            pf[e] = (bf16)p;
+        }
+        lsum = lsum * corr + psum;
+        m = m_new;
+        const bool tail = kb + 32 > ctx;              // values beyond the context are stale: read them as zero
+#pragma unroll
+        for (int i2 = 0; i2 < OB; ++i2) {
+            const int row = dh * (HD / 2) + 16 * i2 + c;
+            bf16x8 vf = *(const bf16x8*)(st + KB + row * 128 + (((4 * kh + g) ^ ((row >> 1) & 7)) * 16));
+            if (tail) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) if (kb + 8 * g + e >= ctx) vf[e] = (bf16)0.f;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc_o[i2][r] *= corr;
+            acc_o[i2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc_o[i2], 0, 0, 0);
+        }
+    }
+#undef DEC_ISSUE
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
+    __syncthreads();                                  // the ring is free: the waves' results meet in it
+    // per wave: O [16 heads][HD / 2], then m [16], l [16]
+    constexpr int WST = 16 * (HD / 2) + 32;
+    float* lds = (float*)dsm;
+    float* my = lds + wave * WST;
+#pragma unroll
+    for (int i2 = 0; i2 < OB; ++i2)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) my[c * (HD / 2) + 16 * i2 + 4 * g + r] = acc_o[i2][r];    // dim 16 i2 + 4 g + r of the half, head c
+    if (g == 0) { my[16 * (HD / 2) + c] = m; my[16 * (HD / 2) + 16 + c] = lsum; }
+    __syncthreads();
+    for (int e = tid; e < nheads * HD; e += 256) {
+        const int h = e / HD, d = e - h * HD;
+        const int w0 = 2 * (d / (HD / 2)), dd = d % (HD / 2);          // the dim half's waves: key halves 0 and 1
+        const float m0 = lds[w0 * WST + 16 * (HD / 2) + h], m1 = lds[(w0 + 1) * WST + 16 * (HD / 2) + h];
+        const float M = fmaxf(m0, m1);
+        float L = 0.f, O = 0.f;
+        if (M > -INFINITY) {
+            const float f0 = fast_exp2(m0 - M), f1 = fast_exp2(m1 - M);
+            L = lds[w0 * WST + 16 * (HD / 2) + 16 + h] * f0 + lds[(w0 + 1) * WST + 16 * (HD / 2) + 16 + h] * f1;
+            O = lds[w0 * WST + h * (HD / 2) + dd] * f0 + lds[(w0 + 1) * WST + h * (HD / 2) + dd] * f1;
+        }
+        const int head = head0 + h;
+        if (nsplit == 1) {
+            out[((size_t)b * nq + head) * HD + d] = (bf16)(L > 0.f ? O / L : 0.f);
+        } else {
+            const size_t pidx = ((size_t)b * nq + head) * nsplit + split;
+            part_o[pidx * HD + d] = O;
+            if (d == 0) { part_ml[pidx * 2] = M; part_ml[pidx * 2 + 1] = L; }
+        }
+    }
+}
+
 // grid = (nq, sequences), block = 64: add the splits in split order
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml,
@@ -601,11 +794,13 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
     return br_check_launch();
 }
 
+
 // part_o: float [B, nq, nsplit, hd]; part_ml: float [B, nq, nsplit, 2] (unused when nsplit == 1)
 extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, const int* slots,
                                    const int* ctx_lens, const int* block_table, int table_stride,
                                    const void* cache, int B, int nq, int nkv, int hd, int page, int window,
-                                   float scale, int nsplit, float* part_o, float* part_ml, hipStream_t s) {
+                                   float scale, int nsplit, float* part_o, float* part_ml, int variant,
+                                   hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
         q_stride % 8 || ((uintptr_t)q % 16) || nsplit < 1 || nsplit > 1024 || B > 65535 ||
@@ -614,6 +809,40 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
     const int G = nq / nkv, nhb = (G + 15) / 16;
     if ((long long)nkv * nhb > 65535) return BR_BAD_ARG;
     dim3 grid(nsplit, nkv * nhb, B);
+    // variant 0: choose; 1: fragments straight from the cache; 2: pages through a ring in LDS
+    // (head sizes 64 and 128, runs of at most DEC_MAX_RUN pages)
+    const bool lds_ok = (hd == 64 || hd == 128) && (table_stride + nsplit - 1) / nsplit <= DEC_MAX_RUN &&
+                        (uintptr_t)cache % 16 == 0;
+    if (variant < 0 || variant > 2 || (variant == 2 && !lds_ok)) return BR_BAD_ARG;
+    if (variant == 0) variant = lds_ok ? 2 : 1;
+    if (variant == 2) {
+        // two stages leave room for two workgroups per CU; with at most one workgroup per CU
+        // a third stage keeps two pages in flight instead (measured: 34 -> 32 us at 8 x 4096 tokens)
+        const int cus = br_device_cus();
+        const bool deep = cus > 0 && (long long)nsplit * nkv * nhb * B <= cus;
+#define BR_DECODE_LDS(HD_, S_)                                                                                  \
+    do {                                                                                                        \
+        auto kern = attn_decode_lds_kernel<HD_, S_>;                                                            \
+        constexpr size_t lds2 = (size_t)S_ * 2 * PAGE * HD_ * 2 + DEC_MAX_RUN * sizeof(int);                    \
+        static bool set = false;                                                                                \
+        if (!set) {                                                                                             \
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2)   \
+                != hipSuccess)                                                                                  \
+                return BR_LAUNCH_FAILED;                                                                        \
+            set = true;                                                                                         \
+        }                                                                                                       \
+        kern<<<grid, 256, lds2, s>>>((const bf16*)q, q_stride, (bf16*)out, slots, ctx_lens, block_table,        \
+                                     table_stride, (const bf16*)cache, nq, nkv, window, scale, nsplit, part_o,  \
+                                     part_ml);                                                                  \
+    } while (0)
+        if (hd == 128) { if (deep) BR_DECODE_LDS(128, 3); else BR_DECODE_LDS(128, 2); }
+        else { if (deep) BR_DECODE_LDS(64, 3); else BR_DECODE_LDS(64, 2); }
+#undef BR_DECODE_LDS
+        int rc2 = br_check_launch();
+        if (rc2 != BR_OK || nsplit == 1) return rc2;
+        attn_decode_combine_kernel<<<dim3(nq, B), 64, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
+        return br_check_launch();
+    }
     const size_t lds = (size_t)4 * (16 * hd + 32) * sizeof(float);
 #define BR_DECODE(N)                                                                                        \
     do {                                                                                                    \

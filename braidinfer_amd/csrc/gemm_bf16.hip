@@ -862,17 +862,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 }
 
 
-static int device_cus() {
-    static int cus[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (!cus[dev]) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
-        cus[dev] = n;
-    }
-    return cus[dev];
-}
 
 #define STREAM_KC 128
 #define STREAM_NW 8
@@ -880,7 +869,7 @@ template <int XR>
 static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                          int mode, hipStream_t s) {
     constexpr int RT = 16, KC = STREAM_KC, S = 2, NW = STREAM_NW;
-    const int cus = device_cus();
+    const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
     const int ntiles = (N + RT - 1) / RT;
     const int grid = ntiles < cus ? ntiles : cus;

@@ -282,8 +282,11 @@ def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu
 def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slots: torch.Tensor,
                           ctx_lens: torch.Tensor, block_table: torch.Tensor, cache: torch.Tensor, B: int,
                           nq: int, nkv: int, hd: int, page: int, window: Optional[int], scale: float,
-                          nsplit: int, part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor]) -> None:
-    """Attention of one new token per sequence over its pages, cut into `nsplit` runs."""
+                          nsplit: int, part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
+                          variant: int = 0) -> None:
+    """Attention of one new token per sequence over its pages, cut into `nsplit` runs.
+    `variant` forces a kernel: 1 reads operands straight from the cache, 2 brings pages
+    through a ring in LDS (head sizes 64 and 128); 0 chooses."""
     _dev("attention_decode_bf16", out, slots, ctx_lens, block_table, cache, part_o, part_ml)
     _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
          "attention_decode_bf16: bfloat16 only")
@@ -296,10 +299,10 @@ def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slo
              and part_ml is not None and part_ml.numel() >= B * nq * nsplit * 2,
              "attention_decode_bf16: scratch for the splits is too small")
     f = _fn("attention_bf16", "br_attn_decode_bf16",
-            [_P, c_size_t, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, c_int, _P, _P, _P])
+            [_P, c_size_t, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, c_int, _P, _P, c_int, _P])
     _check(f(_ptr(q), q_stride, _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1],
              _ptr(cache), B, nq, nkv, hd, page, int(window or 0), float(scale), nsplit, _ptr(part_o),
-             _ptr(part_ml), _stream()), "attention_decode_bf16")
+             _ptr(part_ml), int(variant), _stream()), "attention_decode_bf16")
 
 
 # -------------------------------------------------------------------- sampling -----

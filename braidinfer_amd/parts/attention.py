@@ -26,13 +26,15 @@ from .linear import fuse_rows, linear
 
 def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
     """Into how many runs a sequence's pages are cut for single-token steps: about one
-    workgroup per CU (measured: more runs cost more in the combine than they gain), at least
-    two pages per run.  It depends
-    on the step's shape only (batch and an upper bound of the context), never on the
-    tokens."""
+    workgroup per CU (measured: more runs cost more in the combine than they gain) and at
+    least two pages per run; beyond that, runs of at most 64 pages.  It depends on the
+    step's shape only (batch and an upper bound of the context), never on the tokens."""
     pages = max(1, -(-max_ctx // page))
     want = -(-256 // max(1, batch * nkv))
-    return max(1, min(want, pages // 2 if pages >= 2 else 1, 64))
+    n = max(1, min(want, pages // 2 if pages >= 2 else 1, 64))
+    while n < 64 and pages > 64 * n:
+        n *= 2
+    return n
 
 
 class GQAAttention(Mixer):
