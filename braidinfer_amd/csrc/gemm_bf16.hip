@@ -894,10 +894,216 @@ static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, in
     return br_check_launch();
 }
 
+// ------------------------------------------------------------- gemm_stream_wide ------
+// 16 < M <= 64, K in steps of 128: the same streaming by workgroups that stay, with the
+// activations shared.  A unit of work is a tile of 64 weight rows over one run of k-chunks
+// (the whole K, or one of `parts` runs when the tiles alone would be too few for the chip);
+// unit u of workgroup b is b + u * grid.  A stage of the workgroup's LDS ring holds one
+// 128-wide chunk of the tile (64 rows) and of the activations (16 MB rows), brought by all
+// 8 waves with direct global-to-LDS loads, two chunks ahead; one barrier per chunk.  Wave w
+// multiplies weight rows 16 (w % 4) .. + 16 with k-steps 2 (w / 4), 2 (w / 4) + 1 of the
+// chunk; the two k-halves are added in LDS at the unit's end.  With `parts` > 1 the unit's
+// float sums go to a matrix of its run (`part_stride` elements apart) for
+// gemm_split_sum_kernel; else the epilogue is applied here.
+#define WIDE_S 3
+template <int MB, int MODE, bool PARTIAL>
+__global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                               void* __restrict__ C, int M, int N, int K, size_t lda,
+                                                               size_t ldc, int ntiles, int parts, int cpp,
+                                                               size_t part_stride) {
+    constexpr int S = WIDE_S, D = S - 1, NW = 8;
+    constexpr int ROWS = 64 + 16 * MB;               // stacked rows of a stage: weights, then activations
+    constexpr int STAGE = ROWS * 256;
+    constexpr int NDMA = STAGE / 1024 / NW;          // wave-loads per wave and chunk
+    constexpr int RLD = 16 * MB + 1;
+    static_assert(STAGE % (1024 * NW) == 0 && (D - 1) * NDMA <= 63, "stage");
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    float* red = (float*)(smem + S * STAGE);         // [NW][16][RLD]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const int rb = wave & 3, khalf = wave >> 2;
+    const unsigned ring_lds = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)smem);
+    const int nch = K / 128;
+    const int nunits = ntiles * parts;
+    const int my_units = (nunits - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+
+    f32x4 acc[MB];
+#pragma unroll
+    for (int j = 0; j < MB; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // cursors over this workgroup's chunks in order: (unit, chunk of its run)
+    int is_u = 0, is_c = 0, cp_u = 0, cp_c = 0;
+    int issued = 0, done = 0;
+#define WIDE_RUN(U, C0, C1)                                                  \
+    const int part_##U = ((int)blockIdx.x + (U) * (int)gridDim.x) % parts;    \
+    const int C0 = part_##U * cpp;                                           \
+    const int C1 = C0 + cpp < nch ? C0 + cpp : nch;
+#define WIDE_ISSUE()                                                                                          \
+    do {                                                                                                      \
+        const int unit_ = (int)blockIdx.x + is_u * (int)gridDim.x;                                            \
+        const int tile_ = unit_ / parts, c0_ = (unit_ % parts) * cpp;                                         \
+        const int c1_ = c0_ + cpp < nch ? c0_ + cpp : nch;                                                    \
+        const int chunk_ = c0_ + is_c;                                                                        \
+        _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                 \
+            const int in_ = wave * NDMA + q_;                                                                 \
+            const int row_ = in_ * 4 + (lane >> 4);                                                           \
+            const bf16* gp_;                                                                                  \
+            if (row_ < 64) {                                                                                  \
+                int n_ = tile_ * 64 + row_;                                                                   \
+                if (n_ > N - 1) n_ = N - 1;                                                                   \
+                gp_ = W + (size_t)n_ * K;                                                                     \
+            } else {                                                                                          \
+                int m_ = row_ - 64;                                                                           \
+                if (m_ > M - 1) m_ = M - 1;                                                                   \
+                gp_ = A + (size_t)m_ * lda;                                                                   \
+            }                                                                                                 \
+            gp_ += (size_t)chunk_ * 128 + (((lane & 15) ^ (row_ & 7)) * 8);                                   \
+            const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + (issued % S) * STAGE + in_ * 1024); \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
+        }                                                                                                     \
+        ++issued;                                                                                             \
+        if (c0_ + ++is_c == c1_) { is_c = 0; ++is_u; }                                                        \
+    } while (0)
+
+    for (int j = 0; j < D; ++j)
+        if (is_u < my_units) WIDE_ISSUE();
+    while (cp_u < my_units) {
+        // the chunk to multiply has landed when at most the loads of the chunks issued after it are in flight
+        if (issued - done - 1 >= 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();            // every wave's part of it is there; the chunk before is done with
+        asm volatile("" ::: "memory");
+        if (is_u < my_units) WIDE_ISSUE();
+        const unsigned char* st = smem + (done % S) * STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int col = 4 * (2 * khalf + ks) + g;
+            const int wr = 16 * rb + r16;
+            const bf16x8 wf = *(const bf16x8*)(st + wr * 256 + ((col ^ (wr & 7)) * 16));
+#pragma unroll
+            for (int j = 0; j < MB; ++j) {
+                const int xr = 64 + 16 * j + r16;
+                const bf16x8 xv = *(const bf16x8*)(st + xr * 256 + ((col ^ (xr & 7)) * 16));
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xv, acc[j], 0, 0, 0);
+            }
+        }
+        ++done;
+        const int unit = (int)blockIdx.x + cp_u * (int)gridDim.x;
+        const int part = unit % parts, c0 = part * cpp;
+        const int c1 = c0 + cpp < nch ? c0 + cpp : nch;
+        if (c0 + ++cp_c < c1) continue;
+        // the unit's end: acc[j][r] is weight row 16 rb + 4 g + r of the tile, batch row 16 j + r16
+        cp_c = 0;
+        ++cp_u;
+        const int n0 = (unit / parts) * 64;
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[(wave * 16 + 4 * g + r) * RLD + 16 * j + r16] = acc[j][r];
+            acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();            // the next write to `red` comes after the next chunk's barrier
+        asm volatile("" ::: "memory");
+        if (MODE == OUT_SWIGLU && !PARTIAL) {
+            // blocks of 16 tile rows: 8 gates, then the 8 up values of the same outputs
+            for (int e = tid; e < 32 * 16 * MB; e += 512) {
+                const int m = e >> 5, jl = e & 31;
+                const int gr = (jl >> 3) * 16 + (jl & 7);
+                if (m < M && n0 + gr + 8 < N) {
+                    const float gv = red[gr * RLD + m] + red[(64 + gr) * RLD + m];
+                    const float uv = red[(gr + 8) * RLD + m] + red[(64 + gr + 8) * RLD + m];
+                    ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
+                }
+            }
+        } else {
+            for (int e = tid; e < 64 * 16 * MB; e += 512) {
+                const int m = e >> 6, nl = e & 63, n = n0 + nl;
+                if (m < M && n < N) {
+                    const float v = red[nl * RLD + m] + red[(64 + nl) * RLD + m];      // k-half 0, then 1
+                    if (PARTIAL) ((float*)C)[part * part_stride + (size_t)m * N + n] = v;
+                    else {
+                        const size_t idx = (size_t)m * ldc + n;
+                        if (MODE == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
+                        else if (MODE == OUT_F32) ((float*)C)[idx] = v;
+                        else unsafeAtomicAdd((float*)C + idx, v);     // one add per element, no read to wait for
+                    }
+                }
+            }
+        }
+    }
+#undef WIDE_ISSUE
+#undef WIDE_RUN
+}
+
+// Into how many runs of k-chunks the units of gemm_stream_wide are cut: the least time by a
+// simple count (rounds of units over the compute units, times the run's length, plus the
+// traffic of the partial sums), among 1, 2, 4 and 8 runs of at least 2 chunks.
+static int wide_parts(int M, int N, int K, int mode, int cus, size_t scratch_bytes) {
+    const int tiles = (N + 63) / 64, nch = K / 128;
+    int best = 1;
+    double best_cost = 1e30;
+    for (int parts = 1; parts <= 8; parts *= 2) {
+        if (parts > 1 && (mode == OUT_SWIGLU || parts * 2 > nch ||
+                          (size_t)parts * M * N * sizeof(float) > scratch_bytes))
+            break;
+        const int cpp = (nch + parts - 1) / parts;
+        const long long rounds = ((long long)tiles * parts + cus - 1) / cus;
+        double cost = (double)rounds * cpp;
+        if (parts > 1) cost *= 1.0 + 4.0 * parts * M / K;
+        if (cost < best_cost - 1e-9) { best_cost = cost; best = parts; }
+    }
+    return best;
+}
+
+template <int MB>
+static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                              int mode, float* scratch, size_t scratch_bytes, hipStream_t s) {
+    const int cus = br_device_cus();
+    if (!cus) return BR_LAUNCH_FAILED;
+    const int ntiles = (N + 63) / 64, nch = K / 128;
+    int parts = scratch ? wide_parts(M, N, K, mode, cus, scratch_bytes) : 1;
+    const int cpp = (nch + parts - 1) / parts;
+    parts = (nch + cpp - 1) / cpp;                                   // no empty run
+    const long long nunits = (long long)ntiles * parts;
+    const int grid = nunits < cus ? (int)nunits : cus;
+    constexpr size_t lds = (size_t)WIDE_S * (64 + 16 * MB) * 256 + 8 * 16 * (16 * MB + 1) * 4;
+    const size_t stride = (size_t)M * N;
+#define BR_WIDE(MODE_, PARTIAL_, OUT_)                                                                          \
+    do {                                                                                                        \
+        auto kern = gemm_stream_wide_kernel<MB, MODE_, PARTIAL_>;                                               \
+        static bool set = false;                                                                                \
+        if (!set) {                                                                                             \
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != \
+                hipSuccess)                                                                                     \
+                return BR_LAUNCH_FAILED;                                                                        \
+            set = true;                                                                                         \
+        }                                                                                                       \
+        kern<<<grid, 512, lds, s>>>(A, W, OUT_, M, N, K, lda, ldc, ntiles, parts, cpp, stride);                 \
+    } while (0)
+    if (parts > 1) {
+        BR_WIDE(OUT_F32, true, (void*)scratch);
+        int rc = br_check_launch();
+        if (rc != BR_OK) return rc;
+        const unsigned blocks = (unsigned)((stride + 255) / 256);
+        if (mode == OUT_BF16) gemm_split_sum_kernel<OUT_BF16><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+        else if (mode == OUT_F32) gemm_split_sum_kernel<OUT_F32><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+        else gemm_split_sum_kernel<OUT_F32_ACC><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+        return br_check_launch();
+    }
+    if (mode == OUT_BF16) BR_WIDE(OUT_BF16, false, C);
+    else if (mode == OUT_F32) BR_WIDE(OUT_F32, false, C);
+    else if (mode == OUT_F32_ACC) BR_WIDE(OUT_F32_ACC, false, C);
+    else BR_WIDE(OUT_SWIGLU, false, C);
+#undef BR_WIDE
+    return br_check_launch();
+}
+
 // kernel: 0 = choose, 1 = tile 128x128 through registers (any shape), 2 = the same 256x128,
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
-// rows); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
+// rows), 8 = stream wide (16 < M <= 64, K a multiple of 128); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
 // of registers in three of the four epilogues and was no faster in the fourth.)
 // `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
 // weight rows be split along k (see gemm_split_sum_kernel); BR_GEMM_SCRATCH_BYTES always suffices.
@@ -913,8 +1119,17 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     const bool dma_ok = aligned && K % DMA_BK == 0;
     const bool stream_ok = aligned && M <= 16 && K % STREAM_KC == 0 && K / STREAM_KC >= STREAM_NW;
     if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
-    if ((kernel == 7 && !stream_ok) || kernel > 7 || kernel < 0) return BR_BAD_ARG;
-    if (kernel == 0) kernel = stream_ok ? 7 : (aligned && M <= 64) ? 3 : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
+    const bool wide_ok = aligned && M > 16 && M <= 64 && K % 128 == 0 && K >= 256 &&
+                         (!scratch || (uintptr_t)scratch % 16 == 0);
+    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 8 || kernel < 0) return BR_BAD_ARG;
+    // measured at M = 64: many weight rows (gate/up) are 4 % faster through the 64x128 tile, which kernel 3 picks
+    if (kernel == 0)
+        kernel = stream_ok ? 7
+                 : (wide_ok && !(M > 32 && N >= 16384 && dma_ok)) ? 8
+                 : (aligned && M <= 64) ? 3 : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
+    if (kernel == 8)
+        return M <= 32 ? launch_stream_wide<2>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s)
+                       : launch_stream_wide<4>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s);
     if (kernel == 7) return M <= 8 ? launch_stream<8>(A, W, C, M, N, K, lda, ldc, mode, s)
                                    : launch_stream<16>(A, W, C, M, N, K, lda, ldc, mode, s);
     if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s);

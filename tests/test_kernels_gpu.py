@@ -67,7 +67,9 @@ SHAPES = [(1, 64, 64), (5, 100, 96), (17, 192, 320), (64, 301, 100), (33, 1000, 
           (65, 301, 64), (513, 260, 320),
           # few rows and a long k: what the streaming kernel takes (tiles beyond one per workgroup, a chunk
           # count that the waves do not share evenly)
-          (1, 100, 1024), (8, 301, 1152), (9, 48, 2048), (16, 4100, 1024), (3, 9000, 1280)]
+          (1, 100, 1024), (8, 301, 1152), (9, 48, 2048), (16, 4100, 1024), (3, 9000, 1280),
+          # 17 to 64 rows: what the wide streaming kernel takes
+          (17, 100, 256), (64, 16500, 384), (33, 301, 1152), (48, 4100, 1024)]
 
 
 def _skip_unless_kernel_takes(kernel, M, Kd):
@@ -77,6 +79,8 @@ def _skip_unless_kernel_takes(kernel, M, Kd):
         pytest.skip("the direct-to-LDS tile kernels take K in steps of 64")
     if kernel == 7 and (M > 16 or Kd % 128 or Kd < 1024):
         pytest.skip("the streaming kernel takes M <= 16 and K in steps of 128 from 1024")
+    if kernel == 8 and (M <= 16 or M > 64 or Kd % 128 or Kd < 256):
+        pytest.skip("the wide streaming kernel takes 16 < M <= 64 and K in steps of 128 from 256")
 
 
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
@@ -101,7 +105,7 @@ def test_gemm_f32_rows_do_not_depend_on_the_batch():
     assert torch.equal(one[0], full[33])
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
 def test_gemm_bf16(M, N, Kd, kernel):
     _skip_unless_kernel_takes(kernel, M, Kd)
@@ -141,28 +145,30 @@ def test_gemm_streaming_kernel_rows_and_strides():
         K.gemm(rnd(4, 960, dtype=torch.bfloat16), rnd(N, 960, dtype=torch.bfloat16), torch.empty(4, N, device=DEV), kernel=7)
 
 
+@pytest.mark.parametrize("kernel", [0, 3, 8])
 @pytest.mark.parametrize("M,N,Kd", [(17, 520, 1536), (40, 300, 4096), (64, 4096, 2048), (33, 1000, 1032), (64, 96, 8192)])
-def test_gemm_split_along_k_with_scratch(M, N, Kd):
+def test_gemm_split_along_k_with_scratch(M, N, Kd, kernel):
+    _skip_unless_kernel_takes(kernel, M, Kd)
     a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
     want = a.double() @ w.double().T
     scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
     o32 = torch.empty(M, N, device=DEV)
-    K.gemm(a, w, o32, scratch=scratch)
+    K.gemm(a, w, o32, scratch=scratch, kernel=kernel)
     assert (o32.double() - want).abs().max() < 1e-4 * want.abs().max()
     again = torch.empty(M, N, device=DEV)
-    K.gemm(a, w, again, scratch=scratch)
+    K.gemm(a, w, again, scratch=scratch, kernel=kernel)
     assert torch.equal(again, o32)                                   # the runs are added in a fixed order
     o16 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
-    K.gemm(a, w, o16, scratch=scratch)
+    K.gemm(a, w, o16, scratch=scratch, kernel=kernel)
     assert (o16.double() - want).abs().max() < 1e-2 * want.abs().max()
     base = rnd(M, N + 6, seed=3)
     acc = base.clone()
-    K.gemm(a, w, acc[:, 3:3 + N], accumulate=True, scratch=scratch)
+    K.gemm(a, w, acc[:, 3:3 + N], accumulate=True, scratch=scratch, kernel=kernel)
     assert (acc[:, 3:3 + N].double() - (base[:, 3:3 + N].double() + want)).abs().max() < 1e-4 * want.abs().max()
     assert torch.equal(acc[:, :3], base[:, :3]) and torch.equal(acc[:, 3 + N:], base[:, 3 + N:])
     # too little scratch: the product is not split, and is right all the same
     small = torch.empty(16, device=DEV)
-    K.gemm(a, w, again, scratch=small)
+    K.gemm(a, w, again, scratch=small, kernel=kernel)
     assert (again.double() - want).abs().max() < 1e-4 * want.abs().max()
 
 
@@ -457,8 +463,8 @@ def test_attention_kernels_refuse_what_they_do_not_take():
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7])
-@pytest.mark.parametrize("M,I,Kd", [(1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("M,I,Kd", [(40, 8264, 256), (64, 328, 1152), (1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
                                     (300, 512, 1024), (129, 200, 192), (1, 2056, 1024), (8, 328, 1152), (13, 4400, 1280)])
 def test_gemm_with_swiglu_epilogue(M, I, Kd, kernel):
     _skip_unless_kernel_takes(kernel, M, Kd)
