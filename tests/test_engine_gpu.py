@@ -343,3 +343,58 @@ def test_random_schedules_of_cuts_and_batches(engines, tiny_folders, name, dtype
     for i in range(len(seqs)):
         close(np.concatenate(got[i]), refs[i], dtype, f"{name} request {i} of {len(seqs[i])} tokens")
     assert [g.pool.free_count for g in eng.cache.groups] == free_before
+
+
+# ---- sizes that take the kernels of serving shapes -------------------------------------
+# The tiny configurations run through the kernels for any shape.  This one is wide enough
+# for the others: head size 128 (attention through LDS rings, for prompts and for single
+# tokens), widths of 1024 and 1536 (products by direct-to-LDS tiles for prompts, by the
+# streaming kernels for 1 to 16 and 17 to 64 rows), a vocabulary that is no multiple of 16,
+# a window on one of the two layers.
+SERVING = dict(num_hidden_layers=2, hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, head_dim=128,
+               intermediate_size=1536, vocab_size=1000, rope_theta=1e6, rms_norm_eps=1e-5, sliding_window=100,
+               max_position_embeddings=4096, tie_word_embeddings=False,
+               layer_types=["full_attention", "sliding_attention"])
+
+
+@pytest.fixture(scope="module")
+def serving(tmp_path_factory):
+    folder = str(tmp_path_factory.mktemp("serving_sizes"))
+    B.Engine.write_random_folder(folder, B.MistralConfig.from_dict(SERVING), seed=3, std=0.03, vector_jitter=0.3)
+    cfg, w = P.read_folder(folder)
+    return folder, cfg, w
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_serving_sizes_whole_then_one_by_one_then_batched(serving, dtype):
+    folder, cfg, w = serving
+    eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=8192)
+    toks = tokens(cfg, 340, 7)
+    ref = P.forward(cfg, w, toks)
+    one = whole(eng, toks)
+    close(one, ref, dtype, "serving sizes, whole")
+    s = eng.alloc_slot()
+    n0 = 300
+    parts = [eng.step([StepEntry(s, toks[:n0], list(range(n0)))]).cpu().numpy()]
+    for t in toks[n0:]:
+        parts.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    eng.free_slot(s)
+    cut = np.concatenate(parts)
+    close(cut, ref, dtype, "serving sizes, last 40 one by one")
+    assert np.abs(cut - one).max() <= CUT_TOL[dtype] * np.abs(ref).max()
+    # 20 requests of unequal lengths: prompts in one step, then 6 tokens each in steps of 20 rows
+    lens = [5 + 13 * i for i in range(20)]
+    seqs = [tokens(cfg, n + 6, 50 + i) for i, n in enumerate(lens)]
+    slots = [eng.alloc_slot() for _ in seqs]
+    got = [[] for _ in seqs]
+    out = eng.step([StepEntry(sl, q[:n], [n - 1]) for sl, q, n in zip(slots, seqs, lens)]).cpu().numpy()
+    for i in range(20):
+        got[i].append(out[i:i + 1])
+    for k in range(6):
+        out = eng.step([StepEntry(sl, [q[n + k]], [0]) for sl, q, n in zip(slots, seqs, lens)]).cpu().numpy()
+        for i in range(20):
+            got[i].append(out[i:i + 1])
+    for sl in slots:
+        eng.free_slot(sl)
+    for i in (0, 7, 19):
+        close(np.concatenate(got[i]), P.forward(cfg, w, seqs[i])[lens[i] - 1:], dtype, f"serving sizes, request {i} of 20")
