@@ -538,12 +538,22 @@ __device__ __forceinline__ int kswz(int row, int cols) {      // the 16 key rows
 
 #define DEC_MAX_RUN 1024      // pages of one workgroup's run whose numbers are kept in LDS
 
-template <int HD, int S>
+//
+// FUSE: the step's rotation and cache write are done here instead of by rope_kv_write (one
+// kernel less per layer).  `q` then points at the step's raw rows [q heads | k heads | v
+// heads]; sequence b's token stands at position ctx - 1 and its angles in row b of cs / sn
+// ([B, HD / 2], pairs (p, p + HD / 2); null = no rotation).  Every workgroup rotates its
+// query heads in registers; the workgroup whose run holds the last page first stores the
+// rotated key and the value of the new token in that page (when `write_cache`), and waits
+// for the stores before the page is fetched.  For groups of up to 16 heads, so that one
+// workgroup alone reads that page.
+template <int HD, int S, bool FUSE>
 __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
     const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ slots,
     const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
-    const bf16* __restrict__ cache, int nq, int nkv, int window, float scale, int nsplit,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    bf16* __restrict__ cache, int nq, int nkv, int window, float scale, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ cs,
+    const float* __restrict__ sn, int write_cache) {
     constexpr int NB = HD / 32;                      // 32-wide k-steps of the score product
     constexpr int KROWB = HD * 2, KCOLS = KROWB / 16; // a key row in bytes, in 16-byte columns
     constexpr int KB = PAGE * KROWB, STAGE = 2 * KB;  // keys, then values [HD][128 bytes]
@@ -580,13 +590,52 @@ __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
     bf16x8 qf[NB];
 #pragma unroll
     for (int s = 0; s < NB; ++s) qf[s] = head_ok ? *(const bf16x8*)(qrow + s * 32 + 8 * g) : zero8();
+    const size_t page_elems = (size_t)2 * nkv * PAGE * HD;
+    const size_t k_off = (size_t)kvh * PAGE * HD, v_off = ((size_t)nkv + kvh) * PAGE * HD;
+    if constexpr (FUSE) {
+        constexpr int P = HD / 2;
+        if (cs) {
+            // this lane holds dims 32 s + 8 g + e; their partners are NB / 2 fragments on
+#pragma unroll
+            for (int s = 0; s < NB / 2; ++s) {
+                const float* cp = cs + (size_t)b * P + s * 32 + 8 * g;
+                const float* sp = sn + (size_t)b * P + s * 32 + 8 * g;
+#pragma unroll
+                for (int v4 = 0; v4 < 2; ++v4) {
+                    const f32x4 cc = *(const f32x4*)(cp + 4 * v4), ss = *(const f32x4*)(sp + 4 * v4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float a = (float)qf[s][4 * v4 + e], bb = (float)qf[s + NB / 2][4 * v4 + e];
+                        qf[s][4 * v4 + e] = (bf16)(a * cc[e] - bb * ss[e]);
+                        qf[s + NB / 2][4 * v4 + e] = (bf16)(a * ss[e] + bb * cc[e]);
+                    }
+                }
+            }
+        }
+        const int last_pg = ctx > 0 ? (ctx - 1) / PAGE : -1;
+        if (write_cache && hb == 0 && last_pg >= pg_begin && last_pg < pg_end) {
+            const int off = (ctx - 1) % PAGE;
+            bf16* pg = cache + (size_t)bt[last_pg] * page_elems;
+            const bf16* krow = q + (size_t)b * q_stride + (size_t)(nq + kvh) * HD;
+            const bf16* vrow = krow + (size_t)nkv * HD;
+            if (tid < P) {
+                const float a = (float)krow[tid], bb = (float)krow[tid + P];
+                const float cc = cs ? cs[(size_t)b * P + tid] : 1.f, ss = cs ? sn[(size_t)b * P + tid] : 0.f;
+                pg[k_off + (size_t)off * HD + tid] = (bf16)(a * cc - bb * ss);
+                pg[k_off + (size_t)off * HD + tid + P] = (bf16)(a * ss + bb * cc);
+            } else if (tid < P + HD) {
+                const int d = tid - P;
+                pg[v_off + (size_t)d * PAGE + off] = vrow[d];
+            }
+        }
+        // __syncthreads below waits for these stores (they have reached the L2) before any page is fetched
+    }
     // the query has arrived before the loop: a wait for it inside would also wait for the pages in flight
 #pragma unroll
     for (int s = 0; s < NB; ++s) asm volatile("" ::"v"(qf[s]));
+    if constexpr (FUSE) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    const size_t page_elems = (size_t)2 * nkv * PAGE * HD;
-    const size_t k_off = (size_t)kvh * PAGE * HD, v_off = ((size_t)nkv + kvh) * PAGE * HD;
     const unsigned ring_lds = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)dsm);
 #define DEC_ISSUE(I)                                                                                         \
     do {                                                                                                     \
@@ -798,9 +847,9 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
 // part_o: float [B, nq, nsplit, hd]; part_ml: float [B, nq, nsplit, 2] (unused when nsplit == 1)
 extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, const int* slots,
                                    const int* ctx_lens, const int* block_table, int table_stride,
-                                   const void* cache, int B, int nq, int nkv, int hd, int page, int window,
+                                   void* cache, int B, int nq, int nkv, int hd, int page, int window,
                                    float scale, int nsplit, float* part_o, float* part_ml, int variant,
-                                   hipStream_t s) {
+                                   int fuse, const float* cs, const float* sn, int write_cache, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
         q_stride % 8 || ((uintptr_t)q % 16) || nsplit < 1 || nsplit > 1024 || B > 65535 ||
@@ -815,14 +864,16 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
                         (uintptr_t)cache % 16 == 0;
     if (variant < 0 || variant > 2 || (variant == 2 && !lds_ok)) return BR_BAD_ARG;
     if (variant == 0) variant = lds_ok ? 2 : 1;
+    // fuse: rotation and cache write inside the LDS kernel (see there); the caller asks only where it applies
+    if (fuse && (variant != 2 || G > 16 || (cs && (!sn || ((uintptr_t)cs | (uintptr_t)sn) % 16)))) return BR_BAD_ARG;
     if (variant == 2) {
         // two stages leave room for two workgroups per CU; with at most one workgroup per CU
         // a third stage keeps two pages in flight instead (measured: 34 -> 32 us at 8 x 4096 tokens)
         const int cus = br_device_cus();
         const bool deep = cus > 0 && (long long)nsplit * nkv * nhb * B <= cus;
-#define BR_DECODE_LDS(HD_, S_)                                                                                  \
+#define BR_DECODE_LDS(HD_, S_, FUSE_)                                                                          \
     do {                                                                                                        \
-        auto kern = attn_decode_lds_kernel<HD_, S_>;                                                            \
+        auto kern = attn_decode_lds_kernel<HD_, S_, FUSE_>;                                                     \
         constexpr size_t lds2 = (size_t)S_ * 2 * PAGE * HD_ * 2 + DEC_MAX_RUN * sizeof(int);                    \
         static bool set = false;                                                                                \
         if (!set) {                                                                                             \
@@ -832,11 +883,16 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
             set = true;                                                                                         \
         }                                                                                                       \
         kern<<<grid, 256, lds2, s>>>((const bf16*)q, q_stride, (bf16*)out, slots, ctx_lens, block_table,        \
-                                     table_stride, (const bf16*)cache, nq, nkv, window, scale, nsplit, part_o,  \
-                                     part_ml);                                                                  \
+                                     table_stride, (bf16*)cache, nq, nkv, window, scale, nsplit, part_o,        \
+                                     part_ml, cs, sn, write_cache);                                             \
     } while (0)
-        if (hd == 128) { if (deep) BR_DECODE_LDS(128, 3); else BR_DECODE_LDS(128, 2); }
-        else { if (deep) BR_DECODE_LDS(64, 3); else BR_DECODE_LDS(64, 2); }
+        if (fuse) {
+            if (hd == 128) { if (deep) BR_DECODE_LDS(128, 3, true); else BR_DECODE_LDS(128, 2, true); }
+            else { if (deep) BR_DECODE_LDS(64, 3, true); else BR_DECODE_LDS(64, 2, true); }
+        } else {
+            if (hd == 128) { if (deep) BR_DECODE_LDS(128, 3, false); else BR_DECODE_LDS(128, 2, false); }
+            else { if (deep) BR_DECODE_LDS(64, 3, false); else BR_DECODE_LDS(64, 2, false); }
+        }
 #undef BR_DECODE_LDS
         int rc2 = br_check_launch();
         if (rc2 != BR_OK || nsplit == 1) return rc2;

@@ -284,10 +284,16 @@ def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slo
                           ctx_lens: torch.Tensor, block_table: torch.Tensor, cache: torch.Tensor, B: int,
                           nq: int, nkv: int, hd: int, page: int, window: Optional[int], scale: float,
                           nsplit: int, part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
-                          variant: int = 0) -> None:
+                          variant: int = 0, fuse_rope: bool = False, cos: Optional[torch.Tensor] = None,
+                          sin: Optional[torch.Tensor] = None, write_cache: bool = True) -> None:
     """Attention of one new token per sequence over its pages, cut into `nsplit` runs.
     `variant` forces a kernel: 1 reads operands straight from the cache, 2 brings pages
-    through a ring in LDS (head sizes 64 and 128); 0 chooses."""
+    through a ring in LDS (head sizes 64 and 128); 0 chooses.
+
+    `fuse_rope` (where `attention_decode_fuses_rope` says so): `q` is the step's raw
+    [B, (nq + 2 nkv) * hd] rows; the kernel rotates queries and the new key by `cos` / `sin`
+    ([B, hd / 2], pairs (p, p + hd / 2); None = no rotation) and stores key and value of the
+    new token in the cache itself (`write_cache`), so `rope_kv_write` is not called."""
     _dev("attention_decode_bf16", out, slots, ctx_lens, block_table, cache, part_o, part_ml)
     _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
          "attention_decode_bf16: bfloat16 only")
@@ -300,10 +306,28 @@ def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slo
              and part_ml is not None and part_ml.numel() >= B * nq * nsplit * 2,
              "attention_decode_bf16: scratch for the splits is too small")
     f = _fn("attention_bf16", "br_attn_decode_bf16",
-            [_P, c_size_t, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, c_int, _P, _P, c_int, _P])
+            [_P, c_size_t, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, c_int, _P, _P, c_int, c_int, _P, _P,
+                                                                      c_int, _P])
+    if fuse_rope:
+        _req(attention_decode_fuses_rope(hd, nq, nkv, page, block_table.shape[1], nsplit),
+             "attention_decode_bf16: rotation and cache write are not fused for these sizes")
+        _req(q.shape[-1] == (nq + 2 * nkv) * hd, "attention_decode_bf16: fused rotation needs the raw q, k, v rows")
+        if cos is not None:
+            _dev("attention_decode_bf16", cos, sin)
+            _req(sin is not None and cos.dtype == sin.dtype == torch.float32 and cos.numel() >= B * (hd // 2)
+                 and sin.numel() >= B * (hd // 2), "attention_decode_bf16: rotary tables must be float32 [B, hd / 2]")
     _check(f(_ptr(q), q_stride, _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1],
              _ptr(cache), B, nq, nkv, hd, page, int(window or 0), float(scale), nsplit, _ptr(part_o),
-             _ptr(part_ml), int(variant), _stream()), "attention_decode_bf16")
+             _ptr(part_ml), int(variant), int(fuse_rope), _ptr(cos) if fuse_rope else None,
+             _ptr(sin) if fuse_rope else None, int(write_cache), _stream()), "attention_decode_bf16")
+
+
+def attention_decode_fuses_rope(hd: int, nq: int, nkv: int, page: int, table_pages: int, nsplit: int) -> bool:
+    """Whether `attention_decode_bf16` can do the step's rotation (full head, pairs
+    (p, p + hd / 2), or none) and cache write itself: the kernel that brings pages through
+    LDS (head sizes 64 and 128, runs of at most 1024 pages), groups of up to 16 heads."""
+    return (hd in (64, 128) and page == 64 and nkv > 0 and nq % nkv == 0 and nq // nkv <= 16
+            and -(-table_pages // max(1, nsplit)) <= 1024)
 
 
 # -------------------------------------------------------------------- sampling -----

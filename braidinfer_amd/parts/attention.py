@@ -78,15 +78,30 @@ class GQAAttention(Mixer):
         tables = step.position_data.get(self.position) if self.position else None
         if tables is not None and not isinstance(tables, RotaryTables):
             tables = None
+        if self._fused_decode(qkv, tables, step, ctx):
+            return self._finish(qkv, x, step, ctx, tables, True)
         K.rope_kv_write(qkv, tables.cos if tables else None, tables.sin if tables else None,
                         step.positions, step.seq_of_token, step.slots, ctx.block_table, ctx.storage,
                         nq, nkv, hd, tables.rotary_dim if tables else 0, tables.adjacent if tables else False,
                         ctx.page_tokens, ctx.writes_cache)
-        o = step.ws.get("attn_out", (T, nq * hd), dt)
-        self.attend(qkv, o, step, ctx)
+        self._finish(qkv, x, step, ctx, None, False)
+
+    def _fused_decode(self, qkv, tables, step, ctx: MixerContext) -> bool:
+        """Single-token steps whose attention kernel also rotates and writes the cache:
+        full-head rotation in (p, p + hd / 2) pairs, or none."""
+        if not (step.is_decode and qkv.dtype == torch.bfloat16 and not self.force_simple and ctx.storage is not None):
+            return False
+        if tables is not None and (tables.adjacent or tables.rotary_dim != self.hd):
+            return False
+        nsplit = decode_splits(step.n_seqs, self.nkv, step.max_ctx_bound, ctx.page_tokens)
+        return K.attention_decode_fuses_rope(self.hd, self.nq, self.nkv, ctx.page_tokens, ctx.block_table.shape[1], nsplit)
+
+    def _finish(self, qkv, x, step, ctx: MixerContext, fused_tables, fused: bool) -> None:
+        o = step.ws.get("attn_out", (step.n_tokens, self.nq * self.hd), self.rt.dtype)
+        self.attend(qkv, o, step, ctx, fused_tables, fused)
         linear(o, self.w_o, x, step.ws, accumulate=True)
 
-    def attend(self, qkv, o, step, ctx: MixerContext) -> None:
+    def attend(self, qkv, o, step, ctx: MixerContext, fused_tables=None, fused: bool = False) -> None:
         """bf16 with a head size the matrix-core kernels take: split-context kernel when
         every sequence brings one token, flash kernel otherwise.  Else (32-bit path, head
         sizes beyond 256 or not in steps of 16) the one-wave-per-query kernel."""
@@ -102,7 +117,9 @@ class GQAAttention(Mixer):
                     part_ml = step.ws.get("attn_part_ml", (B * nq * nsplit * 2,), torch.float32)
                 K.attention_decode_bf16(qkv, qkv.stride(0), o, step.slots, step.ctx_lens, ctx.block_table,
                                         ctx.storage, B, nq, nkv, hd, ctx.page_tokens, self.window, self.scale,
-                                        nsplit, part_o, part_ml)
+                                        nsplit, part_o, part_ml, 0, fused,
+                                        fused_tables.cos if fused_tables is not None else None,
+                                        fused_tables.sin if fused_tables is not None else None, ctx.writes_cache)
             else:
                 K.attention_prefill_bf16(qkv, qkv.stride(0), o, step.cu_seqlens, step.slots, step.ctx_lens,
                                          ctx.block_table, ctx.storage, B, step.max_new, nq, nkv, hd,

@@ -452,6 +452,55 @@ def test_attention_decode_matrix_cores(nq, nkv, hd, window, nsplit, variant):
         assert (got - want).abs().max() < 2e-2 * want.abs().max(), f"sequence {b} of length {l}"
 
 
+@pytest.mark.parametrize("rope", [True, False])
+@pytest.mark.parametrize("nsplit", [1, 3])
+@pytest.mark.parametrize("nq,nkv,hd,window", [(32, 8, 128, None), (8, 2, 128, 100), (16, 1, 64, None), (8, 4, 64, 70)])
+def test_attention_decode_with_rotation_and_cache_write_fused(nq, nkv, hd, window, nsplit, rope):
+    """The kernel that rotates and stores the new token itself against rope_kv_write followed
+    by the same kernel: the cache afterwards and the outputs."""
+    lens = [200, 37, 64, 1, 130, 65, 513, 128]                   # the new token included; 64, 65, 128, 1: page edges
+    B, page, theta = len(lens), 64, 1e6
+    _, _, cache, table = _multi_seq_cache(lens, nkv, hd, seed=nq + hd + 7)
+    qkv = rnd(B + 1, (nq + 2 * nkv) * hd, seed=5, dtype=torch.bfloat16)      # the last row is padding (slot -1)
+    slots = i32(list(range(1, B + 1)) + [-1])
+    ctx = i32(lens + [0])
+    pos = i32([l - 1 for l in lens] + [0])
+    sot = torch.arange(B + 1).int().to(DEV)
+    cs = sn = None
+    if rope:
+        inv = (1.0 / theta ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)).to(DEV)
+        cs, sn = torch.empty(B + 1, hd // 2, device=DEV), torch.empty(B + 1, hd // 2, device=DEV)
+        K.rope_table(pos, inv, cs, sn)
+    part = lambda: (torch.empty((B + 1) * nq * nsplit * hd, device=DEV), torch.empty((B + 1) * nq * nsplit * 2, device=DEV))
+    # two steps
+    qkv2, cache2 = qkv.clone(), cache.clone()
+    K.rope_kv_write(qkv2, cs, sn, pos, sot, slots, table, cache2, nq, nkv, hd, hd if rope else 0, False, page, True)
+    want = torch.full((B + 1, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
+    po, pml = part()
+    K.attention_decode_bf16(qkv2, qkv2.stride(0), want, slots, ctx, table, cache2, B + 1, nq, nkv, hd, page, window,
+                            1 / math.sqrt(hd), nsplit, po, pml, 2)
+    # one
+    assert K.attention_decode_fuses_rope(hd, nq, nkv, page, table.shape[1], nsplit)
+    qkv1, cache1 = qkv.clone(), cache.clone()
+    got = torch.full((B + 1, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
+    po, pml = part()
+    K.attention_decode_bf16(qkv1, qkv1.stride(0), got, slots, ctx, table, cache1, B + 1, nq, nkv, hd, page, window,
+                            1 / math.sqrt(hd), nsplit, po, pml, 2, True, cs, sn, True)
+    assert torch.equal(cache1[:, 1], cache2[:, 1])                             # values: copied
+    assert (cache1[:, 0].float() - cache2[:, 0].float()).abs().max() <= 2 ** -7 * cache2[:, 0].float().abs().max()
+    assert torch.all(got[B] == 0)
+    scale = want[:B].float().abs().max()
+    assert (got[:B].float() - want[:B].float()).abs().max() <= 2e-2 * scale
+    # write_cache=False leaves the cache alone
+    cache3 = cache.clone()
+    K.attention_decode_bf16(qkv.clone(), qkv.stride(0), got, slots, ctx, table, cache3, B + 1, nq, nkv, hd, page, window,
+                            1 / math.sqrt(hd), nsplit, po, pml, 2, True, cs, sn, False)
+    assert torch.equal(cache3, cache)
+    with pytest.raises(KernelError):
+        K.attention_decode_bf16(qkv1, qkv1.stride(0), got, slots, ctx, table, cache1, B + 1, 34, 2, hd, page, window,
+                                1 / math.sqrt(hd), nsplit, po, pml, 2, True, cs, sn, True)
+
+
 def test_attention_kernels_refuse_what_they_do_not_take():
     q = rnd(4, 2 * 24, dtype=torch.bfloat16)
     cache = torch.zeros(2, 2, 1, 64, 24, dtype=torch.bfloat16, device=DEV)
