@@ -301,11 +301,14 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int S, int MODE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
-    const bf16* __restrict__ A, const bf16* __restrict__ W, void* __restrict__ C, int M, int N, int K, size_t lda,
-    size_t ldc, int tiles_m, int tiles_n) {
+    const bf16* __restrict__ A, const bf16* __restrict__ W, void* __restrict__ C_, int M, int N, int K, size_t lda,
+    size_t ldc, int tiles_m, int tiles_n, int kt_per_part, size_t part_stride) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int STAGE_BYTES = (BM + BN) * DMA_BK * 2;
+    // blockIdx.y: which run of k-tiles this workgroup sums (one run, or the parts of a split
+    // product, each into a float matrix of its own `part_stride` elements on)
+    void* C = MODE == OUT_F32 ? (void*)((float*)C_ + blockIdx.y * part_stride) : C_;
     constexpr int INSTR = (BM + BN) / 8 / NW;           // 1 KB wave-loads per wave and stage
     static_assert(S == 2 || S == 3, "2 or 3 stages");
     __shared__ __attribute__((aligned(1024))) unsigned char st0[STAGE_BYTES];
@@ -352,9 +355,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
             if (r > N - 1) r = N - 1;
             src[q] = W + (size_t)r * K + c * 8;
         }
+        src[q] += (size_t)blockIdx.y * kt_per_part * DMA_BK;
         dst[q] = (q * NW + wave) * 1024;
     }
-    const int nk = K / DMA_BK;
+    int nk = K / DMA_BK - (int)blockIdx.y * kt_per_part;
+    if (nk > kt_per_part) nk = kt_per_part;
     if (S == 2) {
         DMA_ISSUE(st0, 0);
         for (int kt = 0; kt < nk; kt += 2) {
@@ -400,22 +405,63 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
     tile_epilogue<TM, TN, MODE>(acc, C, M, N, ldc, m0 + wm, n0 + wn, lane);
 }
 
+static int launch_split_sum(const float* scratch, int parts, void* C, int M, int N, size_t ldc, int mode, hipStream_t s);
+
+// parts > 1: the k-tiles are cut into `parts` runs, every (tile, run) workgroup writes its
+// float sums to a matrix of its own in `scratch`, and gemm_split_sum_kernel adds the runs in
+// run order and applies the epilogue (for products with too few tiles to fill the chip).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int S>
 static int launch_tile_dma(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
-                           int mode, hipStream_t s) {
+                           int mode, hipStream_t s, int parts = 1, float* scratch = nullptr) {
     const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     const long long total = (long long)tm * tn;
     if (total > 0x7fffffffLL) return BR_BAD_ARG;
     constexpr int NT = 64 * WAVES_M * WAVES_N;
+    const int nk = K / DMA_BK;
+    if (parts > 1) {
+        const int kpp = (nk + parts - 1) / parts;
+        parts = (nk + kpp - 1) / kpp;                                 // no empty run
+        dim3 grid((unsigned)total, (unsigned)parts);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<grid, NT, 0, s>>>(
+            A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp, (size_t)M * N);
+        int rc = br_check_launch();
+        if (rc != BR_OK) return rc;
+        return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
+    }
     if (mode == OUT_BF16)
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_BF16><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_BF16><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
     else if (mode == OUT_F32)
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
     else if (mode == OUT_F32_ACC)
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32_ACC><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32_ACC><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
     else
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_SWIGLU><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_SWIGLU><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
     return br_check_launch();
+}
+
+// Which direct-to-LDS tile (5: 128x256, one workgroup per CU; 6: 128x128, two) and how many
+// runs of k-tiles for a product of more than 64 rows: the least time by a rough count in
+// microseconds (rounds of workgroups over the chip times k-tiles times 1.0-1.3 us a k-tile,
+// plus, when split, a launch and the traffic of the partial sums), runs of at least 4
+// k-tiles that fit the scratch memory.
+static void choose_tile(int M, int N, int K, int cus, size_t scratch_bytes, int* kernel, int* parts) {
+    const int nk = K / DMA_BK;
+    double best = 1e30;
+    *kernel = 5;
+    *parts = 1;
+    for (int k = 5; k <= 6; ++k) {
+        const long long tiles = (long long)((M + 127) / 128) * ((N + (k == 5 ? 255 : 127)) / (k == 5 ? 256 : 128));
+        const long long slots = (long long)cus * (k == 5 ? 1 : 2);
+        for (int p = 1; p <= 16; p *= 2) {
+            if (p > 1 && (p * 4 > nk || (size_t)p * M * N * sizeof(float) > scratch_bytes)) break;
+            const long long units = tiles * p, rounds = (units + slots - 1) / slots;
+            const int kpp = (nk + p - 1) / p;
+            const double per = k == 5 ? 1.14 : (units > cus ? 1.33 : 1.0);
+            double t = (double)rounds * kpp * per;
+            if (p > 1) t += 5.0 + (double)p * M * N * 8.0 / 4e6;
+            if (t < best - 1e-9) { best = t; *kernel = k; *parts = p; }
+        }
+    }
 }
 
 // ----------------------------------------------------------------- gemm_skinny ------
@@ -679,11 +725,32 @@ template <int MODE>
 __global__ void gemm_split_sum_kernel(const float* __restrict__ part, int parts, size_t part_stride, void* __restrict__ C,
                                       int M, int N, size_t ldc) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (MODE == OUT_SWIGLU) {
+        // output j of a row: gate column 16 (j / 8) + j % 8, its up value 8 columns on
+        const size_t half = (size_t)N / 2;
+        if (i >= (size_t)M * half) return;
+        const size_t m = i / half, j = i - m * half;
+        const size_t gc = m * N + (j >> 3) * 16 + (j & 7);
+        float gv = 0.f, uv = 0.f;
+        for (int p = 0; p < parts; ++p) { gv += part[p * part_stride + gc]; uv += part[p * part_stride + gc + 8]; }
+        ((bf16*)C)[m * ldc + j] = (bf16)silu_mul(gv, uv);
+        return;
+    }
     if (i >= (size_t)M * N) return;
     float v = 0.f;
     for (int p = 0; p < parts; ++p) v += part[p * part_stride + i];
     const size_t m = i / N, n = i - m * N;
     store_out<MODE>(C, m * ldc + n, v);
+}
+
+static int launch_split_sum(const float* scratch, int parts, void* C, int M, int N, size_t ldc, int mode, hipStream_t s) {
+    const size_t stride = (size_t)M * N;
+    const unsigned blocks = (unsigned)((stride + 255) / 256);
+    if (mode == OUT_BF16) gemm_split_sum_kernel<OUT_BF16><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    else if (mode == OUT_F32) gemm_split_sum_kernel<OUT_F32><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    else if (mode == OUT_F32_ACC) gemm_split_sum_kernel<OUT_F32_ACC><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    else gemm_split_sum_kernel<OUT_SWIGLU><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
+    return br_check_launch();
 }
 
 template <int MB>
@@ -698,11 +765,7 @@ static int launch_split(const bf16* A, const bf16* W, void* C, int M, int N, int
     gemm_skinny_lds_kernel<MB, RB, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, spp, stride);
     int rc = br_check_launch();
     if (rc != BR_OK) return rc;
-    const unsigned blocks = (unsigned)((stride + 255) / 256);
-    if (mode == OUT_BF16) gemm_split_sum_kernel<OUT_BF16><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
-    else if (mode == OUT_F32) gemm_split_sum_kernel<OUT_F32><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
-    else gemm_split_sum_kernel<OUT_F32_ACC><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
-    return br_check_launch();
+    return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
 }
 
 // How many runs of k-slabs a product of 16 < M <= 64 rows is cut into when the caller gives
@@ -1086,11 +1149,7 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
         BR_WIDE(OUT_F32, true, (void*)scratch);
         int rc = br_check_launch();
         if (rc != BR_OK) return rc;
-        const unsigned blocks = (unsigned)((stride + 255) / 256);
-        if (mode == OUT_BF16) gemm_split_sum_kernel<OUT_BF16><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
-        else if (mode == OUT_F32) gemm_split_sum_kernel<OUT_F32><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
-        else gemm_split_sum_kernel<OUT_F32_ACC><<<blocks, 256, 0, s>>>(scratch, parts, stride, C, M, N, ldc);
-        return br_check_launch();
+        return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
     }
     if (mode == OUT_BF16) BR_WIDE(OUT_BF16, false, C);
     else if (mode == OUT_F32) BR_WIDE(OUT_F32, false, C);
@@ -1123,6 +1182,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
                          (!scratch || (uintptr_t)scratch % 16 == 0);
     if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 8 || kernel < 0) return BR_BAD_ARG;
     // measured at M = 64: many weight rows (gate/up) are 4 % faster through the 64x128 tile, which kernel 3 picks
+    const bool chosen = kernel == 0;
     if (kernel == 0)
         kernel = stream_ok ? 7
                  : (wide_ok && !(M > 32 && N >= 16384 && dma_ok)) ? 8
@@ -1132,9 +1192,14 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
                        : launch_stream_wide<4>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s);
     if (kernel == 7) return M <= 8 ? launch_stream<8>(A, W, C, M, N, K, lda, ldc, mode, s)
                                    : launch_stream<16>(A, W, C, M, N, K, lda, ldc, mode, s);
+    int parts = 1;
+    if (chosen && (kernel == 5 || kernel == 6)) {
+        const int cus = br_device_cus();
+        if (cus > 0) choose_tile(M, N, K, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
+    }
     if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
-    if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
-    if (kernel == 6) return launch_tile_dma<128, 128, 2, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s);
+    if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch);
+    if (kernel == 6) return launch_tile_dma<128, 128, 2, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch);
     if (kernel == 3) {
         // shapes measured on cold weights (cycled through more than the 256 MB cache)
         const bool wide = N >= 16384;
@@ -1158,4 +1223,12 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
 extern "C" int br_gemm_bf16(const void* A, const void* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                             int mode, hipStream_t s) {
     return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, nullptr, 0, s);
+}
+
+// what br_gemm_bf16_ex would pick for more than 64 rows (tests and benchmarks print it)
+extern "C" int br_gemm_bf16_tile_choice(int M, int N, int K, size_t scratch_bytes, int* kernel, int* parts) {
+    const int cus = br_device_cus();
+    if (!cus) return BR_LAUNCH_FAILED;
+    choose_tile(M, N, K, cus, scratch_bytes, kernel, parts);
+    return BR_OK;
 }

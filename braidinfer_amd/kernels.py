@@ -165,7 +165,7 @@ def convert(a: torch.Tensor, out: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------------ GEMM ------
-GEMM_SCRATCH_FLOATS = 8 * 64 * 8192      # room for every product that the bf16 kernels split along k
+GEMM_SCRATCH_FLOATS = 16 * 1024 * 1024   # 64 MB: room for the partial sums of the products that the bf16 kernels split along k
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, kernel: int = 0,
@@ -181,8 +181,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     loaded straight into LDS, K in steps of 64; 7: streaming by workgroups that stay, M <= 16
     and K in steps of 128 from 1024; 8: the same for 17 to 64 rows, K in steps of 128); 0 chooses by
     shape.
-    `scratch` (float32, on the device): with it, a bf16 product of 17 to 64 rows with few
-    weight rows is cut along k into runs that are summed in a fixed order by a second kernel.
+    `scratch` (float32, on the device): with it, a bf16 product of more than 16 rows with too
+    few tiles to fill the chip is cut along k into runs that a second kernel sums in a fixed order.
     """
     name = "gemm"
     for t in (a, w, out):
@@ -216,9 +216,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"gemm: a is {a.dtype} and w is {w.dtype}; both float32 or both bfloat16")
 
 
-def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: int = 0) -> None:
+def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: int = 0,
+                scratch: Optional[torch.Tensor] = None) -> None:
     """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) in one bf16 product: `w_gu` [2 I, K] holds
-    gate and up rows interleaved in blocks of 16 (see `interleave_gate_up`)."""
+    gate and up rows interleaved in blocks of 16 (see `interleave_gate_up`).  `scratch` as
+    for `gemm`."""
     for t in (a, w_gu, out):
         if not t.is_cuda:
             raise KernelError(f"gemm_swiglu: tensor on {t.device}; kernels run on the GPU only")
@@ -230,7 +232,10 @@ def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: 
     lda, ldc = (a.stride(0) if M > 1 else K), (out.stride(0) if M > 1 else N // 2)
     f = _fn("gemm_bf16", "br_gemm_bf16_ex",
             [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, _P])
-    _check(f(_ptr(a), _ptr(w_gu), _ptr(out), M, N, K, lda, ldc, 3, kernel, None, 0, _stream()), "gemm_swiglu")
+    if scratch is not None:
+        _req(scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous(), "gemm_swiglu: scratch must be float32 on the device")
+    _check(f(_ptr(a), _ptr(w_gu), _ptr(out), M, N, K, lda, ldc, 3, kernel, _ptr(scratch),
+             0 if scratch is None else scratch.numel() * 4, _stream()), "gemm_swiglu")
 
 
 def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:

@@ -41,7 +41,8 @@ class SwiGLU(FeedForward):
         dt = self.rt.dtype
         a = step.ws.get("ffn_act", (T, self.I), dt)
         if self.fused:
-            K.gemm_swiglu(h, self.w_gu, a)
+            scratch = step.ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if 64 < T <= 1024 else None
+            K.gemm_swiglu(h, self.w_gu, a, scratch=scratch)
         else:
             gu = step.ws.get("ffn_gu", (T, 2 * self.I), dt)
             linear(h, self.w_gu, gu, step.ws)

@@ -20,7 +20,7 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, ws, accumulate: 
                 K.convert(tmp, out)
                 return
             scratch = None
-            if a.dtype == torch.bfloat16 and 16 < a.shape[0] <= 64:
+            if a.dtype == torch.bfloat16 and 16 < a.shape[0] <= 1024:     # products that may be split along k
                 scratch = ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32)
             K.gemm(a, w, out, accumulate, scratch=scratch)
             return
