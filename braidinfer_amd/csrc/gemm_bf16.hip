@@ -1171,6 +1171,9 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (M <= 0 || N <= 0) return BR_OK;
     if (K <= 0 || lda < (size_t)K || mode < 0 || mode > 3) return BR_BAD_ARG;
     if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
+    // kernel / 16: a forced number of runs along k for kernels 5 and 6 (measurements), 0 = by shape
+    const int forced_parts = kernel >= 16 ? kernel / 16 : 0;
+    kernel %= 16;
     const bf16* A = (const bf16*)A_;
     const bf16* W = (const bf16*)W_;
     const bool aligned = (K % 8 == 0) && (lda % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
@@ -1196,6 +1199,12 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (chosen && (kernel == 5 || kernel == 6)) {
         const int cus = br_device_cus();
         if (cus > 0) choose_tile(M, N, K, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
+    }
+    if (forced_parts > 1 && (kernel == 5 || kernel == 6)) {
+        if (!scratch || (uintptr_t)scratch % 16 || (size_t)forced_parts * M * N * sizeof(float) > scratch_bytes ||
+            forced_parts > K / DMA_BK)
+            return BR_BAD_ARG;
+        parts = forced_parts;
     }
     if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
     if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch);

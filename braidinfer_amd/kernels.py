@@ -179,8 +179,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     `kernel` forces one bf16 kernel (1, 2: 128x128 and 256x128 tiles staged through
     registers, any shape; 3: skinny, M <= 64; 4, 5, 6: 256x128, 128x256 and 128x128 tiles
     loaded straight into LDS, K in steps of 64; 7: streaming by workgroups that stay, M <= 16
-    and K in steps of 128 from 1024; 8: the same for 17 to 64 rows, K in steps of 128); 0 chooses by
-    shape.
+    and K in steps of 128 from 1024; 8: the same for 17 to 64 rows, K in steps of 128; 5 or 6 plus
+    16 p: that tile with p runs along k, for measurements); 0 chooses by shape.
     `scratch` (float32, on the device): with it, a bf16 product of more than 16 rows with too
     few tiles to fill the chip is cut along k into runs that a second kernel sums in a fixed order.
     """

@@ -145,13 +145,16 @@ def test_gemm_streaming_kernel_rows_and_strides():
         K.gemm(rnd(4, 960, dtype=torch.bfloat16), rnd(N, 960, dtype=torch.bfloat16), torch.empty(4, N, device=DEV), kernel=7)
 
 
-@pytest.mark.parametrize("kernel", [0, 3, 8])
+@pytest.mark.parametrize("kernel", [0, 3, 8, 5 + 16 * 2, 6 + 16 * 4])      # 16 * p: the tile kernel with p runs, forced
 @pytest.mark.parametrize("M,N,Kd", [(17, 520, 1536), (40, 300, 4096), (64, 4096, 2048), (33, 1000, 1032), (64, 96, 8192),
                                     (100, 520, 4096), (300, 260, 2048), (129, 1000, 1024)])
 def test_gemm_split_along_k_with_scratch(M, N, Kd, kernel):
-    if kernel != 0 and M > 64:
-        pytest.skip("more than 64 rows: the tiles, chosen by shape")
-    _skip_unless_kernel_takes(kernel, M, Kd)
+    if kernel in (3, 8) and M > 64:
+        pytest.skip("more than 64 rows: the tiles")
+    if kernel >= 16 and Kd % 64:
+        pytest.skip("the direct-to-LDS tile kernels take K in steps of 64")
+    if kernel < 16:
+        _skip_unless_kernel_takes(kernel, M, Kd)
     a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
     want = a.double() @ w.double().T
     scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
@@ -169,8 +172,12 @@ def test_gemm_split_along_k_with_scratch(M, N, Kd, kernel):
     K.gemm(a, w, acc[:, 3:3 + N], accumulate=True, scratch=scratch, kernel=kernel)
     assert (acc[:, 3:3 + N].double() - (base[:, 3:3 + N].double() + want)).abs().max() < 1e-4 * want.abs().max()
     assert torch.equal(acc[:, :3], base[:, :3]) and torch.equal(acc[:, 3 + N:], base[:, 3 + N:])
-    # too little scratch: the product is not split, and is right all the same
     small = torch.empty(16, device=DEV)
+    if kernel >= 16:
+        with pytest.raises(KernelError):                 # forced runs need their room
+            K.gemm(a, w, again, scratch=small, kernel=kernel)
+        return
+    # too little scratch: the product is not split, and is right all the same
     K.gemm(a, w, again, scratch=small, kernel=kernel)
     assert (again.double() - want).abs().max() < 1e-4 * want.abs().max()
 
