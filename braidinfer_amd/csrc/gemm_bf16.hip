@@ -792,10 +792,31 @@ static int split_parts(int M, int N, int K, int mode, size_t scratch_bytes) {
 // inside a tile; at a tile's end the waves' sums meet in LDS (one barrier, two buffers)
 // and are added in wave order.  The 16-byte columns of a row are XOR-swizzled by the row
 // number through the choice of the global column a lane fetches.
-template <int RT, int XR, int KC, int S, int NW, int MODE>
+//
+// Two forms serve the RMS norm between a product that adds into the residual stream and the
+// product that reads the normed rows, so that single-token steps launch no norm kernel
+// (reference: op_rmsnorm, kernels/megakernel_ops.hip:1421-1446, a step of its own there):
+//  * NORM = 1, the producer (with the accumulate epilogue): it reads the element it adds to,
+//    writes the sum h back, writes bf16(h * g) (g: the next norm's weights) to `xg`, and the
+//    sum of h^2 over its tile's 16 columns to ssq[tile * 16 + row].
+//  * NORM = 2, the consumer: its activations are those bf16(h * g) rows; before its first
+//    tile it adds the `ssq_tiles` sums of every row in a fixed order, and 1 / rms, the same
+//    for a whole row, multiplies the sums at a tile's end:
+//    y = rsqrt(mean(h^2) + eps) * sum_k W[n,k] (h[k] g[k]).
+struct StreamNorm {
+    const float* gain;     // producer: the next norm's weights [N]
+    bf16* xg;              // producer: [M, ldx]
+    size_t ldx;
+    float* ssq;            // producer writes, consumer reads: [tiles, 16]
+    int ssq_tiles;         // consumer: tiles of the producer
+    float inv_k, eps;      // consumer: 1 / width of the normed rows, the norm's eps
+};
+
+template <int RT, int XR, int KC, int S, int NW, int MODE, int NORM>
 __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                               void* __restrict__ C, int M, int N, int K, size_t lda,
-                                                              size_t ldc, int ntiles) {
+                                                              size_t ldc, int ntiles, StreamNorm nrm) {
+    static_assert(NORM == 0 || (NORM == 1 && MODE == OUT_F32_ACC) || (NORM == 2 && MODE != OUT_F32_ACC), "norm forms");
     constexpr int STEPS = KC / 32;
     constexpr int ROWB = KC * 2;
     constexpr int STAGE = (RT + XR) * ROWB;
@@ -808,6 +829,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
     static_assert(RPI >= 1 && (D - 1) * LPI <= 63, "wait count");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     float* red = (float*)(smem + NW * S * STAGE);       // [2][NW][16][17]
+    float* rstd = red + 2 * NW * 16 * 17;               // NORM 2: [16]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
@@ -853,6 +875,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 #pragma unroll
     for (int j = 0; j < D; ++j)
         if (j < nitems) ISSUE(j);
+    if constexpr (NORM == 2) {
+        // row m = tid / 32: its 32 lanes take the tiles' sums in turn, then a butterfly; read at the first tile's end
+        const int m = tid >> 5, l = tid & 31;
+        float t = 0.f;
+        if (m < M)
+            for (int c = l; c < nrm.ssq_tiles; c += 32) t += nrm.ssq[(size_t)c * 16 + m];
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+        if (l == 0) rstd[m] = m < M ? rsqrtf(t * nrm.inv_k + nrm.eps) : 0.f;
+    }
 
     for (int base = 0; base < nitems; base += S) {
 #pragma unroll
@@ -897,8 +929,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
                                 float gv = 0.f, uv = 0.f;
 #pragma unroll
                                 for (int w = 0; w < NW; ++w) { gv += rb[(w * 16 + jl) * 17 + m]; uv += rb[(w * 16 + jl + 8) * 17 + m]; }
+                                if (NORM == 2) { gv *= rstd[m]; uv *= rstd[m]; }
                                 ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
                             }
+                        }
+                    } else if (NORM == 1) {
+                        // whole waves (16 lanes a row): the row's 16 squares of this tile are added by shuffles
+                        if (tid < 16 * XR) {
+                            const int m = tid >> 4, nl = tid & 15, n = n0 + nl;
+                            const bool ok = m < M && n < N;
+                            float h = 0.f;
+                            if (ok) {
+                                float v = 0.f;
+#pragma unroll
+                                for (int w = 0; w < NW; ++w) v += rb[(w * 16 + nl) * 17 + m];
+                                const size_t idx = (size_t)m * ldc + n;
+                                h = ((float*)C)[idx] + v;
+                                ((float*)C)[idx] = h;
+                                nrm.xg[(size_t)m * nrm.ldx + n] = (bf16)(h * nrm.gain[n]);
+                            }
+                            float sq = h * h;
+#pragma unroll
+                            for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+                            if (nl == 0 && m < M) nrm.ssq[(size_t)(n0 / 16) * 16 + m] = sq;
                         }
                     } else {
                         for (int e = tid; e < RT * 16; e += NW * 64) {
@@ -907,6 +960,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
                                 float v = 0.f;
 #pragma unroll
                                 for (int w = 0; w < NW; ++w) v += rb[(w * 16 + nl) * 17 + m];
+                                if (NORM == 2) v *= rstd[m];
                                 const size_t idx = (size_t)m * ldc + n;
                                 if (MODE == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
                                 else if (MODE == OUT_F32) ((float*)C)[idx] = v;
@@ -928,18 +982,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 
 #define STREAM_KC 128
 #define STREAM_NW 8
-template <int XR>
+template <int XR, int NORM>
 static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
-                         int mode, hipStream_t s) {
+                         int mode, hipStream_t s, StreamNorm nrm = StreamNorm{}) {
     constexpr int RT = 16, KC = STREAM_KC, S = 2, NW = STREAM_NW;
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
     const int ntiles = (N + RT - 1) / RT;
     const int grid = ntiles < cus ? ntiles : cus;
-    constexpr size_t lds = (size_t)NW * S * (RT + XR) * KC * 2 + 2 * NW * 16 * 17 * 4;
+    constexpr size_t lds = (size_t)NW * S * (RT + XR) * KC * 2 + 2 * NW * 16 * 17 * 4 + 16 * 4;
 #define BR_STREAM(MODE_)                                                                                        \
     do {                                                                                                        \
-        auto kern = gemm_stream_kernel<RT, XR, KC, S, NW, MODE_>;                                               \
+        auto kern = gemm_stream_kernel<RT, XR, KC, S, NW, MODE_, NORM>;                                         \
         static bool set = false;                                                                                \
         if (!set) {                                                                                             \
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != \
@@ -947,12 +1001,17 @@ static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, in
                 return BR_LAUNCH_FAILED;                                                                        \
             set = true;                                                                                         \
         }                                                                                                       \
-        kern<<<grid, NW * 64, lds, s>>>(A, W, C, M, N, K, lda, ldc, ntiles);                                    \
+        kern<<<grid, NW * 64, lds, s>>>(A, W, C, M, N, K, lda, ldc, ntiles, nrm);                               \
     } while (0)
-    if (mode == OUT_BF16) BR_STREAM(OUT_BF16);
-    else if (mode == OUT_F32) BR_STREAM(OUT_F32);
-    else if (mode == OUT_F32_ACC) BR_STREAM(OUT_F32_ACC);
-    else BR_STREAM(OUT_SWIGLU);
+    if constexpr (NORM == 1) {
+        BR_STREAM(OUT_F32_ACC);
+    } else {
+        if (mode == OUT_BF16) BR_STREAM(OUT_BF16);
+        else if (mode == OUT_F32) BR_STREAM(OUT_F32);
+        else if (mode == OUT_SWIGLU) BR_STREAM(OUT_SWIGLU);
+        else if constexpr (NORM == 0) BR_STREAM(OUT_F32_ACC);
+        else return BR_BAD_ARG;
+    }
 #undef BR_STREAM
     return br_check_launch();
 }
@@ -1193,8 +1252,8 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel == 8)
         return M <= 32 ? launch_stream_wide<2>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s)
                        : launch_stream_wide<4>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s);
-    if (kernel == 7) return M <= 8 ? launch_stream<8>(A, W, C, M, N, K, lda, ldc, mode, s)
-                                   : launch_stream<16>(A, W, C, M, N, K, lda, ldc, mode, s);
+    if (kernel == 7) return M <= 8 ? launch_stream<8, 0>(A, W, C, M, N, K, lda, ldc, mode, s)
+                                   : launch_stream<16, 0>(A, W, C, M, N, K, lda, ldc, mode, s);
     int parts = 1;
     if (chosen && (kernel == 5 || kernel == 6)) {
         const int cus = br_device_cus();
@@ -1240,4 +1299,38 @@ extern "C" int br_gemm_bf16_tile_choice(int M, int N, int K, size_t scratch_byte
     if (!cus) return BR_LAUNCH_FAILED;
     choose_tile(M, N, K, cus, scratch_bytes, kernel, parts);
     return BR_OK;
+}
+
+static bool stream_takes(const void* A, const void* W, int M, int K, size_t lda) {
+    return M > 0 && M <= 16 && K % STREAM_KC == 0 && K / STREAM_KC >= STREAM_NW && lda % 8 == 0 && lda >= (size_t)K &&
+           ((uintptr_t)A | (uintptr_t)W) % 16 == 0;
+}
+
+// C += A W^T through gemm_stream, which then also prepares the RMS norm that reads C next:
+// xg[M, ldx] = bf16(C * gain), ssq[(N / 16) * 16] = sums of squares per tile and row (see the
+// kernel).  M <= 16, N in steps of 16, K as for kernel 7; refuses (BR_BAD_ARG) anything else.
+extern "C" int br_gemm_bf16_norm_prepare(const void* A, const void* W, float* C, int M, int N, int K, size_t lda,
+                                         size_t ldc, const float* gain, void* xg, size_t ldx, float* ssq,
+                                         hipStream_t s) {
+    if (M <= 0 || N <= 0) return BR_OK;
+    if (!stream_takes(A, W, M, K, lda) || N % 16 || ldc < (size_t)N || ldx < (size_t)N || !gain || !xg || !ssq)
+        return BR_BAD_ARG;
+    StreamNorm nrm{gain, (bf16*)xg, ldx, ssq, 0, 0.f, 0.f};
+    return M <= 8 ? launch_stream<8, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm)
+                  : launch_stream<16, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm);
+}
+
+// C = rsqrt(sum of the ssq tiles / norm_width + eps) * (XG W^T), XG and ssq from br_gemm_bf16_norm_prepare:
+// the product of the normed rows.  mode: 0 bf16, 1 float, 3 SwiGLU.
+extern "C" int br_gemm_bf16_norm_scaled(const void* XG, const void* W, void* C, int M, int N, int K, size_t lda,
+                                        size_t ldc, int mode, const float* ssq, int ssq_tiles, int norm_width,
+                                        float eps, hipStream_t s) {
+    if (M <= 0 || N <= 0) return BR_OK;
+    if (!stream_takes(XG, W, M, K, lda) || !ssq || ssq_tiles <= 0 || norm_width <= 0 ||
+        (mode != OUT_BF16 && mode != OUT_F32 && mode != OUT_SWIGLU))
+        return BR_BAD_ARG;
+    if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
+    StreamNorm nrm{nullptr, nullptr, 0, (float*)ssq, ssq_tiles, 1.f / (float)norm_width, eps};
+    return M <= 8 ? launch_stream<8, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm)
+                  : launch_stream<16, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm);
 }

@@ -145,8 +145,15 @@ class DecoderModel:
         for name, enc in self.positions.items():
             step.position_data[name] = enc.prepare(step)
             enc.add_to_embedding(x, step)
+        step.prepared_norm = None
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
+            # the norm that reads the residual rows after this layer: the next scheduled layer's first
+            # (the final norm reads chosen rows only and is left alone)
+            step.norm_after_layer = None
+            if i + 1 < len(self.schedule):
+                nxt = self.layers[self.schedule[i + 1].layer]
+                step.norm_after_layer = nxt.mixer_norm if nxt.mixer is not None else nxt.ffn_norm
             ctx = MixerContext(unit=e.cache, writes_cache=e.writes_cache)
             if layer.mixer is not None:
                 if e.cache is not None and e.cache in cache.group_of_unit:

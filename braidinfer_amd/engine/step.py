@@ -55,6 +55,10 @@ class StepBatch:
     max_ctx_bound: int = 0           # an upper bound of max_ctx that kernels may size their grids by
     ws: Optional[Workspace] = None
     position_data: Dict[str, Any] = field(default_factory=dict)
+    # between the parts of a step: the norm that reads the residual rows after the running layer, and
+    # what the last product into the rows prepared for a norm, as (norm, rows, preparation)
+    norm_after_layer: Any = None
+    prepared_norm: Any = None
     extras: Dict[str, Any] = field(default_factory=dict)     # per-step scratch of parts (keyed by them)
 
 

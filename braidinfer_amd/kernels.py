@@ -238,6 +238,53 @@ def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: 
              0 if scratch is None else scratch.numel() * 4, _stream()), "gemm_swiglu")
 
 
+def gemm_stream_takes(M: int, K: int) -> bool:
+    """Whether the streaming product (kernel 7 of `gemm`, and the two forms below) takes M
+    rows over K: up to 16 rows, K in steps of 128 from 1024."""
+    return 0 < M <= 16 and K % 128 == 0 and K >= 1024
+
+
+def gemm_norm_prepare(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, xg: torch.Tensor,
+                      ssq: torch.Tensor) -> None:
+    """x += a @ w^T (x float32: rows of the residual stream) and, in the same kernel, what
+    the RMS norm that reads x next needs: xg = bfloat16(x * gain) and, in ssq[N / 16, 16],
+    the sums of x^2 per 16 columns and row.  `gemm_norm_scaled` takes both."""
+    _dev("gemm_norm_prepare", a, w, x, gain, xg, ssq)
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a.dtype == w.dtype == xg.dtype == torch.bfloat16 and x.dtype == gain.dtype == ssq.dtype == torch.float32,
+         "gemm_norm_prepare: bfloat16 product into float32 rows")
+    _req(gemm_stream_takes(M, K) and N % 16 == 0, f"gemm_norm_prepare: {M} rows, N {N}, K {K} are not taken")
+    _req(w.shape[1] == K and x.shape == (M, N) and xg.shape == (M, N) and gain.numel() == N and ssq.numel() >= N,
+         "gemm_norm_prepare: shapes")
+    f = _fn("gemm_bf16", "br_gemm_bf16_norm_prepare",
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, _P, _P, c_size_t, _P, _P])
+    _check(f(_ptr(a), _ptr(w), _ptr(x), M, N, K, a.stride(0) if M > 1 else K, x.stride(0) if M > 1 else N, _ptr(gain),
+             _ptr(xg), xg.stride(0) if M > 1 else N, _ptr(ssq), _stream()), "gemm_norm_prepare")
+
+
+def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
+                     swiglu: bool = False) -> None:
+    """out = rmsnorm(x) @ w^T from what `gemm_norm_prepare` left: xg = bfloat16(x * gain)
+    [M, K] and the sums of squares ssq [K / 16, 16]; 1 / rms multiplies the product's sums.
+    `out` bfloat16 or float32 [M, N]; with `swiglu`, bfloat16 [M, N / 2] as `gemm_swiglu`."""
+    _dev("gemm_norm_scaled", xg, ssq, w, out)
+    M, K = xg.shape
+    N = w.shape[0]
+    _req(xg.dtype == w.dtype == torch.bfloat16 and ssq.dtype == torch.float32, "gemm_norm_scaled: bfloat16 rows and matrix")
+    _req(gemm_stream_takes(M, K) and K % 16 == 0 and w.shape[1] == K and ssq.numel() >= K, "gemm_norm_scaled: sizes")
+    if swiglu:
+        _req(out.dtype == torch.bfloat16 and N % 16 == 0 and out.shape == (M, N // 2), "gemm_norm_scaled: SwiGLU gives bfloat16 [M, N / 2]")
+        mode = 3
+    else:
+        _req(out.shape == (M, N) and out.dtype in (torch.bfloat16, torch.float32), "gemm_norm_scaled: out must be [M, N]")
+        mode = 0 if out.dtype == torch.bfloat16 else 1
+    f = _fn("gemm_bf16", "br_gemm_bf16_norm_scaled",
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P, c_int, c_int, c_float, _P])
+    _check(f(_ptr(xg), _ptr(w), _ptr(out), M, N, K, xg.stride(0) if M > 1 else K, out.stride(0) if M > 1 else out.shape[1],
+             mode, _ptr(ssq), K // 16, K, float(eps), _stream()), "gemm_norm_scaled")
+
+
 def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:
     """[2 I, K]: blocks of 8 gate rows followed by the 8 up rows of the same outputs."""
     I, K = w_gate.shape

@@ -39,6 +39,7 @@ def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
 
 class GQAAttention(Mixer):
     graph_safe = True
+    through_linear_only = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: Optional[int] = None, position: Optional[str] = "rope", scale: Optional[float] = None):

@@ -48,6 +48,11 @@ class Part:
     that decide anything on the host from the step's contents leave it False."""
 
     graph_safe = False
+    # A mixer or feed-forward that reads its input and adds to the residual stream only
+    # through `parts.linear.linear` sets this.  It may then be handed a `NormedInput`
+    # instead of the normed rows and a `ResidualSink` instead of the residual tensor, which
+    # lets the product that adds into the stream prepare the norm that reads it next.
+    through_linear_only = False
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         return []
@@ -59,6 +64,43 @@ class Part:
 class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
+
+    def prepare_in_product(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, ws) -> Any:
+        """x += a @ w^T with this norm of the new x prepared in the same kernel, if the norm
+        has such a kernel for these sizes and types: returns what `product_of_prepared`
+        takes, or None with nothing done."""
+        return None
+
+    def product_of_prepared(self, prepared: Any, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> bool:
+        """out = norm(x) @ w^T from what `prepare_in_product` left; False with nothing done
+        if there is no kernel for these sizes."""
+        return False
+
+
+class ResidualSink:
+    """The residual rows as a part that adds to them sees them, with the norm that reads them
+    next.  `linear(a, w, sink, ws, accumulate=True)` adds the product and, where the norm
+    can, leaves its preparation in `prepared`."""
+
+    def __init__(self, x: torch.Tensor, next_norm: Optional["Norm"]):
+        self.x, self.next_norm, self.prepared = x, next_norm, None
+
+
+class NormedInput:
+    """The input of a mixer or feed-forward before its norm has run: the residual rows, the
+    norm, and what the product before may have prepared for it.  `linear(h, w, out, ws)`
+    multiplies the normed rows with a matrix, from the preparation where there is one;
+    `tensor` norms into a buffer (once) for everything else."""
+
+    def __init__(self, x: torch.Tensor, norm: "Norm", ws, dtype: torch.dtype, prepared: Any = None):
+        self.x, self.norm, self.ws, self.dtype, self.prepared = x, norm, ws, dtype, prepared
+        self._tensor: Optional[torch.Tensor] = None
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = self.ws.get("block_h", tuple(self.x.shape), self.dtype)
+            self.norm.forward(self.x, self._tensor)
+        return self._tensor
 
 
 class PositionEncoding(Part):

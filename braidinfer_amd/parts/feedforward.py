@@ -9,12 +9,13 @@ import torch
 
 from .. import kernels as K
 from ..weights import TensorSpec
-from .base import FeedForward, Runtime, register_part
+from .base import FeedForward, NormedInput, Runtime, register_part
 from .linear import fuse_rows, linear
 
 
 class SwiGLU(FeedForward):
     graph_safe = True
+    through_linear_only = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.H, self.I = int(hidden_size), int(intermediate_size)
@@ -41,8 +42,14 @@ class SwiGLU(FeedForward):
         dt = self.rt.dtype
         a = step.ws.get("ffn_act", (T, self.I), dt)
         if self.fused:
-            scratch = step.ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if 64 < T <= 1024 else None
-            K.gemm_swiglu(h, self.w_gu, a, scratch=scratch)
+            if isinstance(h, NormedInput):
+                if h.prepared is not None and h.norm.product_of_prepared(h.prepared, self.w_gu, a, swiglu=True):
+                    h = None
+                else:
+                    h = h.tensor()
+            if h is not None:
+                scratch = step.ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if 64 < T <= 1024 else None
+                K.gemm_swiglu(h, self.w_gu, a, scratch=scratch)
         else:
             gu = step.ws.get("ffn_gu", (T, 2 * self.I), dt)
             linear(h, self.w_gu, gu, step.ws)

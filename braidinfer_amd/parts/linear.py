@@ -8,10 +8,26 @@ from __future__ import annotations
 import torch
 
 from .. import kernels as K
+from .base import NormedInput, ResidualSink
 
 
-def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, ws, accumulate: bool = False) -> None:
-    """out (+)= a @ w^T.  `accumulate` needs a float32 `out`."""
+def linear(a, w: torch.Tensor, out, ws, accumulate: bool = False) -> None:
+    """out (+)= a @ w^T.  `accumulate` needs a float32 `out`.
+
+    `a` may be a `NormedInput` (the product is then taken of the normed rows, from what the
+    product before prepared where it did) and `out` a `ResidualSink` (the product is added
+    to its rows and, where the next norm can, prepares that norm in the same kernel)."""
+    if isinstance(a, NormedInput):
+        if a.prepared is not None and not accumulate and not isinstance(out, ResidualSink) \
+                and a.norm.product_of_prepared(a.prepared, w, out):
+            return
+        a = a.tensor()
+    if isinstance(out, ResidualSink):
+        sink, out = out, out.x
+        if accumulate and sink.next_norm is not None:
+            sink.prepared = sink.next_norm.prepare_in_product(a, w, out, ws)
+            if sink.prepared is not None:
+                return
     if a.dtype == w.dtype:
         if a.dtype == torch.float32 or out.dtype == torch.float32 or not accumulate:
             if a.dtype == torch.float32 and out.dtype != torch.float32:

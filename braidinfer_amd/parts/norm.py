@@ -29,5 +29,23 @@ class RMSNorm(Norm):
         K.rmsnorm(x, self.weight, out, self.eps, rows)
         return out
 
+    def prepare_in_product(self, a, w, x, ws):
+        M, N = x.shape
+        if not (a.dtype == w.dtype == torch.bfloat16 and x.dtype == torch.float32 and N == self.size and N % 16 == 0
+                and K.gemm_stream_takes(M, a.shape[1]) and K.gemm_stream_takes(M, N) and a.is_contiguous()
+                and x.is_contiguous()):
+            return None
+        xg = ws.get("norm_xg", (M, N), torch.bfloat16)
+        ssq = ws.get("norm_ssq", (N,), torch.float32)
+        K.gemm_norm_prepare(a, w, x, self.weight, xg, ssq)
+        return xg, ssq
+
+    def product_of_prepared(self, prepared, w, out, swiglu=False):
+        xg, ssq = prepared
+        if w.dtype != torch.bfloat16 or (not swiglu and out.dtype not in (torch.bfloat16, torch.float32)):
+            return False
+        K.gemm_norm_scaled(xg, ssq, self.eps, w, out, swiglu=swiglu)
+        return True
+
 
 register_part("norm", "rmsnorm", RMSNorm, replace=True)

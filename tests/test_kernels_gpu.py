@@ -182,6 +182,50 @@ def test_gemm_split_along_k_with_scratch(M, N, Kd, kernel):
     assert (again.double() - want).abs().max() < 1e-4 * want.abs().max()
 
 
+@pytest.mark.parametrize("M,H,Kd,N2", [(1, 1024, 1024, 304), (8, 1152, 2048, 4112), (13, 2048, 1280, 96), (16, 1024, 1536, 1000)])
+def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
+    # x += a W1^T, then rmsnorm(x) W2^T, in two kernels instead of three
+    a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
+    w1 = rnd(H, Kd, seed=2, scale=0.05, dtype=torch.bfloat16)
+    w2 = rnd(N2, H, seed=3, scale=0.5, dtype=torch.bfloat16)
+    x0 = rnd(M, H, seed=4) * torch.logspace(-1, 1, M, device=DEV)[:, None]     # rows of very different sizes
+    gain = 1.0 + 0.5 * rnd(H, seed=5)
+    eps = 1e-5
+    x = x0.clone()
+    xg = torch.empty(M, H, device=DEV, dtype=torch.bfloat16)
+    ssq = torch.full((H,), float("nan"), device=DEV)
+    K.gemm_norm_prepare(a, w1, x, gain, xg, ssq)
+    xw = x0.double() + a.double() @ w1.double().T
+    assert (x.double() - xw).abs().max() < 1e-4 * xw.abs().max()
+    assert (xg.double() - xw * gain.double()).abs().max() < 1e-2 * (xw * gain.double()).abs().max()
+    tiles = ssq.view(H // 16, 16)[:, :M].double()
+    assert (tiles.sum(0) - (xw * xw).sum(-1)).abs().max() < 1e-4 * (xw * xw).sum(-1).max()
+    normed = xw / torch.sqrt((xw * xw).mean(-1, keepdim=True) + eps) * gain.double()
+    want = normed @ w2.double().T
+    o32 = torch.empty(M, N2, device=DEV)
+    K.gemm_norm_scaled(xg, ssq, eps, w2, o32)
+    assert (o32.double() - want).abs().max() < 1e-2 * want.abs().max()
+    # against the same product with the rows normed by the norm kernel: bf16 roundings apart
+    h = torch.empty(M, H, device=DEV, dtype=torch.bfloat16)
+    K.rmsnorm(x, gain, h, eps, None)
+    two = torch.empty(M, N2, device=DEV)
+    K.gemm(h, w2, two)
+    assert (o32 - two).abs().max() < 1e-2 * want.abs().max()
+    o16 = torch.empty(M, N2, device=DEV, dtype=torch.bfloat16)
+    K.gemm_norm_scaled(xg, ssq, eps, w2, o16)
+    assert (o16.double() - want).abs().max() < 2e-2 * want.abs().max()
+    if N2 % 16 == 0:
+        out = torch.empty(M, N2 // 2, device=DEV, dtype=torch.bfloat16)
+        K.gemm_norm_scaled(xg, ssq, eps, w2, out, swiglu=True)
+        gu = want.view(M, N2 // 16, 2, 8)
+        g, u = gu[:, :, 0].reshape(M, -1), gu[:, :, 1].reshape(M, -1)
+        sw = g / (1 + torch.exp(-g)) * u
+        assert (out.double() - sw).abs().max() < 2e-2 * sw.abs().max()
+    with pytest.raises(KernelError):
+        K.gemm_norm_prepare(rnd(17, Kd, dtype=torch.bfloat16), w1, torch.zeros(17, H, device=DEV), gain,
+                            torch.empty(17, H, device=DEV, dtype=torch.bfloat16), ssq)
+
+
 def test_gemm_reference_vectors():
     # tests/wmma_gemm_test.rs:27-69,72-114: sin/cos ramps times 0.5 / 0.3, tol 1e-3
     for M, N, Kd in ((32, 32, 64), (256, 256, 1024)):
