@@ -417,3 +417,39 @@ def test_single_token_steps_launch_few_norm_kernels(serving, monkeypatch):
     eng.step([StepEntry(s, [5], [0])])
     assert len(calls) == 2
     eng.free_slot(s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_serving_sizes_random_schedule(serving, dtype):
+    """The random schedule at the sizes that take the serving kernels: up to 30 requests live,
+    so steps bring 1 to 16, 17 to 64 and more rows; chunks of 1 (mostly), a few, and more than
+    a page."""
+    folder, cfg, w = serving
+    eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=16384)
+    rng = np.random.default_rng(11)
+    free_before = [g.pool.free_count for g in eng.cache.groups]
+    seqs = [tokens(cfg, int(n), 300 + i) for i, n in enumerate(rng.integers(1, 230, 36))]
+    waiting = list(range(len(seqs)))
+    live, pos, got = {}, {}, {i: [] for i in range(len(seqs))}
+    while waiting or live:
+        for i in list(waiting):
+            if len(live) < 30 and rng.random() < 0.6:
+                waiting.remove(i); live[i] = eng.alloc_slot(); pos[i] = 0
+        if not live:
+            continue
+        chosen = [i for i in live if rng.random() < 0.85] or list(live)[:1]
+        single = rng.random() < 0.7                     # mostly steps of one token each, as in generation
+        entries, takes = [], []
+        for i in chosen:
+            n = 1 if single else min(int(rng.choice([1, 3, 17, 64, 70])), len(seqs[i]) - pos[i])
+            entries.append(StepEntry(live[i], seqs[i][pos[i]:pos[i] + n], list(range(n))))
+            takes.append(n)
+        out = eng.step(entries).cpu().numpy()
+        o = 0
+        for i, n in zip(chosen, takes):
+            got[i].append(out[o:o + n]); o += n; pos[i] += n
+            if pos[i] == len(seqs[i]):
+                eng.free_slot(live.pop(i))
+    for i in range(0, len(seqs), 3):                     # every third request against the plain implementation
+        close(np.concatenate(got[i]), P.forward(cfg, w, seqs[i]), dtype, f"request {i} of {len(seqs[i])} tokens")
+    assert [g.pool.free_count for g in eng.cache.groups] == free_before
