@@ -29,6 +29,7 @@
 // out[m][8 b + j] = silu(gate) * up, silu(g) = g / (1 + exp(-g))
 // (reference: kernels/megakernel_ops.hip:1538-1544, fused there too, per output row).
 #define OUT_SWIGLU 3
+#define SSQ_LD 64           // row stride of the sums of squares that a product leaves for the next RMS norm
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
 
@@ -743,6 +744,27 @@ __global__ void gemm_split_sum_kernel(const float* __restrict__ part, int parts,
     store_out<MODE>(C, m * ldc + n, v);
 }
 
+// The sum of the runs added into the residual rows C, with the next RMS norm prepared as by
+// gemm_stream's NORM = 1 form: a workgroup takes 256 consecutive columns of one row (N in
+// steps of 256), writes h = C + sum back, bf16(h * gain) to xg, and the sum of its 256
+// squares to ssq[(column / 256) * SSQ_LD + row].
+__global__ __launch_bounds__(256) void gemm_split_sum_prep_kernel(const float* __restrict__ part, int parts,
+                                                                  size_t part_stride, float* __restrict__ C, int N,
+                                                                  size_t ldc, const float* __restrict__ gain,
+                                                                  bf16* __restrict__ xg, size_t ldx,
+                                                                  float* __restrict__ ssq) {
+    __shared__ float red[16];
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t m = i / N, n = i - m * N;
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += part[p * part_stride + i];
+    const float h = C[m * ldc + n] + v;
+    C[m * ldc + n] = h;
+    xg[m * ldx + n] = (bf16)(h * gain[n]);
+    const float tot = block_sum(h * h, red);
+    if (threadIdx.x == 0) ssq[(n / 256) * SSQ_LD + m] = tot;
+}
+
 static int launch_split_sum(const float* scratch, int parts, void* C, int M, int N, size_t ldc, int mode, hipStream_t s) {
     const size_t stride = (size_t)M * N;
     const unsigned blocks = (unsigned)((stride + 255) / 256);
@@ -798,7 +820,7 @@ static int split_parts(int M, int N, int K, int mode, size_t scratch_bytes) {
 // (reference: op_rmsnorm, kernels/megakernel_ops.hip:1421-1446, a step of its own there):
 //  * NORM = 1, the producer (with the accumulate epilogue): it reads the element it adds to,
 //    writes the sum h back, writes bf16(h * g) (g: the next norm's weights) to `xg`, and the
-//    sum of h^2 over its tile's 16 columns to ssq[tile * 16 + row].
+//    sum of h^2 over its tile's 16 columns to ssq[tile * SSQ_LD + row].
 //  * NORM = 2, the consumer: its activations are those bf16(h * g) rows; before its first
 //    tile it adds the `ssq_tiles` sums of every row in a fixed order, and 1 / rms, the same
 //    for a whole row, multiplies the sums at a tile's end:
@@ -807,7 +829,7 @@ struct StreamNorm {
     const float* gain;     // producer: the next norm's weights [N]
     bf16* xg;              // producer: [M, ldx]
     size_t ldx;
-    float* ssq;            // producer writes, consumer reads: [tiles, 16]
+    float* ssq;            // producer writes, consumer reads: [tiles, SSQ_LD]
     int ssq_tiles;         // consumer: tiles of the producer
     float inv_k, eps;      // consumer: 1 / width of the normed rows, the norm's eps
 };
@@ -880,7 +902,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
         const int m = tid >> 5, l = tid & 31;
         float t = 0.f;
         if (m < M)
-            for (int c = l; c < nrm.ssq_tiles; c += 32) t += nrm.ssq[(size_t)c * 16 + m];
+            for (int c = l; c < nrm.ssq_tiles; c += 32) t += nrm.ssq[(size_t)c * SSQ_LD + m];
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
         if (l == 0) rstd[m] = m < M ? rsqrtf(t * nrm.inv_k + nrm.eps) : 0.f;
@@ -951,7 +973,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
                             float sq = h * h;
 #pragma unroll
                             for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
-                            if (nl == 0 && m < M) nrm.ssq[(size_t)(n0 / 16) * 16 + m] = sq;
+                            if (nl == 0 && m < M) nrm.ssq[(size_t)(n0 / 16) * SSQ_LD + m] = sq;
                         }
                     } else {
                         for (int e = tid; e < RT * 16; e += NW * 64) {
@@ -1028,11 +1050,13 @@ static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, in
 // float sums go to a matrix of its run (`part_stride` elements apart) for
 // gemm_split_sum_kernel; else the epilogue is applied here.
 #define WIDE_S 3
-template <int MB, int MODE, bool PARTIAL>
+// SCALE: the activations are the bf16(h * g) rows that the product before left for an RMS norm
+// (see gemm_stream's NORM forms); the sums are multiplied by 1 / rms of their row, run by run.
+template <int MB, int MODE, bool PARTIAL, bool SCALE>
 __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                                void* __restrict__ C, int M, int N, int K, size_t lda,
                                                                size_t ldc, int ntiles, int parts, int cpp,
-                                                               size_t part_stride) {
+                                                               size_t part_stride, StreamNorm nrm) {
     constexpr int S = WIDE_S, D = S - 1, NW = 8;
     constexpr int ROWS = 64 + 16 * MB;               // stacked rows of a stage: weights, then activations
     constexpr int STAGE = ROWS * 256;
@@ -1041,6 +1065,7 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
     static_assert(STAGE % (1024 * NW) == 0 && (D - 1) * NDMA <= 63, "stage");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     float* red = (float*)(smem + S * STAGE);         // [NW][16][RLD]
+    float* rstd = red + NW * 16 * RLD;               // SCALE: [64]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
@@ -1090,6 +1115,16 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
 
     for (int j = 0; j < D; ++j)
         if (is_u < my_units) WIDE_ISSUE();
+    if constexpr (SCALE) {
+        // row m = tid / 8: its 8 lanes take the tiles' sums in turn, then a butterfly; read at the first unit's end
+        const int m = tid >> 3, l = tid & 7;
+        float t = 0.f;
+        if (m < M)
+            for (int c = l; c < nrm.ssq_tiles; c += 8) t += nrm.ssq[(size_t)c * SSQ_LD + m];
+#pragma unroll
+        for (int o = 4; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+        if (l == 0) rstd[m] = m < M ? rsqrtf(t * nrm.inv_k + nrm.eps) : 0.f;
+    }
     while (cp_u < my_units) {
         // the chunk to multiply has landed when at most the loads of the chunks issued after it are in flight
         if (issued - done - 1 >= 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
@@ -1134,8 +1169,9 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
                 const int m = e >> 5, jl = e & 31;
                 const int gr = (jl >> 3) * 16 + (jl & 7);
                 if (m < M && n0 + gr + 8 < N) {
-                    const float gv = red[gr * RLD + m] + red[(64 + gr) * RLD + m];
-                    const float uv = red[(gr + 8) * RLD + m] + red[(64 + gr + 8) * RLD + m];
+                    float gv = red[gr * RLD + m] + red[(64 + gr) * RLD + m];
+                    float uv = red[(gr + 8) * RLD + m] + red[(64 + gr + 8) * RLD + m];
+                    if (SCALE) { gv *= rstd[m]; uv *= rstd[m]; }
                     ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
                 }
             }
@@ -1143,7 +1179,8 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
             for (int e = tid; e < 64 * 16 * MB; e += 512) {
                 const int m = e >> 6, nl = e & 63, n = n0 + nl;
                 if (m < M && n < N) {
-                    const float v = red[nl * RLD + m] + red[(64 + nl) * RLD + m];      // k-half 0, then 1
+                    float v = red[nl * RLD + m] + red[(64 + nl) * RLD + m];      // k-half 0, then 1
+                    if (SCALE) v *= rstd[m];
                     if (PARTIAL) ((float*)C)[part * part_stride + (size_t)m * N + n] = v;
                     else {
                         const size_t idx = (size_t)m * ldc + n;
@@ -1179,22 +1216,29 @@ static int wide_parts(int M, int N, int K, int mode, int cus, size_t scratch_byt
     return best;
 }
 
+// norm: 0 none; 1 the product is added into the residual rows C and prepares the next RMS norm
+// (needs a split product: the sum kernel does it; refused otherwise); 2 the activations were so
+// prepared and the sums are scaled (modes 0, 1, 3).
 template <int MB>
 static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
-                              int mode, float* scratch, size_t scratch_bytes, hipStream_t s) {
+                              int mode, float* scratch, size_t scratch_bytes, hipStream_t s, int norm = 0,
+                              StreamNorm nrm = StreamNorm{}) {
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
     const int ntiles = (N + 63) / 64, nch = K / 128;
     int parts = scratch ? wide_parts(M, N, K, mode, cus, scratch_bytes) : 1;
+    if (norm == 1 && (parts < 2 || N % 256 || mode != OUT_F32_ACC)) return BR_BAD_ARG;
+    if (norm == 2 && mode == OUT_F32_ACC) return BR_BAD_ARG;
     const int cpp = (nch + parts - 1) / parts;
     parts = (nch + cpp - 1) / cpp;                                   // no empty run
     const long long nunits = (long long)ntiles * parts;
     const int grid = nunits < cus ? (int)nunits : cus;
-    constexpr size_t lds = (size_t)WIDE_S * (64 + 16 * MB) * 256 + 8 * 16 * (16 * MB + 1) * 4;
+    constexpr size_t lds = (size_t)WIDE_S * (64 + 16 * MB) * 256 + 8 * 16 * (16 * MB + 1) * 4 + 64 * 4;
     const size_t stride = (size_t)M * N;
-#define BR_WIDE(MODE_, PARTIAL_, OUT_)                                                                          \
+#define BR_WIDE(MODE_, PARTIAL_, OUT_) do { if (norm == 2) BR_WIDE2(MODE_, PARTIAL_, true, OUT_); else BR_WIDE2(MODE_, PARTIAL_, false, OUT_); } while (0)
+#define BR_WIDE2(MODE_, PARTIAL_, SCALE_, OUT_)                                                                 \
     do {                                                                                                        \
-        auto kern = gemm_stream_wide_kernel<MB, MODE_, PARTIAL_>;                                               \
+        auto kern = gemm_stream_wide_kernel<MB, MODE_, PARTIAL_, SCALE_>;                                       \
         static bool set = false;                                                                                \
         if (!set) {                                                                                             \
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != \
@@ -1202,12 +1246,17 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
                 return BR_LAUNCH_FAILED;                                                                        \
             set = true;                                                                                         \
         }                                                                                                       \
-        kern<<<grid, 512, lds, s>>>(A, W, OUT_, M, N, K, lda, ldc, ntiles, parts, cpp, stride);                 \
+        kern<<<grid, 512, lds, s>>>(A, W, OUT_, M, N, K, lda, ldc, ntiles, parts, cpp, stride, nrm);            \
     } while (0)
     if (parts > 1) {
         BR_WIDE(OUT_F32, true, (void*)scratch);
         int rc = br_check_launch();
         if (rc != BR_OK) return rc;
+        if (norm == 1) {
+            gemm_split_sum_prep_kernel<<<(unsigned)(stride / 256), 256, 0, s>>>(scratch, parts, stride, (float*)C, N, ldc,
+                                                                                nrm.gain, nrm.xg, nrm.ldx, nrm.ssq);
+            return br_check_launch();
+        }
         return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
     }
     if (mode == OUT_BF16) BR_WIDE(OUT_BF16, false, C);
@@ -1215,6 +1264,7 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
     else if (mode == OUT_F32_ACC) BR_WIDE(OUT_F32_ACC, false, C);
     else BR_WIDE(OUT_SWIGLU, false, C);
 #undef BR_WIDE
+#undef BR_WIDE2
     return br_check_launch();
 }
 
@@ -1305,32 +1355,63 @@ static bool stream_takes(const void* A, const void* W, int M, int K, size_t lda)
     return M > 0 && M <= 16 && K % STREAM_KC == 0 && K / STREAM_KC >= STREAM_NW && lda % 8 == 0 && lda >= (size_t)K &&
            ((uintptr_t)A | (uintptr_t)W) % 16 == 0;
 }
+static bool wide_takes(const void* A, const void* W, int M, int K, size_t lda) {
+    return M > 16 && M <= 64 && K % 128 == 0 && K >= 256 && lda % 8 == 0 && lda >= (size_t)K &&
+           ((uintptr_t)A | (uintptr_t)W) % 16 == 0;
+}
 
-// C += A W^T through gemm_stream, which then also prepares the RMS norm that reads C next:
-// xg[M, ldx] = bf16(C * gain), ssq[(N / 16) * 16] = sums of squares per tile and row (see the
-// kernel).  M <= 16, N in steps of 16, K as for kernel 7; refuses (BR_BAD_ARG) anything else.
+// C += A W^T through the streaming products, which then also prepare the RMS norm that reads C
+// next: xg[M, ldx] = bf16(C * gain) and sums of squares in ssq[tiles, SSQ_LD] (see the kernels);
+// *ssq_tiles says how many.  Up to 16 rows: gemm_stream (N in steps of 16).  17 to 64 rows:
+// gemm_stream_wide cut along k, the preparation in the sum kernel (N in steps of 256, scratch
+// needed).  Refuses (BR_BAD_ARG) anything else: the caller then runs the norm itself.
 extern "C" int br_gemm_bf16_norm_prepare(const void* A, const void* W, float* C, int M, int N, int K, size_t lda,
                                          size_t ldc, const float* gain, void* xg, size_t ldx, float* ssq,
-                                         hipStream_t s) {
-    if (M <= 0 || N <= 0) return BR_OK;
-    if (!stream_takes(A, W, M, K, lda) || N % 16 || ldc < (size_t)N || ldx < (size_t)N || !gain || !xg || !ssq)
-        return BR_BAD_ARG;
+                                         int* ssq_tiles, void* scratch, size_t scratch_bytes, hipStream_t s) {
+    if (M <= 0 || N <= 0) return BR_BAD_ARG;
+    if (ldc < (size_t)N || ldx < (size_t)N || !gain || !xg || !ssq || !ssq_tiles) return BR_BAD_ARG;
     StreamNorm nrm{gain, (bf16*)xg, ldx, ssq, 0, 0.f, 0.f};
-    return M <= 8 ? launch_stream<8, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm)
-                  : launch_stream<16, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm);
+    if (stream_takes(A, W, M, K, lda) && N % 16 == 0) {
+        *ssq_tiles = N / 16;
+        return M <= 8 ? launch_stream<8, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm)
+                      : launch_stream<16, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm);
+    }
+    if (wide_takes(A, W, M, K, lda) && N % 256 == 0 && scratch && (uintptr_t)scratch % 16 == 0) {
+        *ssq_tiles = N / 256;
+        return M <= 32 ? launch_stream_wide<2>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC,
+                                               (float*)scratch, scratch_bytes, s, 1, nrm)
+                       : launch_stream_wide<4>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC,
+                                               (float*)scratch, scratch_bytes, s, 1, nrm);
+    }
+    return BR_BAD_ARG;
 }
 
 // C = rsqrt(sum of the ssq tiles / norm_width + eps) * (XG W^T), XG and ssq from br_gemm_bf16_norm_prepare:
 // the product of the normed rows.  mode: 0 bf16, 1 float, 3 SwiGLU.
 extern "C" int br_gemm_bf16_norm_scaled(const void* XG, const void* W, void* C, int M, int N, int K, size_t lda,
                                         size_t ldc, int mode, const float* ssq, int ssq_tiles, int norm_width,
-                                        float eps, hipStream_t s) {
+                                        float eps, void* scratch, size_t scratch_bytes, hipStream_t s) {
     if (M <= 0 || N <= 0) return BR_OK;
-    if (!stream_takes(XG, W, M, K, lda) || !ssq || ssq_tiles <= 0 || norm_width <= 0 ||
-        (mode != OUT_BF16 && mode != OUT_F32 && mode != OUT_SWIGLU))
+    if (!ssq || ssq_tiles <= 0 || norm_width <= 0 || (mode != OUT_BF16 && mode != OUT_F32 && mode != OUT_SWIGLU))
         return BR_BAD_ARG;
     if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
     StreamNorm nrm{nullptr, nullptr, 0, (float*)ssq, ssq_tiles, 1.f / (float)norm_width, eps};
-    return M <= 8 ? launch_stream<8, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm)
-                  : launch_stream<16, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm);
+    if (stream_takes(XG, W, M, K, lda))
+        return M <= 8 ? launch_stream<8, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm)
+                      : launch_stream<16, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm);
+    if (wide_takes(XG, W, M, K, lda)) {
+        float* sc = (scratch && (uintptr_t)scratch % 16 == 0) ? (float*)scratch : nullptr;
+        return M <= 32 ? launch_stream_wide<2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, sc,
+                                               scratch_bytes, s, 2, nrm)
+                       : launch_stream_wide<4>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, sc,
+                                               scratch_bytes, s, 2, nrm);
+    }
+    return BR_BAD_ARG;
+}
+
+// into how many runs along k br_gemm_bf16_ex and br_gemm_bf16_norm_prepare cut a product of 17 to 64 rows
+extern "C" int br_gemm_bf16_wide_parts(int M, int N, int K, int mode, size_t scratch_bytes) {
+    const int cus = br_device_cus();
+    if (!cus || M <= 16 || M > 64 || K % 128 || K < 256) return 0;
+    return wide_parts(M, N, K, mode, cus, scratch_bytes);
 }

@@ -239,40 +239,58 @@ def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: 
 
 
 def gemm_stream_takes(M: int, K: int) -> bool:
-    """Whether the streaming product (kernel 7 of `gemm`, and the two forms below) takes M
-    rows over K: up to 16 rows, K in steps of 128 from 1024."""
-    return 0 < M <= 16 and K % 128 == 0 and K >= 1024
+    """Whether the streaming products (kernels 7 and 8 of `gemm`, and the two forms below)
+    take M rows over K: up to 16 rows with K in steps of 128 from 1024, or 17 to 64 rows with
+    K in steps of 128 from 256."""
+    return (0 < M <= 16 and K % 128 == 0 and K >= 1024) or (16 < M <= 64 and K % 128 == 0 and K >= 256)
+
+
+def gemm_wide_parts(M: int, N: int, K: int, scratch_floats: int, accumulate: bool = True) -> int:
+    """Into how many runs along k a bf16 product of 17 to 64 rows is cut when it is given that
+    much scratch (0: the wide streaming product does not take it)."""
+    f = _fn("gemm_bf16", "br_gemm_bf16_wide_parts", [c_int, c_int, c_int, c_int, c_size_t])
+    return int(f(M, N, K, 2 if accumulate else 1, scratch_floats * 4))
+
+
+SSQ_LD = 64        # row stride of the sums of squares that a product leaves for the next norm (SSQ_LD in csrc/gemm_bf16.hip)
 
 
 def gemm_norm_prepare(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, xg: torch.Tensor,
-                      ssq: torch.Tensor) -> None:
-    """x += a @ w^T (x float32: rows of the residual stream) and, in the same kernel, what
-    the RMS norm that reads x next needs: xg = bfloat16(x * gain) and, in ssq[N / 16, 16],
-    the sums of x^2 per 16 columns and row.  `gemm_norm_scaled` takes both."""
-    _dev("gemm_norm_prepare", a, w, x, gain, xg, ssq)
+                      ssq: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> int:
+    """x += a @ w^T (x float32: rows of the residual stream) and, in the same kernels, what
+    the RMS norm that reads x next needs: xg = bfloat16(x * gain) and, in ssq[tiles, 64],
+    sums of x^2 per row over runs of columns.  Returns the number of tiles; `gemm_norm_scaled`
+    takes all three.  Up to 16 rows: N in steps of 16.  17 to 64 rows: N in steps of 256 and
+    `scratch` (float32, as for `gemm`) for the product's runs along k.  Raises KernelError for
+    anything else."""
+    _dev("gemm_norm_prepare", a, w, x, gain, xg, ssq, scratch)
     M, K = a.shape
     N = w.shape[0]
     _req(a.dtype == w.dtype == xg.dtype == torch.bfloat16 and x.dtype == gain.dtype == ssq.dtype == torch.float32,
          "gemm_norm_prepare: bfloat16 product into float32 rows")
-    _req(gemm_stream_takes(M, K) and N % 16 == 0, f"gemm_norm_prepare: {M} rows, N {N}, K {K} are not taken")
-    _req(w.shape[1] == K and x.shape == (M, N) and xg.shape == (M, N) and gain.numel() == N and ssq.numel() >= N,
-         "gemm_norm_prepare: shapes")
+    _req(gemm_stream_takes(M, K) and N % (16 if M <= 16 else 256) == 0, f"gemm_norm_prepare: {M} rows, N {N}, K {K} are not taken")
+    _req(w.shape[1] == K and x.shape == (M, N) and xg.shape == (M, N) and gain.numel() == N
+         and ssq.numel() >= (N // 16) * SSQ_LD, "gemm_norm_prepare: shapes")
+    tiles = c_int(0)
     f = _fn("gemm_bf16", "br_gemm_bf16_norm_prepare",
-            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, _P, _P, c_size_t, _P, _P])
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, _P, _P, c_size_t, _P, ctypes.POINTER(c_int), _P, c_size_t, _P])
     _check(f(_ptr(a), _ptr(w), _ptr(x), M, N, K, a.stride(0) if M > 1 else K, x.stride(0) if M > 1 else N, _ptr(gain),
-             _ptr(xg), xg.stride(0) if M > 1 else N, _ptr(ssq), _stream()), "gemm_norm_prepare")
+             _ptr(xg), xg.stride(0) if M > 1 else N, _ptr(ssq), ctypes.byref(tiles), _ptr(scratch),
+             0 if scratch is None else scratch.numel() * 4, _stream()), "gemm_norm_prepare")
+    return tiles.value
 
 
-def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
-                     swiglu: bool = False) -> None:
+def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, tiles: int, eps: float, w: torch.Tensor, out: torch.Tensor,
+                     swiglu: bool = False, scratch: Optional[torch.Tensor] = None) -> None:
     """out = rmsnorm(x) @ w^T from what `gemm_norm_prepare` left: xg = bfloat16(x * gain)
-    [M, K] and the sums of squares ssq [K / 16, 16]; 1 / rms multiplies the product's sums.
-    `out` bfloat16 or float32 [M, N]; with `swiglu`, bfloat16 [M, N / 2] as `gemm_swiglu`."""
-    _dev("gemm_norm_scaled", xg, ssq, w, out)
+    [M, K], the sums of squares ssq and their number of tiles; 1 / rms multiplies the
+    product's sums.  `out` bfloat16 or float32 [M, N]; with `swiglu`, bfloat16 [M, N / 2] as
+    `gemm_swiglu`."""
+    _dev("gemm_norm_scaled", xg, ssq, w, out, scratch)
     M, K = xg.shape
     N = w.shape[0]
     _req(xg.dtype == w.dtype == torch.bfloat16 and ssq.dtype == torch.float32, "gemm_norm_scaled: bfloat16 rows and matrix")
-    _req(gemm_stream_takes(M, K) and K % 16 == 0 and w.shape[1] == K and ssq.numel() >= K, "gemm_norm_scaled: sizes")
+    _req(gemm_stream_takes(M, K) and w.shape[1] == K and tiles > 0 and ssq.numel() >= tiles * SSQ_LD, "gemm_norm_scaled: sizes")
     if swiglu:
         _req(out.dtype == torch.bfloat16 and N % 16 == 0 and out.shape == (M, N // 2), "gemm_norm_scaled: SwiGLU gives bfloat16 [M, N / 2]")
         mode = 3
@@ -280,9 +298,10 @@ def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, eps: float, w: torch.T
         _req(out.shape == (M, N) and out.dtype in (torch.bfloat16, torch.float32), "gemm_norm_scaled: out must be [M, N]")
         mode = 0 if out.dtype == torch.bfloat16 else 1
     f = _fn("gemm_bf16", "br_gemm_bf16_norm_scaled",
-            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P, c_int, c_int, c_float, _P])
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P, c_int, c_int, c_float, _P, c_size_t, _P])
     _check(f(_ptr(xg), _ptr(w), _ptr(out), M, N, K, xg.stride(0) if M > 1 else K, out.stride(0) if M > 1 else out.shape[1],
-             mode, _ptr(ssq), K // 16, K, float(eps), _stream()), "gemm_norm_scaled")
+             mode, _ptr(ssq), int(tiles), K, float(eps), _ptr(scratch), 0 if scratch is None else scratch.numel() * 4,
+             _stream()), "gemm_norm_scaled")
 
 
 def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:

@@ -31,20 +31,24 @@ class RMSNorm(Norm):
 
     def prepare_in_product(self, a, w, x, ws):
         M, N = x.shape
-        if not (a.dtype == w.dtype == torch.bfloat16 and x.dtype == torch.float32 and N == self.size and N % 16 == 0
-                and K.gemm_stream_takes(M, a.shape[1]) and K.gemm_stream_takes(M, N) and a.is_contiguous()
-                and x.is_contiguous()):
+        if not (a.dtype == w.dtype == torch.bfloat16 and x.dtype == torch.float32 and N == self.size
+                and N % (16 if M <= 16 else 256) == 0 and K.gemm_stream_takes(M, a.shape[1])
+                and K.gemm_stream_takes(M, N) and a.is_contiguous() and x.is_contiguous()):
+            return None
+        # 17 to 64 rows: the preparation rides on the sum of a product cut along k
+        if M > 16 and K.gemm_wide_parts(M, N, a.shape[1], K.GEMM_SCRATCH_FLOATS) < 2:
             return None
         xg = ws.get("norm_xg", (M, N), torch.bfloat16)
-        ssq = ws.get("norm_ssq", (N,), torch.float32)
-        K.gemm_norm_prepare(a, w, x, self.weight, xg, ssq)
-        return xg, ssq
+        ssq = ws.get("norm_ssq", ((N // 16) * K.SSQ_LD,), torch.float32)
+        scratch = ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if M > 16 else None
+        tiles = K.gemm_norm_prepare(a, w, x, self.weight, xg, ssq, scratch)
+        return xg, ssq, tiles, scratch
 
     def product_of_prepared(self, prepared, w, out, swiglu=False):
-        xg, ssq = prepared
+        xg, ssq, tiles, scratch = prepared
         if w.dtype != torch.bfloat16 or (not swiglu and out.dtype not in (torch.bfloat16, torch.float32)):
             return False
-        K.gemm_norm_scaled(xg, ssq, self.eps, w, out, swiglu=swiglu)
+        K.gemm_norm_scaled(xg, ssq, tiles, self.eps, w, out, swiglu=swiglu, scratch=scratch)
         return True
 
 

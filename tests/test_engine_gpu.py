@@ -401,9 +401,9 @@ def test_serving_sizes_whole_then_one_by_one_then_batched(serving, dtype):
 
 
 def test_single_token_steps_launch_few_norm_kernels(serving, monkeypatch):
-    """bfloat16, one token per sequence, sizes the streaming product takes: only the first
+    """bfloat16, steps of up to 64 rows, sizes the streaming products take: only the first
     layer's first norm and the final norm run as kernels of their own; the others are prepared
-    by the product before them.  A prompt runs all five."""
+    by the product before them.  A longer prompt runs all five."""
     from braidinfer_amd import kernels as K
     folder, cfg, w = serving
     eng = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=1024, use_graphs=False)
@@ -411,10 +411,13 @@ def test_single_token_steps_launch_few_norm_kernels(serving, monkeypatch):
     real = K.rmsnorm
     monkeypatch.setattr(K, "rmsnorm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
     s = eng.alloc_slot()
-    eng.step([StepEntry(s, tokens(cfg, 40, 1), [39])])
+    eng.step([StepEntry(s, tokens(cfg, 100, 1), [99])])
     assert len(calls) == 2 * cfg["num_hidden_layers"] + 1
     calls.clear()
     eng.step([StepEntry(s, [5], [0])])
+    assert len(calls) == 2
+    calls.clear()
+    eng.step([StepEntry(s, tokens(cfg, 40, 2), [39])])
     assert len(calls) == 2
     eng.free_slot(s)
 

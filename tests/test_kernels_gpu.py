@@ -182,7 +182,8 @@ def test_gemm_split_along_k_with_scratch(M, N, Kd, kernel):
     assert (again.double() - want).abs().max() < 1e-4 * want.abs().max()
 
 
-@pytest.mark.parametrize("M,H,Kd,N2", [(1, 1024, 1024, 304), (8, 1152, 2048, 4112), (13, 2048, 1280, 96), (16, 1024, 1536, 1000)])
+@pytest.mark.parametrize("M,H,Kd,N2", [(1, 1024, 1024, 304), (8, 1152, 2048, 4112), (13, 2048, 1280, 96), (16, 1024, 1536, 1000),
+                                       (17, 1024, 2048, 304), (40, 2048, 1024, 4112), (64, 1280, 4096, 96)])
 def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
     # x += a W1^T, then rmsnorm(x) W2^T, in two kernels instead of three
     a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
@@ -193,17 +194,21 @@ def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
     eps = 1e-5
     x = x0.clone()
     xg = torch.empty(M, H, device=DEV, dtype=torch.bfloat16)
-    ssq = torch.full((H,), float("nan"), device=DEV)
-    K.gemm_norm_prepare(a, w1, x, gain, xg, ssq)
+    ssq = torch.full(((H // 16) * K.SSQ_LD,), float("nan"), device=DEV)
+    scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV) if M > 16 else None
+    if M > 16:
+        assert K.gemm_wide_parts(M, H, Kd, K.GEMM_SCRATCH_FLOATS) >= 2
+    tiles = K.gemm_norm_prepare(a, w1, x, gain, xg, ssq, scratch)
+    assert tiles == (H // 16 if M <= 16 else H // 256)
     xw = x0.double() + a.double() @ w1.double().T
     assert (x.double() - xw).abs().max() < 1e-4 * xw.abs().max()
     assert (xg.double() - xw * gain.double()).abs().max() < 1e-2 * (xw * gain.double()).abs().max()
-    tiles = ssq.view(H // 16, 16)[:, :M].double()
-    assert (tiles.sum(0) - (xw * xw).sum(-1)).abs().max() < 1e-4 * (xw * xw).sum(-1).max()
+    sums = ssq[:tiles * K.SSQ_LD].view(tiles, K.SSQ_LD)[:, :M].double()
+    assert (sums.sum(0) - (xw * xw).sum(-1)).abs().max() < 1e-4 * (xw * xw).sum(-1).max()
     normed = xw / torch.sqrt((xw * xw).mean(-1, keepdim=True) + eps) * gain.double()
     want = normed @ w2.double().T
     o32 = torch.empty(M, N2, device=DEV)
-    K.gemm_norm_scaled(xg, ssq, eps, w2, o32)
+    K.gemm_norm_scaled(xg, ssq, tiles, eps, w2, o32, scratch=scratch)
     assert (o32.double() - want).abs().max() < 1e-2 * want.abs().max()
     # against the same product with the rows normed by the norm kernel: bf16 roundings apart
     h = torch.empty(M, H, device=DEV, dtype=torch.bfloat16)
@@ -212,18 +217,18 @@ def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
     K.gemm(h, w2, two)
     assert (o32 - two).abs().max() < 1e-2 * want.abs().max()
     o16 = torch.empty(M, N2, device=DEV, dtype=torch.bfloat16)
-    K.gemm_norm_scaled(xg, ssq, eps, w2, o16)
+    K.gemm_norm_scaled(xg, ssq, tiles, eps, w2, o16, scratch=scratch)
     assert (o16.double() - want).abs().max() < 2e-2 * want.abs().max()
     if N2 % 16 == 0:
         out = torch.empty(M, N2 // 2, device=DEV, dtype=torch.bfloat16)
-        K.gemm_norm_scaled(xg, ssq, eps, w2, out, swiglu=True)
+        K.gemm_norm_scaled(xg, ssq, tiles, eps, w2, out, swiglu=True, scratch=scratch)
         gu = want.view(M, N2 // 16, 2, 8)
         g, u = gu[:, :, 0].reshape(M, -1), gu[:, :, 1].reshape(M, -1)
         sw = g / (1 + torch.exp(-g)) * u
         assert (out.double() - sw).abs().max() < 2e-2 * sw.abs().max()
     with pytest.raises(KernelError):
-        K.gemm_norm_prepare(rnd(17, Kd, dtype=torch.bfloat16), w1, torch.zeros(17, H, device=DEV), gain,
-                            torch.empty(17, H, device=DEV, dtype=torch.bfloat16), ssq)
+        K.gemm_norm_prepare(rnd(65, Kd, dtype=torch.bfloat16), w1, torch.zeros(65, H, device=DEV), gain,
+                            torch.empty(65, H, device=DEV, dtype=torch.bfloat16), ssq, scratch)
 
 
 def test_gemm_reference_vectors():
