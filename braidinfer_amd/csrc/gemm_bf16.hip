@@ -897,15 +897,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 #pragma unroll
     for (int j = 0; j < D; ++j)
         if (j < nitems) ISSUE(j);
+    // NORM 2: row m = tid / 32, its 32 lanes take the tiles' sums in turn.  The first eight a lane are requested
+    // here and added at the first tile's end, so that their way from memory runs under the first tile.
+    float ssq_pre[8];
     if constexpr (NORM == 2) {
-        // row m = tid / 32: its 32 lanes take the tiles' sums in turn, then a butterfly; read at the first tile's end
         const int m = tid >> 5, l = tid & 31;
-        float t = 0.f;
-        if (m < M)
-            for (int c = l; c < nrm.ssq_tiles; c += 32) t += nrm.ssq[(size_t)c * SSQ_LD + m];
 #pragma unroll
-        for (int o = 16; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
-        if (l == 0) rstd[m] = m < M ? rsqrtf(t * nrm.inv_k + nrm.eps) : 0.f;
+        for (int j = 0; j < 8; ++j)
+            ssq_pre[j] = (m < M && l + 32 * j < nrm.ssq_tiles) ? nrm.ssq[(size_t)(l + 32 * j) * SSQ_LD + m] : 0.f;
     }
 
     for (int base = 0; base < nitems; base += S) {
@@ -937,6 +936,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
                     const int n0 = ((int)blockIdx.x + cp_t * (int)gridDim.x) * RT;
                     ++cp_t;
                     float* rb = red + buf * (NW * 16 * 17);
+                    if (NORM == 2 && cp_t == 1) {
+                        const int m = tid >> 5, l = tid & 31;
+                        float t = 0.f;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) t += ssq_pre[j];
+                        if (m < M)
+                            for (int c = l + 256; c < nrm.ssq_tiles; c += 32) t += nrm.ssq[(size_t)c * SSQ_LD + m];
+#pragma unroll
+                        for (int o = 16; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+                        if (l == 0) rstd[m] = m < M ? rsqrtf(t * nrm.inv_k + nrm.eps) : 0.f;
+                    }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) rb[(wave * 16 + 4 * g + r) * 17 + r16] = acc[r] + acc1[r];
                     acc = {0.f, 0.f, 0.f, 0.f};
