@@ -765,22 +765,52 @@ __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
     }
 }
 
-// grid = (nq, sequences), block = 64: add the splits in split order
-__global__ __launch_bounds__(64) void attn_decode_combine_kernel(const float* __restrict__ part_o,
-                                                                 const float* __restrict__ part_ml,
-                                                                 bf16* __restrict__ out, int nq, int hd, int nsplit) {
-    const int head = blockIdx.x, b = blockIdx.y;
+// grid = (nq, sequences), block = 256: the splits of one head are added by four waves, wave w taking
+// the splits s = w, w + 4, ... in that order and the four sums being added in wave order, so the
+// result depends on nsplit only.  The weights 2^(m_s - M) are computed once into LDS.
+#define COMBINE_MAX_SPLIT 1024
+__global__ __launch_bounds__(256) void attn_decode_combine_kernel(const float* __restrict__ part_o,
+                                                                  const float* __restrict__ part_ml,
+                                                                  bf16* __restrict__ out, int nq, int hd, int nsplit) {
+    __shared__ float wgt[COMBINE_MAX_SPLIT];
+    __shared__ float red[4];
+    __shared__ float psum[4][64];
+    const int head = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t base = ((size_t)b * nq + head) * nsplit;
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
-    float L = 0.f;
-    if (M > -INFINITY)
-        for (int s = 0; s < nsplit; ++s) L += part_ml[(base + s) * 2 + 1] * fast_exp2(part_ml[(base + s) * 2] - M);
-    for (int d = threadIdx.x; d < hd; d += 64) {
+    float m = -INFINITY;
+    for (int s = tid; s < nsplit; s += 256) m = fmaxf(m, part_ml[(base + s) * 2]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float l = 0.f;
+    for (int s = tid; s < nsplit; s += 256) {
+        const float w = M > -INFINITY ? fast_exp2(part_ml[(base + s) * 2] - M) : 0.f;
+        wgt[s] = w;
+        l += part_ml[(base + s) * 2 + 1] * w;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    if (lane == 0) red[wave] = l;
+    __syncthreads();
+    const float L = ((red[0] + red[1]) + red[2]) + red[3];
+    for (int d0 = 0; d0 < hd; d0 += 64) {
+        const int d = d0 + lane;
         float O = 0.f;
-        if (M > -INFINITY)
-            for (int s = 0; s < nsplit; ++s) O += part_o[(base + s) * hd + d] * fast_exp2(part_ml[(base + s) * 2] - M);
-        out[((size_t)b * nq + head) * hd + d] = (bf16)(L > 0.f ? O / L : 0.f);
+        if (d < hd) {
+            const float* po = part_o + base * hd + d;
+#pragma unroll 4
+            for (int s = wave; s < nsplit; s += 4) O += po[(size_t)s * hd] * wgt[s];
+        }
+        psum[wave][lane] = O;
+        __syncthreads();
+        if (wave == 0 && d < hd) {
+            const float sum = ((psum[0][lane] + psum[1][lane]) + psum[2][lane]) + psum[3][lane];
+            out[((size_t)b * nq + head) * hd + d] = (bf16)(L > 0.f ? sum / L : 0.f);
+        }
+        __syncthreads();
     }
 }
 
@@ -896,7 +926,7 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
 #undef BR_DECODE_LDS
         int rc2 = br_check_launch();
         if (rc2 != BR_OK || nsplit == 1) return rc2;
-        attn_decode_combine_kernel<<<dim3(nq, B), 64, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
+        attn_decode_combine_kernel<<<dim3(nq, B), 256, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
         return br_check_launch();
     }
     const size_t lds = (size_t)4 * (16 * hd + 32) * sizeof(float);
@@ -927,6 +957,6 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
 #undef BR_DECODE
     int rc = br_check_launch();
     if (rc != BR_OK || nsplit == 1) return rc;
-    attn_decode_combine_kernel<<<dim3(nq, B), 64, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
+    attn_decode_combine_kernel<<<dim3(nq, B), 256, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
     return br_check_launch();
 }
