@@ -264,16 +264,33 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
 // barrier makes every wave's part of the stage visible (and says that the stage about to
 // be overwritten has been read by all).  The kernel issues no other vector memory
 // operation inside the loop, so the count is exact.
+// Weight layouts (`wl`).  0: N rows of K.  1: blocks of 16 rows x 128 k, 4 KB contiguous each, ordered
+// [row block][k block], rows padded to a multiple of 16 (K in steps of 128): a 16-row strip is one
+// contiguous run along k.  A streaming product then reads 4 KB pieces, in order, instead of 256 bytes
+// from every row, which the memory serves faster (bare loads of a 64-row tile by every workgroup: 5.4 to
+// 5.9 against 4.1 to 4.6 TB/s; in the products: wide matrices at 17 to 128 rows gain 10 to 15 %, up to
+// 16 rows 0 to 5 %, the rest nothing).  Blocks of 64 rows were tried: slower up to 16 rows.
+#define WL_ROWS 0
+#define WL_BLOCKED 1
+#ifndef WL_BLOCK_ROWS
+#define WL_BLOCK_ROWS 16
+#endif
+#define WL_BLOCK_ELEMS (WL_BLOCK_ROWS * 128)
+__device__ __forceinline__ size_t w_row_base(int n, int K, int wl) {
+    return wl ? (size_t)(n / WL_BLOCK_ROWS) * (size_t)(K >> 7) * WL_BLOCK_ELEMS + (size_t)((n % WL_BLOCK_ROWS) << 7)
+              : (size_t)n * K;
+}
 #define DMA_BK 64
 #define DMA_ISSUE(ST, kt)                                                                                      \
     do {                                                                                                       \
         _Pragma("unroll") for (int q = 0; q < INSTR; ++q) {                                                    \
             const unsigned lds_ = __builtin_amdgcn_readfirstlane(                                              \
                 (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)(ST)) + dst[q]);          \
-            const bf16* gp_ = src[q] + (size_t)(kt) * DMA_BK;                                                  \
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q]) \
                          : "m0");                                                                              \
+            src[q] += (knext & 1) ? hop[q] : DMA_BK;       /* k-tiles are issued in order, (kt) is the next */ \
         }                                                                                                      \
+        ++knext;                                                                                               \
     } while (0)
 #define DMA_COMPUTE(ST)                                                                                        \
     do {                                                                                                       \
@@ -303,7 +320,7 @@ static int launch_tile(const bf16* A, const bf16* W, void* C, int M, int N, int 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int S, int MODE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ W, void* __restrict__ C_, int M, int N, int K, size_t lda,
-    size_t ldc, int tiles_m, int tiles_n, int kt_per_part, size_t part_stride) {
+    size_t ldc, int tiles_m, int tiles_n, int kt_per_part, size_t part_stride, int wl) {
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int STAGE_BYTES = (BM + BN) * DMA_BK * 2;
@@ -343,6 +360,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
     // wave-load q of this wave covers rows (q NW + wave) 8 .. + 8 of the stacked tile [A rows | W rows]
     const bf16* src[INSTR];
     int dst[INSTR];
+    int hop[INSTR];                                      // elements from an odd k-tile to the next (even) one
+    const int kt0 = (int)blockIdx.y * kt_per_part;       // the run's first k-tile
+    int knext = kt0;                                     // the k-tile that src[] points at
 #pragma unroll
     for (int q = 0; q < INSTR; ++q) {
         const int R = (q * NW + wave) * 8 + (lane >> 3);
@@ -350,16 +370,19 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
         if (R < BM) {
             int r = m0 + R;
             if (r > M - 1) r = M - 1;
-            src[q] = A + (size_t)r * lda + c * 8;
+            src[q] = A + (size_t)r * lda + c * 8 + (size_t)kt0 * DMA_BK;
+            hop[q] = DMA_BK;
         } else {
             int r = n0 + R - BM;
             if (r > N - 1) r = N - 1;
-            src[q] = W + (size_t)r * K + c * 8;
+            src[q] = W + w_row_base(r, K, wl) + c * 8 +
+                     (wl ? (size_t)(kt0 >> 1) * WL_BLOCK_ELEMS + (kt0 & 1) * DMA_BK : (size_t)kt0 * DMA_BK);
+            hop[q] = wl ? WL_BLOCK_ELEMS - DMA_BK : DMA_BK;
         }
-        src[q] += (size_t)blockIdx.y * kt_per_part * DMA_BK;
+        hop[q] = __builtin_amdgcn_readfirstlane(hop[q]);             // the same for the 8 rows of a wave-load
         dst[q] = (q * NW + wave) * 1024;
     }
-    int nk = K / DMA_BK - (int)blockIdx.y * kt_per_part;
+    int nk = K / DMA_BK - kt0;
     if (nk > kt_per_part) nk = kt_per_part;
     if (S == 2) {
         DMA_ISSUE(st0, 0);
@@ -413,7 +436,7 @@ static int launch_split_sum(const float* scratch, int parts, void* C, int M, int
 // run order and applies the epilogue (for products with too few tiles to fill the chip).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int S>
 static int launch_tile_dma(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
-                           int mode, hipStream_t s, int parts = 1, float* scratch = nullptr) {
+                           int mode, hipStream_t s, int parts = 1, float* scratch = nullptr, int wl = 0) {
     const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     const long long total = (long long)tm * tn;
     if (total > 0x7fffffffLL) return BR_BAD_ARG;
@@ -424,19 +447,19 @@ static int launch_tile_dma(const bf16* A, const bf16* W, void* C, int M, int N, 
         parts = (nk + kpp - 1) / kpp;                                 // no empty run
         dim3 grid((unsigned)total, (unsigned)parts);
         gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<grid, NT, 0, s>>>(
-            A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp, (size_t)M * N);
+            A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp, (size_t)M * N, wl);
         int rc = br_check_launch();
         if (rc != BR_OK) return rc;
         return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
     }
     if (mode == OUT_BF16)
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_BF16><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_BF16><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else if (mode == OUT_F32)
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else if (mode == OUT_F32_ACC)
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32_ACC><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_F32_ACC><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else
-        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_SWIGLU><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0);
+        gemm_tile_dma_kernel<BM, BN, WAVES_M, WAVES_N, S, OUT_SWIGLU><<<(unsigned)total, NT, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     return br_check_launch();
 }
 
@@ -837,7 +860,7 @@ struct StreamNorm {
 template <int RT, int XR, int KC, int S, int NW, int MODE, int NORM>
 __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                               void* __restrict__ C, int M, int N, int K, size_t lda,
-                                                              size_t ldc, int ntiles, StreamNorm nrm) {
+                                                              size_t ldc, int ntiles, StreamNorm nrm, int wl) {
     static_assert(NORM == 0 || (NORM == 1 && MODE == OUT_F32_ACC) || (NORM == 2 && MODE != OUT_F32_ACC), "norm forms");
     constexpr int STEPS = KC / 32;
     constexpr int ROWB = KC * 2;
@@ -860,11 +883,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 
     const int nch = K / KC;
     const int ncw = (nch - wave + NW - 1) / NW;
+    // Where in k this workgroup starts: workgroups that walk their rows in step ask the same few memory
+    // channels at the same time; a start of its own for each spreads them (measured: 4 to 9 % on the
+    // products of 4,096 to 6,144 weight rows).  The order of a column's sum depends on the column only.
+    const int rot = (int)(((unsigned)blockIdx.x * 2654435761u) >> 8) % nch;
     const int my_tiles = (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
     const int nitems = my_tiles * ncw;
 
     // DMA lane mapping
     const int drow = lane / CPL, dcol = lane % CPL;
+    const int wstep = wl ? WL_BLOCK_ELEMS : KC;        // elements from a chunk of a weight row to the next
     f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 
     int is_t = 0, is_c = 0;      // issue cursor: local tile index, local chunk index
@@ -873,7 +901,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 
 #define ISSUE(J)                                                                                         \
     do {                                                                                                 \
-        const int chunk_ = wave + is_c * NW;                                                             \
+        int chunk_ = wave + is_c * NW + rot;                                                             \
+        if (chunk_ >= nch) chunk_ -= nch;                                                                \
         const int n0_ = ((int)blockIdx.x + is_t * (int)gridDim.x) * RT;                                  \
         _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                            \
             const int row_ = q_ * RPI + drow;                                                            \
@@ -881,7 +910,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
             if (q_ < WDMA) {                                                                             \
                 int nrow_ = n0_ + row_;                                                                  \
                 if (nrow_ > N - 1) nrow_ = N - 1;                                                        \
-                gp_ = W + (size_t)nrow_ * K + (size_t)chunk_ * KC + ((dcol ^ (row_ & 7)) * 8);           \
+                gp_ = W + w_row_base(nrow_, K, wl) + (size_t)chunk_ * wstep + ((dcol ^ (row_ & 7)) * 8);  \
             } else {                                                                                     \
                 int m_ = row_ - RT;                                                                      \
                 if (m_ > M - 1) m_ = M - 1;                                                              \
@@ -1016,8 +1045,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
 #define STREAM_NW 8
 template <int XR, int NORM>
 static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
-                         int mode, hipStream_t s, StreamNorm nrm = StreamNorm{}) {
+                         int mode, hipStream_t s, StreamNorm nrm = StreamNorm{}, int wl = 0) {
     constexpr int RT = 16, KC = STREAM_KC, S = 2, NW = STREAM_NW;
+    static_assert(KC == 128, "the blocked weight layout has 128 k a block");
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
     const int ntiles = (N + RT - 1) / RT;
@@ -1033,7 +1063,7 @@ static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, in
                 return BR_LAUNCH_FAILED;                                                                        \
             set = true;                                                                                         \
         }                                                                                                       \
-        kern<<<grid, NW * 64, lds, s>>>(A, W, C, M, N, K, lda, ldc, ntiles, nrm);                               \
+        kern<<<grid, NW * 64, lds, s>>>(A, W, C, M, N, K, lda, ldc, ntiles, nrm, wl);                           \
     } while (0)
     if constexpr (NORM == 1) {
         BR_STREAM(OUT_F32_ACC);
@@ -1050,82 +1080,103 @@ static int launch_stream(const bf16* A, const bf16* W, void* C, int M, int N, in
 
 // ------------------------------------------------------------- gemm_stream_wide ------
 // 16 < M <= 64, K in steps of 128: the same streaming by workgroups that stay, with the
-// activations shared.  A unit of work is a tile of 64 weight rows over one run of k-chunks
-// (the whole K, or one of `parts` runs when the tiles alone would be too few for the chip);
-// unit u of workgroup b is b + u * grid.  A stage of the workgroup's LDS ring holds one
-// 128-wide chunk of the tile (64 rows) and of the activations (16 MB rows), brought by all
-// 8 waves with direct global-to-LDS loads, two chunks ahead; one barrier per chunk.  Wave w
-// multiplies weight rows 16 (w % 4) .. + 16 with k-steps 2 (w / 4), 2 (w / 4) + 1 of the
-// chunk; the two k-halves are added in LDS at the unit's end.  With `parts` > 1 the unit's
-// float sums go to a matrix of its run (`part_stride` elements apart) for
-// gemm_split_sum_kernel; else the epilogue is applied here.
-#define WIDE_S 3
-// SCALE: the activations are the bf16(h * g) rows that the product before left for an RMS norm
+// activations shared.  A unit of work is a tile of 16 HB weight rows (64 to 128) over one run of
+// k-chunks (the whole K, or one of `parts` runs); height and runs are chosen so that the units
+// fill the compute units in whole rounds (wide_shape below: 28,672 rows are 256 tiles of 112).
+// Unit u of workgroup b is b + u * grid.  A stage of the workgroup's 3-stage LDS ring holds one
+// 128-wide chunk of the tile and of the activations (16 MB rows), brought by all 8 waves with
+// direct global-to-LDS loads, two chunks ahead; one barrier per chunk.  Wave w multiplies the
+// weight rows 16 (w % 4) .. + 16 (and 64 + 16 (w % 4) .. + 16 where the tile has them) with
+// k-steps 2 (w / 4), 2 (w / 4) + 1 of the chunk; the two k-halves are added in LDS at the
+// unit's end (half 0 + half 1), in the stage that was multiplied last.  With `parts` > 1 the
+// unit's float sums go to a matrix of its run (`part_stride` elements apart) for
+// gemm_split_sum_kernel; else the epilogue (`mode`) is applied here.  The epilogue's form is
+// chosen at run time: it runs once per unit, the chunk loop is the same for all.
+// scale: the activations are the bf16(h * g) rows that the product before left for an RMS norm
 // (see gemm_stream's NORM forms); the sums are multiplied by 1 / rms of their row, run by run.
-template <int MB, int MODE, bool PARTIAL, bool SCALE>
+#define WIDE_S 3
+template <int MB, int HB>
 __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                                void* __restrict__ C, int M, int N, int K, size_t lda,
-                                                               size_t ldc, int ntiles, int parts, int cpp,
-                                                               size_t part_stride, StreamNorm nrm) {
-    constexpr int S = WIDE_S, D = S - 1, NW = 8;
-    constexpr int ROWS = 64 + 16 * MB;               // stacked rows of a stage: weights, then activations
+                                                               size_t ldc, int mode, int partial, int scale,
+                                                               int ntiles, int parts, int cpp, size_t part_stride,
+                                                               StreamNorm nrm, int wl) {
+    constexpr int S = WIDE_S, D = S - 1, NW = 8, H = 16 * HB;
+    constexpr int ROWS = H + 16 * MB;                // stacked rows of a stage: weights, then activations
     constexpr int STAGE = ROWS * 256;
-    constexpr int NDMA = STAGE / 1024 / NW;          // wave-loads per wave and chunk
+    constexpr int NLD = ROWS / 4;                    // wave-loads of a chunk: 4 rows of 256 bytes each
+    constexpr int NDMA = (NLD + NW - 1) / NW;        // of each wave; surplus ones repeat the chunk's last load
     constexpr int RLD = 16 * MB + 1;
-    static_assert(STAGE % (1024 * NW) == 0 && (D - 1) * NDMA <= 63, "stage");
+    constexpr bool TWO = HB > 4;
+    static_assert(HB >= 4 && HB <= 8 && (D - 1) * NDMA <= 63 && H * RLD * 4 <= STAGE, "stage");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    float* red = (float*)(smem + S * STAGE);         // [NW][16][RLD]
-    float* rstd = red + NW * 16 * RLD;               // SCALE: [64]
+    float* rstd = (float*)(smem + S * STAGE);        // scale: [64]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
     const int rb = wave & 3, khalf = wave >> 2;
+    const bool has1 = TWO && rb + 4 < HB;
     const unsigned ring_lds = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)smem);
     const int nch = K / 128;
     const int nunits = ntiles * parts;
     const int my_units = (nunits - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
 
-    f32x4 acc[MB];
+    f32x4 acc[TWO ? 2 : 1][MB];
 #pragma unroll
-    for (int j = 0; j < MB; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < (TWO ? 2 : 1); ++t)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // cursors over this workgroup's chunks in order: (unit, chunk of its run)
-    int is_u = 0, is_c = 0, cp_u = 0, cp_c = 0;
+    // Cursors over this workgroup's chunks in order.  What depends on the unit only (its tile, its run
+    // of chunks, each lane's addresses) is worked out once per unit, so that a chunk costs each wave its
+    // loads, an address step and a count.
+    int is_u = 0, is_left = 0, cp_u = 0, cp_left = 0;       // units begun, chunks of the current one to go
     int issued = 0, done = 0;
-#define WIDE_RUN(U, C0, C1)                                                  \
-    const int part_##U = ((int)blockIdx.x + (U) * (int)gridDim.x) % parts;    \
-    const int C0 = part_##U * cpp;                                           \
-    const int C1 = C0 + cpp < nch ? C0 + cpp : nch;
-#define WIDE_ISSUE()                                                                                          \
+    unsigned is_off = 0, cp_off = 0;                        // the ring's stage to fill, to multiply (bytes)
+    const bf16* src[NDMA];                                  // this lane's 16 bytes of each of its loads
+    const int wstep = wl ? WL_BLOCK_ELEMS : 128;                      // elements from a chunk of a weight row to the next
+#define WIDE_RUN_LENGTH(U, LEN)                                                                               \
+    do {                                                                                                      \
+        const int c0_ = (((int)blockIdx.x + (U) * (int)gridDim.x) % parts) * cpp;                             \
+        LEN = (c0_ + cpp < nch ? c0_ + cpp : nch) - c0_;                                                      \
+    } while (0)
+#define WIDE_LOAD_INDEX(Q) ((wave * NDMA + (Q)) < NLD - 1 ? (wave * NDMA + (Q)) : NLD - 1)
+#define WIDE_SETUP()                                                                                          \
     do {                                                                                                      \
         const int unit_ = (int)blockIdx.x + is_u * (int)gridDim.x;                                            \
         const int tile_ = unit_ / parts, c0_ = (unit_ % parts) * cpp;                                         \
-        const int c1_ = c0_ + cpp < nch ? c0_ + cpp : nch;                                                    \
-        const int chunk_ = c0_ + is_c;                                                                        \
+        is_left = (c0_ + cpp < nch ? c0_ + cpp : nch) - c0_;                                                  \
         _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                 \
-            const int in_ = wave * NDMA + q_;                                                                 \
-            const int row_ = in_ * 4 + (lane >> 4);                                                           \
+            const int row_ = WIDE_LOAD_INDEX(q_) * 4 + (lane >> 4);                                           \
             const bf16* gp_;                                                                                  \
-            if (row_ < 64) {                                                                                  \
-                int n_ = tile_ * 64 + row_;                                                                   \
+            if (row_ < H) {                                                                                   \
+                int n_ = tile_ * H + row_;                                                                    \
                 if (n_ > N - 1) n_ = N - 1;                                                                   \
-                gp_ = W + (size_t)n_ * K;                                                                     \
+                gp_ = W + w_row_base(n_, K, wl) + (size_t)c0_ * wstep;                                        \
             } else {                                                                                          \
-                int m_ = row_ - 64;                                                                           \
+                int m_ = row_ - H;                                                                            \
                 if (m_ > M - 1) m_ = M - 1;                                                                   \
-                gp_ = A + (size_t)m_ * lda;                                                                   \
+                gp_ = A + (size_t)m_ * lda + (size_t)c0_ * 128;                                               \
             }                                                                                                 \
-            gp_ += (size_t)chunk_ * 128 + (((lane & 15) ^ (row_ & 7)) * 8);                                   \
-            const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + (issued % S) * STAGE + in_ * 1024); \
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
+            src[q_] = gp_ + (((lane & 15) ^ (row_ & 7)) * 8);                                                 \
+        }                                                                                                     \
+    } while (0)
+#define WIDE_ISSUE()                                                                                          \
+    do {                                                                                                      \
+        _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                 \
+            const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + is_off + WIDE_LOAD_INDEX(q_) * 1024); \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q_]) : "m0"); \
+            src[q_] += WIDE_LOAD_INDEX(q_) * 4 < H ? wstep : 128;                                             \
         }                                                                                                     \
         ++issued;                                                                                             \
-        if (c0_ + ++is_c == c1_) { is_c = 0; ++is_u; }                                                        \
+        is_off = is_off + STAGE == S * STAGE ? 0 : is_off + STAGE;                                            \
+        if (--is_left == 0 && ++is_u < my_units) WIDE_SETUP();                                                \
     } while (0)
 
+    if (my_units > 0) WIDE_SETUP();
     for (int j = 0; j < D; ++j)
         if (is_u < my_units) WIDE_ISSUE();
-    if constexpr (SCALE) {
+    if (scale) {
         // row m = tid / 8: its 8 lanes take the tiles' sums in turn, then a butterfly; read at the first unit's end
         const int m = tid >> 3, l = tid & 7;
         float t = 0.f;
@@ -1135,6 +1186,7 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
         for (int o = 4; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
         if (l == 0) rstd[m] = m < M ? rsqrtf(t * nrm.inv_k + nrm.eps) : 0.f;
     }
+    if (my_units > 0) WIDE_RUN_LENGTH(0, cp_left);
     while (cp_u < my_units) {
         // the chunk to multiply has landed when at most the loads of the chunks issued after it are in flight
         if (issued - done - 1 >= 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
@@ -1142,113 +1194,164 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
         __builtin_amdgcn_s_barrier();            // every wave's part of it is there; the chunk before is done with
         asm volatile("" ::: "memory");
         if (is_u < my_units) WIDE_ISSUE();
-        const unsigned char* st = smem + (done % S) * STAGE;
+        unsigned char* st = smem + cp_off;
+        cp_off = cp_off + STAGE == S * STAGE ? 0 : cp_off + STAGE;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int col = 4 * (2 * khalf + ks) + g;
             const int wr = 16 * rb + r16;
-            const bf16x8 wf = *(const bf16x8*)(st + wr * 256 + ((col ^ (wr & 7)) * 16));
+            const bf16x8 wf0 = *(const bf16x8*)(st + wr * 256 + ((col ^ (wr & 7)) * 16));
+            bf16x8 wf1 = wf0;
+            if (TWO && has1) wf1 = *(const bf16x8*)(st + (64 + wr) * 256 + ((col ^ (wr & 7)) * 16));
 #pragma unroll
             for (int j = 0; j < MB; ++j) {
-                const int xr = 64 + 16 * j + r16;
+                const int xr = H + 16 * j + r16;
                 const bf16x8 xv = *(const bf16x8*)(st + xr * 256 + ((col ^ (xr & 7)) * 16));
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xv, acc[j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, xv, acc[0][j], 0, 0, 0);
+                if (TWO && has1) acc[TWO ? 1 : 0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, xv, acc[TWO ? 1 : 0][j], 0, 0, 0);
             }
         }
         ++done;
+        if (--cp_left > 0) continue;
+        // The unit's end: acc[t][j][r] is weight row 64 t + 16 rb + 4 g + r of the tile, batch row 16 j + r16.
+        // The sums meet in the stage that was multiplied last: the next loads into it are issued after
+        // the next chunk's barrier, which a wave reaches after its part of the epilogue.
         const int unit = (int)blockIdx.x + cp_u * (int)gridDim.x;
-        const int part = unit % parts, c0 = part * cpp;
-        const int c1 = c0 + cpp < nch ? c0 + cpp : nch;
-        if (c0 + ++cp_c < c1) continue;
-        // the unit's end: acc[j][r] is weight row 16 rb + 4 g + r of the tile, batch row 16 j + r16
-        cp_c = 0;
-        ++cp_u;
-        const int n0 = (unit / parts) * 64;
+        const int part = unit % parts;
+        const int n0 = (unit / parts) * H;
+        if (++cp_u < my_units) WIDE_RUN_LENGTH(cp_u, cp_left);
+        float* red = (float*)st;                 // [H][RLD]
+        __builtin_amdgcn_s_barrier();            // every wave has read its operands of the stage
+        asm volatile("" ::: "memory");
+        if (khalf == 1) {
 #pragma unroll
-        for (int j = 0; j < MB; ++j) {
+            for (int t = 0; t < (TWO ? 2 : 1); ++t)
+                if (t == 0 || has1)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) red[(wave * 16 + 4 * g + r) * RLD + 16 * j + r16] = acc[j][r];
-            acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    for (int j = 0; j < MB; ++j)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) red[(64 * t + 16 * rb + 4 * g + r) * RLD + 16 * j + r16] = acc[t][j][r];
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();            // the next write to `red` comes after the next chunk's barrier
+        __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (MODE == OUT_SWIGLU && !PARTIAL) {
+        if (khalf == 0) {
+#pragma unroll
+            for (int t = 0; t < (TWO ? 2 : 1); ++t)
+                if (t == 0 || has1)
+#pragma unroll
+                    for (int j = 0; j < MB; ++j)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            float* p = red + (64 * t + 16 * rb + 4 * g + r) * RLD + 16 * j + r16;
+                            *p = acc[t][j][r] + *p;
+                        }
+        }
+#pragma unroll
+        for (int t = 0; t < (TWO ? 2 : 1); ++t)
+#pragma unroll
+            for (int j = 0; j < MB; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (mode == OUT_SWIGLU && !partial) {
             // blocks of 16 tile rows: 8 gates, then the 8 up values of the same outputs
-            for (int e = tid; e < 32 * 16 * MB; e += 512) {
-                const int m = e >> 5, jl = e & 31;
+            for (int e = tid; e < (H / 2) * 16 * MB; e += 512) {
+                const int m = e / (H / 2), jl = e % (H / 2);
                 const int gr = (jl >> 3) * 16 + (jl & 7);
                 if (m < M && n0 + gr + 8 < N) {
-                    float gv = red[gr * RLD + m] + red[(64 + gr) * RLD + m];
-                    float uv = red[(gr + 8) * RLD + m] + red[(64 + gr + 8) * RLD + m];
-                    if (SCALE) { gv *= rstd[m]; uv *= rstd[m]; }
+                    float gv = red[gr * RLD + m];
+                    float uv = red[(gr + 8) * RLD + m];
+                    if (scale) { gv *= rstd[m]; uv *= rstd[m]; }
                     ((bf16*)C)[(size_t)m * ldc + n0 / 2 + jl] = (bf16)silu_mul(gv, uv);
                 }
             }
         } else {
-            for (int e = tid; e < 64 * 16 * MB; e += 512) {
-                const int m = e >> 6, nl = e & 63, n = n0 + nl;
+            for (int e = tid; e < H * 16 * MB; e += 512) {
+                const int m = e / H, nl = e % H, n = n0 + nl;
                 if (m < M && n < N) {
-                    float v = red[nl * RLD + m] + red[(64 + nl) * RLD + m];      // k-half 0, then 1
-                    if (SCALE) v *= rstd[m];
-                    if (PARTIAL) ((float*)C)[part * part_stride + (size_t)m * N + n] = v;
-                    else {
-                        const size_t idx = (size_t)m * ldc + n;
-                        if (MODE == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
-                        else if (MODE == OUT_F32) ((float*)C)[idx] = v;
-                        else unsafeAtomicAdd((float*)C + idx, v);     // one add per element, no read to wait for
-                    }
+                    float v = red[nl * RLD + m];
+                    if (scale) v *= rstd[m];
+                    const size_t idx = (size_t)m * ldc + n;
+                    if (partial) ((float*)C)[part * part_stride + (size_t)m * N + n] = v;
+                    else if (mode == OUT_BF16) ((bf16*)C)[idx] = (bf16)v;
+                    else if (mode == OUT_F32) ((float*)C)[idx] = v;
+                    else unsafeAtomicAdd((float*)C + idx, v);         // one add per element, no read to wait for
                 }
             }
         }
     }
 #undef WIDE_ISSUE
-#undef WIDE_RUN
+#undef WIDE_SETUP
+#undef WIDE_LOAD_INDEX
+#undef WIDE_RUN_LENGTH
 }
 
-// Into how many runs of k-chunks the units of gemm_stream_wide are cut: the least time by a
-// simple count (rounds of units over the compute units, times the run's length, plus the
-// traffic of the partial sums), among 1, 2, 4 and 8 runs of at least 2 chunks.
-static int wide_parts(int M, int N, int K, int mode, int cus, size_t scratch_bytes) {
-    const int tiles = (N + 63) / 64, nch = K / 128;
-    int best = 1;
+// The shape of gemm_stream_wide's units: tile height (64 to 128 rows in steps of 16) and runs
+// along k (1 to 8), the least time by a simple count: rounds of units over the compute
+// units, times the run's chunks, times what a chunk costs (its weight rows and a constant for
+// the activations, which come from the L2, and the barrier), plus the traffic of the partial
+// sums.  Ties go to fewer runs, then to lower tiles.
+static void wide_shape(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* hb_out, int* parts_out) {
+    const int nch = K / 128;
     double best_cost = 1e30;
-    for (int parts = 1; parts <= 8; parts *= 2) {
-        if (parts > 1 && (mode == OUT_SWIGLU || parts * 2 > nch ||
-                          (size_t)parts * M * N * sizeof(float) > scratch_bytes))
+    *hb_out = 4;
+    *parts_out = 1;
+    for (int parts = 1; parts <= 8; ++parts) {
+        if (parts > 1 && (mode == OUT_SWIGLU || parts * 2 > nch || (size_t)parts * M * N * sizeof(float) > scratch_bytes))
             break;
         const int cpp = (nch + parts - 1) / parts;
-        const long long rounds = ((long long)tiles * parts + cus - 1) / cus;
-        double cost = (double)rounds * cpp;
-        if (parts > 1) cost *= 1.0 + 4.0 * parts * M / K;
-        if (cost < best_cost - 1e-9) { best_cost = cost; best = parts; }
+        if ((nch + cpp - 1) / cpp != parts) continue;                // it would leave a run empty
+        for (int hb = 4; hb <= 8; ++hb) {
+            const int h = 16 * hb;
+            const long long tiles = (N + h - 1) / h;
+            const long long rounds = (tiles * parts + cus - 1) / cus;
+            double cost = (double)rounds * cpp * (h + 16.0);
+            if (parts > 1) cost *= 1.0 + 4.0 * parts * M / K;
+            if (cost < best_cost * (1.0 - 1e-9)) { best_cost = cost; *hb_out = hb; *parts_out = parts; }
+        }
     }
-    return best;
 }
 
 // norm: 0 none; 1 the product is added into the residual rows C and prepares the next RMS norm
 // (needs a split product: the sum kernel does it; refused otherwise); 2 the activations were so
-// prepared and the sums are scaled (modes 0, 1, 3).
+// prepared and the sums are scaled (modes 0, 1, 3).  force_hb, force_parts: a tile height (in
+// blocks of 16 rows) and a number of runs other than wide_shape's (tests and measurements).
 template <int MB>
 static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                               int mode, float* scratch, size_t scratch_bytes, hipStream_t s, int norm = 0,
-                              StreamNorm nrm = StreamNorm{}) {
+                              StreamNorm nrm = StreamNorm{}, int force_hb = 0, int force_parts = 0, int wl = 0) {
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
-    const int ntiles = (N + 63) / 64, nch = K / 128;
-    int parts = scratch ? wide_parts(M, N, K, mode, cus, scratch_bytes) : 1;
+    const int nch = K / 128;
+    int hb, parts;
+    wide_shape(M, N, K, mode, cus, scratch ? scratch_bytes : 0, &hb, &parts);
+    if (force_hb) {
+        if (force_hb < 4 || force_hb > 8) return BR_BAD_ARG;
+        hb = force_hb;
+    }
+    if (force_parts) {
+        const int cpp_ = (nch + force_parts - 1) / force_parts;
+        if (force_parts > 1 && (!scratch || mode == OUT_SWIGLU || force_parts > 8 || force_parts * 2 > nch ||
+                                (nch + cpp_ - 1) / cpp_ != force_parts ||
+                                (size_t)force_parts * M * N * sizeof(float) > scratch_bytes))
+            return BR_BAD_ARG;
+        parts = force_parts;
+    }
     if (norm == 1 && (parts < 2 || N % 256 || mode != OUT_F32_ACC)) return BR_BAD_ARG;
     if (norm == 2 && mode == OUT_F32_ACC) return BR_BAD_ARG;
     const int cpp = (nch + parts - 1) / parts;
-    parts = (nch + cpp - 1) / cpp;                                   // no empty run
+    const int h = 16 * hb, ntiles = (N + h - 1) / h;
     const long long nunits = (long long)ntiles * parts;
     const int grid = nunits < cus ? (int)nunits : cus;
-    constexpr size_t lds = (size_t)WIDE_S * (64 + 16 * MB) * 256 + 8 * 16 * (16 * MB + 1) * 4 + 64 * 4;
     const size_t stride = (size_t)M * N;
-#define BR_WIDE(MODE_, PARTIAL_, OUT_) do { if (norm == 2) BR_WIDE2(MODE_, PARTIAL_, true, OUT_); else BR_WIDE2(MODE_, PARTIAL_, false, OUT_); } while (0)
-#define BR_WIDE2(MODE_, PARTIAL_, SCALE_, OUT_)                                                                 \
+    const int partial = parts > 1;
+    void* out = partial ? (void*)scratch : C;
+#define BR_WIDE(HB_)                                                                                            \
     do {                                                                                                        \
-        auto kern = gemm_stream_wide_kernel<MB, MODE_, PARTIAL_, SCALE_>;                                       \
+        auto kern = gemm_stream_wide_kernel<MB, HB_>;                                                           \
+        constexpr size_t lds = (size_t)WIDE_S * (16 * HB_ + 16 * MB) * 256 + 64 * 4;                            \
+        static_assert(lds <= 160 * 1024, "LDS of a compute unit");                                              \
         static bool set = false;                                                                                \
         if (!set) {                                                                                             \
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != \
@@ -1256,41 +1359,44 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
                 return BR_LAUNCH_FAILED;                                                                        \
             set = true;                                                                                         \
         }                                                                                                       \
-        kern<<<grid, 512, lds, s>>>(A, W, OUT_, M, N, K, lda, ldc, ntiles, parts, cpp, stride, nrm);            \
+        kern<<<grid, 512, lds, s>>>(A, W, out, M, N, K, lda, ldc, mode, partial, norm == 2, ntiles, parts, cpp, \
+                                    stride, nrm, wl);                                                           \
     } while (0)
-    if (parts > 1) {
-        BR_WIDE(OUT_F32, true, (void*)scratch);
-        int rc = br_check_launch();
-        if (rc != BR_OK) return rc;
-        if (norm == 1) {
-            gemm_split_sum_prep_kernel<<<(unsigned)(stride / 256), 256, 0, s>>>(scratch, parts, stride, (float*)C, N, ldc,
-                                                                                nrm.gain, nrm.xg, nrm.ldx, nrm.ssq);
-            return br_check_launch();
-        }
-        return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
+    switch (hb) {
+        case 4: BR_WIDE(4); break;
+        case 5: BR_WIDE(5); break;
+        case 6: BR_WIDE(6); break;
+        case 7: BR_WIDE(7); break;
+        default: BR_WIDE(8); break;
     }
-    if (mode == OUT_BF16) BR_WIDE(OUT_BF16, false, C);
-    else if (mode == OUT_F32) BR_WIDE(OUT_F32, false, C);
-    else if (mode == OUT_F32_ACC) BR_WIDE(OUT_F32_ACC, false, C);
-    else BR_WIDE(OUT_SWIGLU, false, C);
 #undef BR_WIDE
-#undef BR_WIDE2
-    return br_check_launch();
+    int rc = br_check_launch();
+    if (rc != BR_OK || !partial) return rc;
+    if (norm == 1) {
+        gemm_split_sum_prep_kernel<<<(unsigned)(stride / 256), 256, 0, s>>>(scratch, parts, stride, (float*)C, N, ldc,
+                                                                            nrm.gain, nrm.xg, nrm.ldx, nrm.ssq);
+        return br_check_launch();
+    }
+    return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
 }
 
 // kernel: 0 = choose, 1 = tile 128x128 through registers (any shape), 2 = the same 256x128,
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
-// rows), 8 = stream wide (16 < M <= 64, K a multiple of 128); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out
-// of registers in three of the four epilogues and was no faster in the fourth.)
+// rows), 8 = stream wide (16 < M <= 64, K a multiple of 128), 9 = direct-to-LDS tile 64x128
+// (M <= 64); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out of registers in
+// three of the four epilogues and was no faster in the fourth.)
+// `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 9).
 // `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
 // weight rows be split along k (see gemm_split_sum_kernel); BR_GEMM_SCRATCH_BYTES always suffices.
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
-                               size_t ldc, int mode, int kernel, void* scratch, size_t scratch_bytes, hipStream_t s) {
+                               size_t ldc, int mode, int kernel, void* scratch, size_t scratch_bytes, int wl,
+                               hipStream_t s) {
     if (M <= 0 || N <= 0) return BR_OK;
     if (K <= 0 || lda < (size_t)K || mode < 0 || mode > 3) return BR_BAD_ARG;
     if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
-    // kernel / 16: a forced number of runs along k for kernels 5 and 6 (measurements), 0 = by shape
+    // kernel / 16: a forced number of runs along k for kernels 5 and 6, or for kernel 8 a forced tile
+    // height in blocks of 16 rows plus 16 times a forced number of runs (measurements and tests), 0 = by shape
     const int forced_parts = kernel >= 16 ? kernel / 16 : 0;
     kernel %= 16;
     const bf16* A = (const bf16*)A_;
@@ -1302,18 +1408,29 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
     const bool wide_ok = aligned && M > 16 && M <= 64 && K % 128 == 0 && K >= 256 &&
                          (!scratch || (uintptr_t)scratch % 16 == 0);
-    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 8 || kernel < 0) return BR_BAD_ARG;
+    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 9 || kernel < 0 ||
+        (kernel == 9 && (!dma_ok || M > 64)))
+        return BR_BAD_ARG;
+    if (wl != WL_ROWS) {
+        if (wl != WL_BLOCKED || !aligned || K % 128 || (kernel != 0 && kernel < 4)) return BR_BAD_ARG;
+        if (kernel == 0 && M <= 16 && !stream_ok) return BR_BAD_ARG;      // blocked weights have K from 1024
+    }
     // measured at M = 64: many weight rows (gate/up) are 4 % faster through the 64x128 tile, which kernel 3 picks
     const bool chosen = kernel == 0;
     if (kernel == 0)
         kernel = stream_ok ? 7
                  : (wide_ok && !(M > 32 && N >= 16384 && dma_ok)) ? 8
-                 : (aligned && M <= 64) ? 3 : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
-    if (kernel == 8)
-        return M <= 32 ? launch_stream_wide<2>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s)
-                       : launch_stream_wide<4>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s);
-    if (kernel == 7) return M <= 8 ? launch_stream<8, 0>(A, W, C, M, N, K, lda, ldc, mode, s)
-                                   : launch_stream<16, 0>(A, W, C, M, N, K, lda, ldc, mode, s);
+                 : (aligned && M <= 64) ? (wl ? 9 : 3) : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
+    if (kernel == 9) return launch_tile_dma<64, 128, 1, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
+    if (kernel == 8) {
+        const int fh = chosen ? 0 : forced_parts % 16, fp = chosen ? 0 : forced_parts / 16;
+        return M <= 32 ? launch_stream_wide<2>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s, 0,
+                                               StreamNorm{}, fh, fp, wl)
+                       : launch_stream_wide<4>(A, W, C, M, N, K, lda, ldc, mode, (float*)scratch, scratch_bytes, s, 0,
+                                               StreamNorm{}, fh, fp, wl);
+    }
+    if (kernel == 7) return M <= 8 ? launch_stream<8, 0>(A, W, C, M, N, K, lda, ldc, mode, s, StreamNorm{}, wl)
+                                   : launch_stream<16, 0>(A, W, C, M, N, K, lda, ldc, mode, s, StreamNorm{}, wl);
     int parts = 1;
     if (chosen && (kernel == 5 || kernel == 6)) {
         const int cus = br_device_cus();
@@ -1325,9 +1442,9 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
             return BR_BAD_ARG;
         parts = forced_parts;
     }
-    if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s);
-    if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch);
-    if (kernel == 6) return launch_tile_dma<128, 128, 2, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch);
+    if (kernel == 4) return launch_tile_dma<256, 128, 4, 2, 3>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
+    if (kernel == 5) return launch_tile_dma<128, 256, 2, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch, wl);
+    if (kernel == 6) return launch_tile_dma<128, 128, 2, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, parts, (float*)scratch, wl);
     if (kernel == 3) {
         // shapes measured on cold weights (cycled through more than the 256 MB cache)
         const bool wide = N >= 16384;
@@ -1350,7 +1467,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
 
 extern "C" int br_gemm_bf16(const void* A, const void* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                             int mode, hipStream_t s) {
-    return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, nullptr, 0, s);
+    return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, nullptr, 0, WL_ROWS, s);
 }
 
 // what br_gemm_bf16_ex would pick for more than 64 rows (tests and benchmarks print it)
@@ -1377,21 +1494,21 @@ static bool wide_takes(const void* A, const void* W, int M, int K, size_t lda) {
 // needed).  Refuses (BR_BAD_ARG) anything else: the caller then runs the norm itself.
 extern "C" int br_gemm_bf16_norm_prepare(const void* A, const void* W, float* C, int M, int N, int K, size_t lda,
                                          size_t ldc, const float* gain, void* xg, size_t ldx, float* ssq,
-                                         int* ssq_tiles, void* scratch, size_t scratch_bytes, hipStream_t s) {
-    if (M <= 0 || N <= 0) return BR_BAD_ARG;
+                                         int* ssq_tiles, void* scratch, size_t scratch_bytes, int wl, hipStream_t s) {
+    if (M <= 0 || N <= 0 || (wl != WL_ROWS && wl != WL_BLOCKED)) return BR_BAD_ARG;
     if (ldc < (size_t)N || ldx < (size_t)N || !gain || !xg || !ssq || !ssq_tiles) return BR_BAD_ARG;
     StreamNorm nrm{gain, (bf16*)xg, ldx, ssq, 0, 0.f, 0.f};
     if (stream_takes(A, W, M, K, lda) && N % 16 == 0) {
         *ssq_tiles = N / 16;
-        return M <= 8 ? launch_stream<8, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm)
-                      : launch_stream<16, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm);
+        return M <= 8 ? launch_stream<8, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm, wl)
+                      : launch_stream<16, 1>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC, s, nrm, wl);
     }
     if (wide_takes(A, W, M, K, lda) && N % 256 == 0 && scratch && (uintptr_t)scratch % 16 == 0) {
         *ssq_tiles = N / 256;
         return M <= 32 ? launch_stream_wide<2>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC,
-                                               (float*)scratch, scratch_bytes, s, 1, nrm)
+                                               (float*)scratch, scratch_bytes, s, 1, nrm, 0, 0, wl)
                        : launch_stream_wide<4>((const bf16*)A, (const bf16*)W, C, M, N, K, lda, ldc, OUT_F32_ACC,
-                                               (float*)scratch, scratch_bytes, s, 1, nrm);
+                                               (float*)scratch, scratch_bytes, s, 1, nrm, 0, 0, wl);
     }
     return BR_BAD_ARG;
 }
@@ -1400,21 +1517,22 @@ extern "C" int br_gemm_bf16_norm_prepare(const void* A, const void* W, float* C,
 // the product of the normed rows.  mode: 0 bf16, 1 float, 3 SwiGLU.
 extern "C" int br_gemm_bf16_norm_scaled(const void* XG, const void* W, void* C, int M, int N, int K, size_t lda,
                                         size_t ldc, int mode, const float* ssq, int ssq_tiles, int norm_width,
-                                        float eps, void* scratch, size_t scratch_bytes, hipStream_t s) {
+                                        float eps, void* scratch, size_t scratch_bytes, int wl, hipStream_t s) {
     if (M <= 0 || N <= 0) return BR_OK;
+    if (wl != WL_ROWS && wl != WL_BLOCKED) return BR_BAD_ARG;
     if (!ssq || ssq_tiles <= 0 || norm_width <= 0 || (mode != OUT_BF16 && mode != OUT_F32 && mode != OUT_SWIGLU))
         return BR_BAD_ARG;
     if (mode == OUT_SWIGLU ? (N % 16 != 0 || ldc < (size_t)N / 2) : ldc < (size_t)N) return BR_BAD_ARG;
     StreamNorm nrm{nullptr, nullptr, 0, (float*)ssq, ssq_tiles, 1.f / (float)norm_width, eps};
     if (stream_takes(XG, W, M, K, lda))
-        return M <= 8 ? launch_stream<8, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm)
-                      : launch_stream<16, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm);
+        return M <= 8 ? launch_stream<8, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm, wl)
+                      : launch_stream<16, 2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, s, nrm, wl);
     if (wide_takes(XG, W, M, K, lda)) {
         float* sc = (scratch && (uintptr_t)scratch % 16 == 0) ? (float*)scratch : nullptr;
         return M <= 32 ? launch_stream_wide<2>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, sc,
-                                               scratch_bytes, s, 2, nrm)
+                                               scratch_bytes, s, 2, nrm, 0, 0, wl)
                        : launch_stream_wide<4>((const bf16*)XG, (const bf16*)W, C, M, N, K, lda, ldc, mode, sc,
-                                               scratch_bytes, s, 2, nrm);
+                                               scratch_bytes, s, 2, nrm, 0, 0, wl);
     }
     return BR_BAD_ARG;
 }
@@ -1423,5 +1541,10 @@ extern "C" int br_gemm_bf16_norm_scaled(const void* XG, const void* W, void* C, 
 extern "C" int br_gemm_bf16_wide_parts(int M, int N, int K, int mode, size_t scratch_bytes) {
     const int cus = br_device_cus();
     if (!cus || M <= 16 || M > 64 || K % 128 || K < 256) return 0;
-    return wide_parts(M, N, K, mode, cus, scratch_bytes);
+    int hb, parts;
+    wide_shape(M, N, K, mode, cus, scratch_bytes, &hb, &parts);
+    return parts;
 }
+
+// rows of a block of the blocked weight layout (the host lays weights out by it)
+extern "C" int br_gemm_bf16_block_rows() { return WL_BLOCK_ROWS; }

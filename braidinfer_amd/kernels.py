@@ -168,6 +168,51 @@ def convert(a: torch.Tensor, out: torch.Tensor) -> None:
 GEMM_SCRATCH_FLOATS = 16 * 1024 * 1024   # 64 MB: room for the partial sums of the products that the bf16 kernels split along k
 
 
+def weight_blockable(w: torch.Tensor) -> bool:
+    """Whether `block_weight` takes this matrix: bfloat16 [N, K] on the device with K in steps of
+    128 from 1024 (what every bf16 kernel family that reads the blocked layout takes)."""
+    return w.dim() == 2 and w.is_cuda and w.dtype == torch.bfloat16 and w.shape[1] % 128 == 0 and w.shape[1] >= 1024
+
+
+def weight_block_rows() -> int:
+    """Rows of a block of the blocked weight layout (WL_BLOCK_ROWS in csrc/gemm_bf16.hip)."""
+    return int(_fn("gemm_bf16", "br_gemm_bf16_block_rows", [])())
+
+
+def block_weight(w: torch.Tensor) -> torch.Tensor:
+    """The matrix [N, K] as blocks [ceil(N / R), K / 128, R, 128], R = `weight_block_rows()` = 16:
+    R rows by 128 k are contiguous and a strip of R rows is one run along k; rows are padded
+    with zeros to a multiple of R.  The products that stream a weight matrix once per step
+    read it faster in this order than 256 bytes from every row.  `gemm`, `gemm_swiglu`,
+    `gemm_norm_prepare` and `gemm_norm_scaled` take either form and tell them apart by the
+    number of dimensions; N is then the output's width."""
+    if not weight_blockable(w):
+        raise KernelError(f"block_weight: {tuple(w.shape)} {w.dtype} on {w.device} is not taken")
+    N, K = w.shape
+    R = weight_block_rows()
+    nb = -(-N // R)
+    if nb * R != N:
+        w = torch.cat([w, torch.zeros(nb * R - N, K, dtype=w.dtype, device=w.device)], dim=0)
+    return w.view(nb, R, K // 128, 128).permute(0, 2, 1, 3).contiguous()
+
+
+def unblock_weight(wb: torch.Tensor, N: int) -> torch.Tensor:
+    """The rows [N, K] of a blocked matrix (tests, and parts that need rows again)."""
+    nb, kb, R = wb.shape[0], wb.shape[1], wb.shape[2]
+    return wb.permute(0, 2, 1, 3).reshape(nb * R, kb * 128)[:N].contiguous()
+
+
+def _weight_dims(name: str, w: torch.Tensor, n_out: int):
+    """(N, K, layout) of a weight argument: rows [N, K] (layout 0) or blocks (layout 1, N = n_out)."""
+    if w.dim() == 4:
+        R = weight_block_rows()
+        _req(w.shape[2] == R and w.shape[3] == 128 and w.dtype == torch.bfloat16 and w.is_contiguous()
+             and w.shape[0] == -(-n_out // R), f"{name}: blocked weight {tuple(w.shape)} for {n_out} outputs")
+        return n_out, w.shape[1] * 128, 1
+    _req(w.dim() == 2 and w.is_contiguous(), f"{name}: the weight must be [N, K], dense")
+    return w.shape[0], w.shape[1], 0
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, kernel: int = 0,
          scratch: Optional[torch.Tensor] = None) -> None:
     """out[M, N] (+)= a[M, K] @ w[N, K]^T.
@@ -180,7 +225,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     registers, any shape; 3: skinny, M <= 64; 4, 5, 6: 256x128, 128x256 and 128x128 tiles
     loaded straight into LDS, K in steps of 64; 7: streaming by workgroups that stay, M <= 16
     and K in steps of 128 from 1024; 8: the same for 17 to 64 rows, K in steps of 128; 5 or 6 plus
-    16 p: that tile with p runs along k, for measurements); 0 chooses by shape.
+    16 p: that tile with p runs along k, for measurements; 9: a 64x128 tile loaded straight into
+    LDS, M <= 64); 0 chooses by shape.  A weight from `block_weight` is taken by kernels 4 to 9.
     `scratch` (float32, on the device): with it, a bf16 product of more than 16 rows with too
     few tiles to fill the chip is cut along k into runs that a second kernel sums in a fixed order.
     """
@@ -188,11 +234,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     for t in (a, w, out):
         if not t.is_cuda:
             raise KernelError(f"{name}: tensor on {t.device}; kernels run on the GPU only")
-    _req(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm: 2-D tensors")
+    _req(a.dim() == 2 and out.dim() == 2, "gemm: 2-D tensors")
     M, K = a.shape
-    N = w.shape[0]
-    _req(w.shape[1] == K and out.shape == (M, N), f"gemm: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)}")
-    _req(w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1, "gemm: rows must be dense")
+    N, wk, wl = _weight_dims(name, w, out.shape[1])
+    _req(wk == K and out.shape == (M, N), f"gemm: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)}")
+    _req(a.stride(1) == 1 and out.stride(1) == 1, "gemm: rows must be dense")
     lda, ldc = (a.stride(0) if M > 1 else K), (out.stride(0) if M > 1 else N)
     if a.dtype == torch.float32 and w.dtype == torch.float32:
         _req(out.dtype == torch.float32, "gemm: float32 inputs give a float32 output")
@@ -209,9 +255,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         if scratch is not None:
             _req(scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous(), "gemm: scratch must be float32 on the device")
         f = _fn("gemm_bf16", "br_gemm_bf16_ex",
-                [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, _P])
+                [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, c_int, _P])
         _check(f(_ptr(a), _ptr(w), _ptr(out), M, N, K, lda, ldc, mode, kernel, _ptr(scratch),
-                 0 if scratch is None else scratch.numel() * 4, _stream()), name)
+                 0 if scratch is None else scratch.numel() * 4, wl, _stream()), name)
     else:
         raise KernelError(f"gemm: a is {a.dtype} and w is {w.dtype}; both float32 or both bfloat16")
 
@@ -226,16 +272,16 @@ def gemm_swiglu(a: torch.Tensor, w_gu: torch.Tensor, out: torch.Tensor, kernel: 
             raise KernelError(f"gemm_swiglu: tensor on {t.device}; kernels run on the GPU only")
     _req(a.dtype == w_gu.dtype == out.dtype == torch.bfloat16, "gemm_swiglu: bfloat16 only")
     M, K = a.shape
-    N = w_gu.shape[0]
-    _req(N % 16 == 0 and w_gu.shape[1] == K and out.shape == (M, N // 2), "gemm_swiglu: shapes")
-    _req(w_gu.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1, "gemm_swiglu: rows must be dense")
+    N, wk, wl = _weight_dims("gemm_swiglu", w_gu, 2 * out.shape[1])
+    _req(N % 16 == 0 and wk == K and out.shape == (M, N // 2), "gemm_swiglu: shapes")
+    _req(a.stride(1) == 1 and out.stride(1) == 1, "gemm_swiglu: rows must be dense")
     lda, ldc = (a.stride(0) if M > 1 else K), (out.stride(0) if M > 1 else N // 2)
     f = _fn("gemm_bf16", "br_gemm_bf16_ex",
-            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, _P])
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, c_int, _P, c_size_t, c_int, _P])
     if scratch is not None:
         _req(scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous(), "gemm_swiglu: scratch must be float32 on the device")
     _check(f(_ptr(a), _ptr(w_gu), _ptr(out), M, N, K, lda, ldc, 3, kernel, _ptr(scratch),
-             0 if scratch is None else scratch.numel() * 4, _stream()), "gemm_swiglu")
+             0 if scratch is None else scratch.numel() * 4, wl, _stream()), "gemm_swiglu")
 
 
 def gemm_stream_takes(M: int, K: int) -> bool:
@@ -265,18 +311,18 @@ def gemm_norm_prepare(a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, gain: t
     anything else."""
     _dev("gemm_norm_prepare", a, w, x, gain, xg, ssq, scratch)
     M, K = a.shape
-    N = w.shape[0]
+    N, wk, wl = _weight_dims("gemm_norm_prepare", w, x.shape[1])
     _req(a.dtype == w.dtype == xg.dtype == torch.bfloat16 and x.dtype == gain.dtype == ssq.dtype == torch.float32,
          "gemm_norm_prepare: bfloat16 product into float32 rows")
     _req(gemm_stream_takes(M, K) and N % (16 if M <= 16 else 256) == 0, f"gemm_norm_prepare: {M} rows, N {N}, K {K} are not taken")
-    _req(w.shape[1] == K and x.shape == (M, N) and xg.shape == (M, N) and gain.numel() == N
+    _req(wk == K and x.shape == (M, N) and xg.shape == (M, N) and gain.numel() == N
          and ssq.numel() >= (N // 16) * SSQ_LD, "gemm_norm_prepare: shapes")
     tiles = c_int(0)
     f = _fn("gemm_bf16", "br_gemm_bf16_norm_prepare",
-            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, _P, _P, c_size_t, _P, ctypes.POINTER(c_int), _P, c_size_t, _P])
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, _P, _P, c_size_t, _P, ctypes.POINTER(c_int), _P, c_size_t, c_int, _P])
     _check(f(_ptr(a), _ptr(w), _ptr(x), M, N, K, a.stride(0) if M > 1 else K, x.stride(0) if M > 1 else N, _ptr(gain),
              _ptr(xg), xg.stride(0) if M > 1 else N, _ptr(ssq), ctypes.byref(tiles), _ptr(scratch),
-             0 if scratch is None else scratch.numel() * 4, _stream()), "gemm_norm_prepare")
+             0 if scratch is None else scratch.numel() * 4, wl, _stream()), "gemm_norm_prepare")
     return tiles.value
 
 
@@ -288,9 +334,9 @@ def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, tiles: int, eps: float
     `gemm_swiglu`."""
     _dev("gemm_norm_scaled", xg, ssq, w, out, scratch)
     M, K = xg.shape
-    N = w.shape[0]
+    N, wk, wl = _weight_dims("gemm_norm_scaled", w, 2 * out.shape[1] if swiglu else out.shape[1])
     _req(xg.dtype == w.dtype == torch.bfloat16 and ssq.dtype == torch.float32, "gemm_norm_scaled: bfloat16 rows and matrix")
-    _req(gemm_stream_takes(M, K) and w.shape[1] == K and tiles > 0 and ssq.numel() >= tiles * SSQ_LD, "gemm_norm_scaled: sizes")
+    _req(gemm_stream_takes(M, K) and wk == K and tiles > 0 and ssq.numel() >= tiles * SSQ_LD, "gemm_norm_scaled: sizes")
     if swiglu:
         _req(out.dtype == torch.bfloat16 and N % 16 == 0 and out.shape == (M, N // 2), "gemm_norm_scaled: SwiGLU gives bfloat16 [M, N / 2]")
         mode = 3
@@ -298,10 +344,10 @@ def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, tiles: int, eps: float
         _req(out.shape == (M, N) and out.dtype in (torch.bfloat16, torch.float32), "gemm_norm_scaled: out must be [M, N]")
         mode = 0 if out.dtype == torch.bfloat16 else 1
     f = _fn("gemm_bf16", "br_gemm_bf16_norm_scaled",
-            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P, c_int, c_int, c_float, _P, c_size_t, _P])
+            [_P, _P, _P, c_int, c_int, c_int, c_size_t, c_size_t, c_int, _P, c_int, c_int, c_float, _P, c_size_t, c_int, _P])
     _check(f(_ptr(xg), _ptr(w), _ptr(out), M, N, K, xg.stride(0) if M > 1 else K, out.stride(0) if M > 1 else out.shape[1],
              mode, _ptr(ssq), int(tiles), K, float(eps), _ptr(scratch), 0 if scratch is None else scratch.numel() * 4,
-             _stream()), "gemm_norm_scaled")
+             wl, _stream()), "gemm_norm_scaled")
 
 
 def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:

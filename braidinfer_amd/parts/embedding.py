@@ -14,7 +14,7 @@ from .. import kernels as K
 from ..errors import WeightError
 from ..weights import TensorSpec
 from .base import Embedding, OutputHead, Runtime, register_part
-from .linear import linear
+from .linear import linear, stream_layout
 
 
 class TokenEmbedding(Embedding):
@@ -55,6 +55,8 @@ class LMHead(OutputHead):
         if name not in tensors:
             raise WeightError(f"output head: tensor {name} is missing", missing=[name])
         self.weight = tensors[name].contiguous()
+        if not self.tied_to:                       # a tied table is also read row by row by the embedding
+            self.weight = stream_layout(self.weight, rt)
 
     def forward(self, h, out, ws=None) -> None:
         linear(h, self.weight, out, ws)

@@ -422,13 +422,18 @@ def test_single_token_steps_launch_few_norm_kernels(serving, monkeypatch):
     eng.free_slot(s)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_serving_sizes_random_schedule(serving, dtype):
+@pytest.mark.parametrize("dtype,layout", [("float32", ""), ("bfloat16", ""), ("bfloat16", "blocks")])
+def test_serving_sizes_random_schedule(serving, dtype, layout, monkeypatch):
     """The random schedule at the sizes that take the serving kernels: up to 30 requests live,
     so steps bring 1 to 16, 17 to 64 and more rows; chunks of 1 (mostly), a few, and more than
-    a page."""
+    a page.  Once more with every matrix in the blocked layout that only wide matrices get
+    by themselves (none of this configuration is wide enough)."""
     folder, cfg, w = serving
+    if layout:
+        monkeypatch.setenv("BRAIDINFER_WEIGHT_LAYOUT", layout)
     eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=16384)
+    assert eng.model.layers[0].feed_forward.w_gu.dim() == (4 if layout == "blocks" else 2)
+    assert eng.model.lm_head.weight.dim() == (4 if layout == "blocks" else 2)
     rng = np.random.default_rng(11)
     free_before = [g.pool.free_count for g in eng.cache.groups]
     seqs = [tokens(cfg, int(n), 300 + i) for i, n in enumerate(rng.integers(1, 230, 36))]

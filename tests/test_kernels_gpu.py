@@ -182,13 +182,56 @@ def test_gemm_split_along_k_with_scratch(M, N, Kd, kernel):
     assert (again.double() - want).abs().max() < 1e-4 * want.abs().max()
 
 
+@pytest.mark.parametrize("blocked", [False, True])
+@pytest.mark.parametrize("parts", [0, 1, 2, 3])
+@pytest.mark.parametrize("rows", [64, 80, 96, 112, 128])
+def test_gemm_wide_streaming_kernel_tile_heights_and_runs(rows, parts, blocked):
+    # kernel 8 with a forced tile height (rows) and number of runs along k (0: by shape); N is no
+    # multiple of any height, and the first shape has more tiles than the chip has compute units
+    code = 8 + 16 * (rows // 16 + 16 * parts)
+    scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
+    for M, N, Kd in ((64, 257 * rows + 40, 1024), (20, 1000, 1664)):
+        a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
+        want = a.double() @ w.double().T
+        if blocked:
+            w = K.block_weight(w)
+        o32 = torch.empty(M, N, device=DEV)
+        K.gemm(a, w, o32, scratch=scratch, kernel=code)
+        assert (o32.double() - want).abs().max() < 1e-4 * want.abs().max()
+        o16 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+        K.gemm(a, w, o16, scratch=scratch, kernel=code)
+        assert (o16.double() - want).abs().max() < 1e-2 * want.abs().max()
+        base = rnd(M, N, seed=3)
+        acc = base.clone()
+        K.gemm(a, w, acc, accumulate=True, scratch=scratch, kernel=code)
+        assert (acc.double() - (base.double() + want)).abs().max() < 1e-4 * want.abs().max()
+        if parts <= 1:
+            I = 264 if M == 20 else 4104
+            wg, wu = rnd(I, Kd, seed=4, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=5, scale=0.3, dtype=torch.bfloat16)
+            out = torch.empty(M, I, device=DEV, dtype=torch.bfloat16)
+            wgu = K.interleave_gate_up(wg, wu)
+            K.gemm_swiglu(a, K.block_weight(wgu) if blocked else wgu, out, kernel=code)
+            g, u = a.double() @ wg.double().T, a.double() @ wu.double().T
+            want2 = g / (1 + torch.exp(-g)) * u
+            assert (out.double() - want2).abs().max() < 1e-2 * want2.abs().max()
+        else:
+            with pytest.raises(KernelError):             # the runs of a split product need scratch
+                K.gemm(a, w, o32, kernel=code)
+    with pytest.raises(KernelError):
+        K.gemm(a, w, o32, scratch=scratch, kernel=8 + 16 * 3)       # 48 rows: no such tile
+
+
 @pytest.mark.parametrize("M,H,Kd,N2", [(1, 1024, 1024, 304), (8, 1152, 2048, 4112), (13, 2048, 1280, 96), (16, 1024, 1536, 1000),
                                        (17, 1024, 2048, 304), (40, 2048, 1024, 4112), (64, 1280, 4096, 96)])
-def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
+@pytest.mark.parametrize("blocked", [False, True])
+def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2, blocked):
     # x += a W1^T, then rmsnorm(x) W2^T, in two kernels instead of three
     a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
     w1 = rnd(H, Kd, seed=2, scale=0.05, dtype=torch.bfloat16)
     w2 = rnd(N2, H, seed=3, scale=0.5, dtype=torch.bfloat16)
+    w1_rows, w2_rows = w1, w2
+    if blocked:
+        w1, w2 = K.block_weight(w1), K.block_weight(w2)
     x0 = rnd(M, H, seed=4) * torch.logspace(-1, 1, M, device=DEV)[:, None]     # rows of very different sizes
     gain = 1.0 + 0.5 * rnd(H, seed=5)
     eps = 1e-5
@@ -200,13 +243,13 @@ def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
         assert K.gemm_wide_parts(M, H, Kd, K.GEMM_SCRATCH_FLOATS) >= 2
     tiles = K.gemm_norm_prepare(a, w1, x, gain, xg, ssq, scratch)
     assert tiles == (H // 16 if M <= 16 else H // 256)
-    xw = x0.double() + a.double() @ w1.double().T
+    xw = x0.double() + a.double() @ w1_rows.double().T
     assert (x.double() - xw).abs().max() < 1e-4 * xw.abs().max()
     assert (xg.double() - xw * gain.double()).abs().max() < 1e-2 * (xw * gain.double()).abs().max()
     sums = ssq[:tiles * K.SSQ_LD].view(tiles, K.SSQ_LD)[:, :M].double()
     assert (sums.sum(0) - (xw * xw).sum(-1)).abs().max() < 1e-4 * (xw * xw).sum(-1).max()
     normed = xw / torch.sqrt((xw * xw).mean(-1, keepdim=True) + eps) * gain.double()
-    want = normed @ w2.double().T
+    want = normed @ w2_rows.double().T
     o32 = torch.empty(M, N2, device=DEV)
     K.gemm_norm_scaled(xg, ssq, tiles, eps, w2, o32, scratch=scratch)
     assert (o32.double() - want).abs().max() < 1e-2 * want.abs().max()
@@ -229,6 +272,49 @@ def test_gemm_prepares_the_next_norm_and_the_next_product_uses_it(M, H, Kd, N2):
     with pytest.raises(KernelError):
         K.gemm_norm_prepare(rnd(65, Kd, dtype=torch.bfloat16), w1, torch.zeros(65, H, device=DEV), gain,
                             torch.empty(65, H, device=DEV, dtype=torch.bfloat16), ssq, scratch)
+
+
+@pytest.mark.parametrize("kernel", [0, 4, 5, 6, 7, 8, 9, 5 + 16 * 2, 6 + 16 * 4])
+@pytest.mark.parametrize("M,N,Kd", [(1, 100, 1024), (8, 301, 1152), (16, 4100, 1024), (17, 200, 1280), (64, 16500, 1024),
+                                    (48, 4100, 2048), (65, 301, 1024), (130, 514, 1152), (300, 700, 1024), (513, 260, 2048)])
+def test_gemm_with_blocked_weights(M, N, Kd, kernel):
+    # the weight as blocks of 16 rows x 128 k (block_weight): every kernel that takes it, every epilogue
+    k = kernel % 16
+    if k == 7 and M > 16 or k == 8 and not 16 < M <= 64 or k == 9 and M > 64:
+        pytest.skip("not this kernel's rows")
+    w_rows = rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
+    a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), K.block_weight(w_rows)
+    assert w.shape == (-(-N // 16), Kd // 128, 16, 128) and torch.equal(K.unblock_weight(w, N), w_rows)
+    want = a.double() @ w_rows.double().T
+    scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
+    o32 = torch.empty(M, N, device=DEV)
+    K.gemm(a, w, o32, kernel=kernel, scratch=scratch)
+    assert (o32.double() - want).abs().max() < 1e-4 * want.abs().max()
+    rows = torch.empty(M, N, device=DEV)
+    K.gemm(a, w_rows, rows, kernel=kernel, scratch=scratch)
+    assert torch.equal(rows, o32)                                    # the layout changes no sum
+    o16 = torch.empty(M, N + 8, device=DEV, dtype=torch.bfloat16)[:, 3:3 + N]
+    K.gemm(a, w, o16, kernel=kernel, scratch=scratch)
+    assert (o16.double() - want).abs().max() < 1e-2 * want.abs().max()
+    base = rnd(M, N, seed=3)
+    acc = base.clone()
+    K.gemm(a, w, acc, accumulate=True, kernel=kernel, scratch=scratch)
+    assert (acc.double() - (base.double() + want)).abs().max() < 1e-4 * want.abs().max()
+    if kernel < 16:
+        I = (N // 2) // 8 * 8
+        wg, wu = rnd(I, Kd, seed=4, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=5, scale=0.3, dtype=torch.bfloat16)
+        out = torch.empty(M, I, device=DEV, dtype=torch.bfloat16)
+        K.gemm_swiglu(a, K.block_weight(K.interleave_gate_up(wg, wu)), out, kernel=kernel)
+        g, u = a.double() @ wg.double().T, a.double() @ wu.double().T
+        sw = g / (1 + torch.exp(-g)) * u
+        assert (out.double() - sw).abs().max() < 1e-2 * sw.abs().max()
+    for bad in (1, 2, 3):
+        with pytest.raises(KernelError):                 # these read rows only
+            K.gemm(a, w, o32, kernel=bad)
+    with pytest.raises(KernelError):
+        K.gemm(a, w, torch.empty(M, N + 64, device=DEV))             # a width the blocks do not have
+    with pytest.raises(KernelError):
+        K.block_weight(rnd(64, 960, dtype=torch.bfloat16))           # K in steps of 128 from 1024
 
 
 def test_gemm_reference_vectors():
