@@ -1131,6 +1131,10 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
     // of chunks, each lane's addresses) is worked out once per unit, so that a chunk costs each wave its
     // loads, an address step and a count.
     int is_u = 0, is_left = 0, cp_u = 0, cp_left = 0;       // units begun, chunks of the current one to go
+    int is_wrap = 0, is_len = 0;                            // chunks to go before the run's first chunk is next; the run's length
+    // Where in its run of chunks a workgroup starts (it wraps round to the run's first chunk): workgroups
+    // that walk their rows in step ask the same few memory channels at the same time.
+    const unsigned start_hash = ((unsigned)blockIdx.x * 2654435761u) >> 8;
     int issued = 0, done = 0;
     unsigned is_off = 0, cp_off = 0;                        // the ring's stage to fill, to multiply (bytes)
     const bf16* src[NDMA];                                  // this lane's 16 bytes of each of its loads
@@ -1146,17 +1150,20 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
         const int unit_ = (int)blockIdx.x + is_u * (int)gridDim.x;                                            \
         const int tile_ = unit_ / parts, c0_ = (unit_ % parts) * cpp;                                         \
         is_left = (c0_ + cpp < nch ? c0_ + cpp : nch) - c0_;                                                  \
+        is_len = is_left;                                                                                     \
+        const int rot_ = (int)(start_hash % (unsigned)is_left);                                               \
+        is_wrap = is_left - rot_;                                                                             \
         _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                 \
             const int row_ = WIDE_LOAD_INDEX(q_) * 4 + (lane >> 4);                                           \
             const bf16* gp_;                                                                                  \
             if (row_ < H) {                                                                                   \
                 int n_ = tile_ * H + row_;                                                                    \
                 if (n_ > N - 1) n_ = N - 1;                                                                   \
-                gp_ = W + w_row_base(n_, K, wl) + (size_t)c0_ * wstep;                                        \
+                gp_ = W + w_row_base(n_, K, wl) + (size_t)(c0_ + rot_) * wstep;                               \
             } else {                                                                                          \
                 int m_ = row_ - H;                                                                            \
                 if (m_ > M - 1) m_ = M - 1;                                                                   \
-                gp_ = A + (size_t)m_ * lda + (size_t)c0_ * 128;                                               \
+                gp_ = A + (size_t)m_ * lda + (size_t)(c0_ + rot_) * 128;                                      \
             }                                                                                                 \
             src[q_] = gp_ + (((lane & 15) ^ (row_ & 7)) * 8);                                                 \
         }                                                                                                     \
@@ -1167,6 +1174,10 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
             const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + is_off + WIDE_LOAD_INDEX(q_) * 1024); \
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q_]) : "m0"); \
             src[q_] += WIDE_LOAD_INDEX(q_) * 4 < H ? wstep : 128;                                             \
+        }                                                                                                     \
+        if (--is_wrap == 0) {                              /* on to the run's first chunk */                  \
+            _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_)                                               \
+                src[q_] -= (size_t)is_len * (WIDE_LOAD_INDEX(q_) * 4 < H ? wstep : 128);                      \
         }                                                                                                     \
         ++issued;                                                                                             \
         is_off = is_off + STAGE == S * STAGE ? 0 : is_off + STAGE;                                            \
@@ -1415,11 +1426,10 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
         if (wl != WL_BLOCKED || !aligned || K % 128 || (kernel != 0 && kernel < 4)) return BR_BAD_ARG;
         if (kernel == 0 && M <= 16 && !stream_ok) return BR_BAD_ARG;      // blocked weights have K from 1024
     }
-    // measured at M = 64: many weight rows (gate/up) are 4 % faster through the 64x128 tile, which kernel 3 picks
     const bool chosen = kernel == 0;
     if (kernel == 0)
         kernel = stream_ok ? 7
-                 : (wide_ok && !(M > 32 && N >= 16384 && dma_ok)) ? 8
+                 : wide_ok ? 8
                  : (aligned && M <= 64) ? (wl ? 9 : 3) : (!dma_ok ? 1 : (N > 128 ? 5 : 6));
     if (kernel == 9) return launch_tile_dma<64, 128, 1, 4, 3>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
     if (kernel == 8) {
