@@ -290,7 +290,10 @@ __device__ __forceinline__ size_t w_row_base(int n, int K, int wl) {
                          : "m0");                                                                              \
             src[q] += (knext & 1) ? hop[q] : DMA_BK;       /* k-tiles are issued in order, (kt) is the next */ \
         }                                                                                                      \
-        ++knext;                                                                                               \
+        if (++knext == kwrap) {                            /* on to the run's first k-tile */                  \
+            knext = kt0;                                                                                       \
+            _Pragma("unroll") for (int q = 0; q < INSTR; ++q) src[q] -= (size_t)(nk_run >> 1) * (DMA_BK + hop[q]); \
+        }                                                                                                      \
     } while (0)
 #define DMA_COMPUTE(ST)                                                                                        \
     do {                                                                                                       \
@@ -362,7 +365,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
     int dst[INSTR];
     int hop[INSTR];                                      // elements from an odd k-tile to the next (even) one
     const int kt0 = (int)blockIdx.y * kt_per_part;       // the run's first k-tile
-    int knext = kt0;                                     // the k-tile that src[] points at
+    int nk_run = K / DMA_BK - kt0;                       // k-tiles of this run
+    if (nk_run > kt_per_part) nk_run = kt_per_part;
+    // Where in its run a workgroup starts (it wraps round): workgroups that walk k in step ask the same few
+    // memory channels at the same time.  Only with a single row of tiles (3 to 6 % on wide matrices at
+    // 65 to 128 rows): workgroups that share a tile live on reading the same k-tile at the same time (a start
+    // of its own for each made 2,048 rows 50 % slower, one per tile column made 2 rows of tiles 5 to 12 %
+    // slower).  An even start in an even run, so that pairs of k-tiles (one 128-wide block of the blocked
+    // layout) stay together.
+    const int rot = (tiles_m == 1 && nk_run % 2 == 0 && kt0 % 2 == 0)
+                        ? 2 * (int)((((unsigned)tile_n * 2654435761u) >> 8) % (unsigned)(nk_run / 2)) : 0;
+    const int kwrap = kt0 + nk_run;
+    int knext = kt0 + rot;                               // the k-tile that src[] points at
 #pragma unroll
     for (int q = 0; q < INSTR; ++q) {
         const int R = (q * NW + wave) * 8 + (lane >> 3);
@@ -370,20 +384,19 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
         if (R < BM) {
             int r = m0 + R;
             if (r > M - 1) r = M - 1;
-            src[q] = A + (size_t)r * lda + c * 8 + (size_t)kt0 * DMA_BK;
+            src[q] = A + (size_t)r * lda + c * 8 + (size_t)(kt0 + rot) * DMA_BK;
             hop[q] = DMA_BK;
         } else {
             int r = n0 + R - BM;
             if (r > N - 1) r = N - 1;
             src[q] = W + w_row_base(r, K, wl) + c * 8 +
-                     (wl ? (size_t)(kt0 >> 1) * WL_BLOCK_ELEMS + (kt0 & 1) * DMA_BK : (size_t)kt0 * DMA_BK);
+                     (wl ? (size_t)((kt0 + rot) >> 1) * WL_BLOCK_ELEMS + (kt0 & 1) * DMA_BK : (size_t)(kt0 + rot) * DMA_BK);
             hop[q] = wl ? WL_BLOCK_ELEMS - DMA_BK : DMA_BK;
         }
         hop[q] = __builtin_amdgcn_readfirstlane(hop[q]);             // the same for the 8 rows of a wave-load
         dst[q] = (q * NW + wave) * 1024;
     }
-    int nk = K / DMA_BK - kt0;
-    if (nk > kt_per_part) nk = kt_per_part;
+    const int nk = nk_run;
     if (S == 2) {
         DMA_ISSUE(st0, 0);
         for (int kt = 0; kt < nk; kt += 2) {
