@@ -167,27 +167,30 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 
 // ----------------------------------------------------------- prefill through LDS ----
 // The same computation with the keys and values of a page staged in LDS once per
-// workgroup: grid = (row tiles of 256, nkv, sequences), block = 512 (8 waves of 32 rows).
+// workgroup: grid = (row tiles of 32 NW, nkv, sequences), block = 64 NW (NW waves of 32 rows).
 // The page after the current one is fetched into registers while the current one is
 // multiplied, and written to the other LDS buffer afterwards.  Tiles are taken from the
 // last (most keys) to the first so the long workgroups start first.
 #define KPAD 8
 #define VLD 72
-template <int NB>
-__global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4 ? 2 : 1, 2))) void attn_prefill_lds_kernel(
     const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
-    int table_stride, const bf16* __restrict__ cache, int nq, int nkv, int hd, int window, float scale) {
+    int table_stride, const bf16* __restrict__ cache, int nq, int nkv, int hd, int window, float scale, int pair) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int b = blockIdx.z, kvh = blockIdx.y;
     const int slot = slots[b];
     const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
     const int G = nq / nkv;
     const int rows_total = n_new * G;
-    const int tile = gridDim.x - 1 - blockIdx.x;
-    if (tile * 256 >= rows_total) return;                 // the whole workgroup leaves together
+    // Long tiles first when the workgroups run in several rounds; when all are resident at once
+    // (`pair`), the second half of the kv heads goes from short to long, so that the two workgroups of a
+    // compute unit are a long and a short one (measured at 2,048 tokens: 113 -> 99 us).
+    const int tile = (pair && ((blockIdx.y * 2 / gridDim.y) & 1)) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+    if (tile * (NW * 32) >= rows_total) return;                 // the whole workgroup leaves together
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row0 = tile * 256 + wave * 32;
+    const int row0 = tile * (NW * 32) + wave * 32;
     const bool wave_ok = row0 < rows_total;
     const int c = lane & 31, g = lane >> 5;
     const int row = row0 + c;
@@ -204,8 +207,8 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
     // per wave and per workgroup: the positions of the first and last query row
     const int w_last_row = (row0 + 31 < rows_total ? row0 + 31 : rows_total - 1);
     const int pq_min_w = start + (wave_ok ? row0 : rows_total - 1) / G, pq_max_w = start + w_last_row / G;
-    const int g_last_row = (tile * 256 + 255 < rows_total ? tile * 256 + 255 : rows_total - 1);
-    const int pq_min_g = start + (tile * 256) / G, pq_max_g = start + g_last_row / G;
+    const int g_last_row = (tile * (NW * 32) + NW * 32 - 1 < rows_total ? tile * (NW * 32) + NW * 32 - 1 : rows_total - 1);
+    const int pq_min_g = start + (tile * (NW * 32)) / G, pq_max_g = start + g_last_row / G;
 
     const int kld = hd + KPAD;
     bf16* Ks = (bf16*)smem_raw;                          // [2][64][kld]
@@ -234,7 +237,8 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
     const int pg_first = lo / PAGE, pg_last = pq_max_g / PAGE;
 
     // cooperative loads: chunk id -> 8 consecutive elements of the page's K part / V^T part
-    constexpr int CH = (NB * 32 * PAGE / 8 + 511) / 512;  // 16-byte chunks per thread and part (NB * 32 >= hd)
+    constexpr int NT = NW * 64;
+    constexpr int CH = (NB * 32 * PAGE / 8 + NT - 1) / NT;  // 16-byte chunks per thread and part (NB * 32 >= hd)
     bf16x8 rk[CH], rv[CH];
     const int kchunks = PAGE * hd / 8;                   // chunks that exist in each part
     auto gload = [&](int pi) {
@@ -242,7 +246,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
         const int limit_local = ctx - pi * PAGE;
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-            const int id = tid + j * 512;
+            const int id = tid + j * NT;
             if (id < kchunks) {
                 rk[j] = *(const bf16x8*)(pg + k_off + (size_t)id * 8);
                 bf16x8 v = *(const bf16x8*)(pg + v_off + (size_t)id * 8);
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
         bf16* vs = Vs + buf * NB * 32 * VLD;
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-            const int id = tid + j * 512;
+            const int id = tid + j * NT;
             if (id < kchunks) {
                 const int e0 = id * 8;
                 *(bf16x8*)(ks + (e0 / hd) * kld + (e0 % hd)) = rk[j];
@@ -298,19 +302,21 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
             // needs no mask
             const bool whole = row0 + 31 < rows_total && kb + 31 <= pq_min_w &&
                                (window <= 0 || kb > pq_max_w - window);
+            // the scale is positive: the largest raw score is the largest scaled one, and the scaling rides
+            // on the subtraction of the maximum (one fused multiply-add per score)
             if (whole) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) { sv[r] = s_acc[r] * scale2; mx = fmaxf(mx, sv[r]); }
+                for (int r = 0; r < 16; ++r) { sv[r] = s_acc[r]; mx = fmaxf(mx, sv[r]); }
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
                     const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
-                    sv[r] = ok ? s_acc[r] * scale2 : -INFINITY;
+                    sv[r] = ok ? s_acc[r] : -INFINITY;
                     mx = fmaxf(mx, sv[r]);
                 }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;
             const float m_new = fmaxf(m, mx);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
             // the accumulators are rescaled only when some row's maximum moved
@@ -327,7 +333,7 @@ __global__ __launch_bounds__(512) void attn_prefill_lds_kernel(
             bf16x8 p1, p2;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float p = fast_exp2(sv[r] - m_use);
+                const float p = fast_exp2(fmaf(sv[r], scale2, -m_use));
                 psum += p;
                 if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
             }
@@ -822,18 +828,26 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
                                     int hd, int page, int window, float scale, int variant, hipStream_t s) {
     if (B <= 0 || max_new <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
-        q_stride % 8 || ((uintptr_t)q % 16) || nkv > 65535 || B > 65535)
+        q_stride % 8 || ((uintptr_t)q % 16) || nkv > 65535 || B > 65535 || !(scale > 0.f))
         return BR_BAD_ARG;
     const int G = nq / nkv;
-    // variant 0: choose; 1: fragments straight from the cache; 2: pages staged in LDS
-    if (variant == 0) variant = ((size_t)max_new * G >= 256 && hd <= 192) ? 2 : 1;   // beyond 192 the LDS form spills registers
-    if (variant == 2) {
-        dim3 grid2(((size_t)max_new * G + 255) / 256, nkv, B);
+    // variant 0: choose; 1: fragments straight from the cache; 2: pages staged in LDS by workgroups of
+    // 8 waves; 3: the same by workgroups of 4 waves
+    // (up to head size 128 two such workgroups fit a compute unit and fill each other's gaps between the
+    // page barriers: 18 to 21 % faster at 8,192 tokens; beyond 128 four waves spill registers, beyond 192 eight do)
+    if (variant == 0) variant = ((size_t)max_new * G >= 256 && hd <= 192) ? (hd <= 128 ? 3 : 2) : 1;
+    if (variant == 2 || variant == 3) {
+        const int variant_waves = variant == 3 ? 4 : 8;
+        const int nw = variant_waves;
+        dim3 grid2(((size_t)max_new * G + nw * 32 - 1) / (nw * 32), nkv, B);
+        const int cus = br_device_cus();
+        const int pair = nw == 4 && cus > 0 && (long long)grid2.x * nkv * B <= 2LL * cus;
         const int nb = nb_of(hd) == 5 ? 6 : (nb_of(hd) == 7 ? 8 : nb_of(hd));
         const size_t lds = (size_t)2 * (PAGE * (hd + KPAD) + nb * 32 * VLD) * sizeof(bf16);
-#define BR_PREFILL_LDS(N)                                                                                  \
+#define BR_PREFILL_LDS(N) do { if (nw == 4) BR_PREFILL_LDS2(N, 4); else BR_PREFILL_LDS2(N, 8); } while (0)
+#define BR_PREFILL_LDS2(N, NW_)                                                                            \
     do {                                                                                                   \
-        auto kern = attn_prefill_lds_kernel<N>;                                                            \
+        auto kern = attn_prefill_lds_kernel<N, NW_>;                                                       \
         static bool set = false;                                                                           \
         if (!set) {                                                                                        \
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,         \
@@ -841,9 +855,9 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
                 return BR_LAUNCH_FAILED;                                                                   \
             set = true;                                                                                    \
         }                                                                                                  \
-        kern<<<grid2, 512, lds, s>>>((const bf16*)q, q_stride, (bf16*)out, cu_seqlens, slots, ctx_lens,   \
+        kern<<<grid2, NW_ * 64, lds, s>>>((const bf16*)q, q_stride, (bf16*)out, cu_seqlens, slots, ctx_lens, \
                                      block_table, table_stride, (const bf16*)cache, nq, nkv, hd, window,   \
-                                     scale);                                                               \
+                                     scale, pair);                                                         \
     } while (0)
         switch (nb) {
             case 1: BR_PREFILL_LDS(1); break;
@@ -854,6 +868,7 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
             default: BR_PREFILL_LDS(8); break;
         }
 #undef BR_PREFILL_LDS
+#undef BR_PREFILL_LDS2
         return br_check_launch();
     }
     dim3 grid(((size_t)max_new * G + 127) / 128, nkv, B);
