@@ -371,6 +371,203 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
         }
 }
 
+// ------------------------------------------------- prefill through an LDS ring ----
+// Head sizes 64 and 128: the same computation by workgroups of 4 waves (128 rows), two to a compute
+// unit, with the pages brought into a ring of two LDS stages by direct global-to-LDS loads: the page
+// after the current one is in flight while this one is multiplied, nothing passes through registers and
+// nothing is stored to LDS by the waves.  A stage holds the page's keys [64][HD] and values [HD][64] as
+// they lie in the cache; 16-byte columns are XOR-swizzled by the row (through the choice of the global
+// column a lane fetches) so that the operand reads of 16 consecutive lanes spread over the banks.  The
+// workgroup's page numbers are kept in LDS (at most PF_MAX_RUN): no wave waits for a read of the block
+// table behind its loads in flight.  One barrier per page.
+#define PF_MAX_RUN 2048
+template <int HD>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_dma_kernel(
+    const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
+    int table_stride, const bf16* __restrict__ cache, int nq, int nkv, int window, float scale, int pair) {
+    constexpr int NB = HD / 32, NW = 4;
+    constexpr int KROWB = HD * 2, KCOLS = KROWB / 16;       // a key row in bytes, in 16-byte columns
+    constexpr int KB = PAGE * KROWB, STAGE = 2 * KB;        // keys, then values [HD][128 bytes]
+    constexpr int KINSTR = KB / 1024, NDMA = STAGE / 1024 / NW;   // wave-loads: of the keys; per wave and page
+    constexpr int KROWS = 1024 / KROWB;                     // key rows per wave-load
+    extern __shared__ __attribute__((aligned(1024))) unsigned char dsm[];
+    int* bts = (int*)(dsm + 2 * STAGE);
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int slot = slots[b];
+    const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
+    const int G = nq / nkv;
+    const int rows_total = n_new * G;
+    const int tile = (pair && ((blockIdx.y * 2 / gridDim.y) & 1)) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+    if (tile * (NW * 32) >= rows_total) return;           // the whole workgroup leaves together
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row0 = tile * (NW * 32) + wave * 32;
+    const bool wave_ok = row0 < rows_total;
+    const int c = lane & 31, g = lane >> 5;
+    const int row = row0 + c;
+    const bool row_ok = row < rows_total;
+    const int rr = row_ok ? row : rows_total - 1;
+    const int tok = rr / G, head = kvh * G + rr % G;
+    bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * HD;
+    if (slot < 0) {
+        if (row_ok && g == 0) for (int d = 0; d < HD; ++d) orow[d] = (bf16)0.f;
+        return;
+    }
+    const int ctx = ctx_lens[b], start = ctx - n_new;
+    const int pq = start + tok;
+    const int w_last_row = (row0 + 31 < rows_total ? row0 + 31 : rows_total - 1);
+    const int pq_min_w = start + (wave_ok ? row0 : rows_total - 1) / G, pq_max_w = start + w_last_row / G;
+    const int g_last_row = (tile * (NW * 32) + NW * 32 - 1 < rows_total ? tile * (NW * 32) + NW * 32 - 1 : rows_total - 1);
+    const int pq_min_g = start + (tile * (NW * 32)) / G, pq_max_g = start + g_last_row / G;
+    int lo = 0;
+    if (window > 0 && pq_min_g - window + 1 > 0) lo = pq_min_g - window + 1;
+    const int pg_first = lo / PAGE, pg_last = pq_max_g / PAGE;
+    const int n_run = pg_last - pg_first + 1;               // at most PF_MAX_RUN (the launcher checks)
+    const int* bt = block_table + (size_t)slot * table_stride;
+    for (int i = tid; i < n_run; i += NW * 64) bts[i] = bt[pg_first + i];
+
+    const bf16* qrow = q + (size_t)(t0 + tok) * q_stride + (size_t)head * HD;
+    bf16x8 qf[2 * NB];
+#pragma unroll
+    for (int s = 0; s < 2 * NB; ++s) qf[s] = *(const bf16x8*)(qrow + s * 16 + 8 * g);
+    f32x16 acc_o[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+    const float scale2 = scale * LOG2E;
+    const size_t page_elems = (size_t)2 * nkv * PAGE * HD;
+    const size_t k_off = (size_t)kvh * PAGE * HD, v_off = ((size_t)nkv + kvh) * PAGE * HD;
+    // the query has arrived before the loop: a wait for it inside would also wait for the page in flight
+#pragma unroll
+    for (int s = 0; s < 2 * NB; ++s) asm volatile("" ::"v"(qf[s]));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                                        // the page numbers are in LDS
+
+    const unsigned ring_lds = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)dsm);
+    // this lane's part of each of its wave-loads: offset in the page (elements) and in the stage (bytes)
+    int goff[NDMA];
+#pragma unroll
+    for (int q_ = 0; q_ < NDMA; ++q_) {
+        const int in_ = wave * NDMA + q_;
+        if (in_ < KINSTR) {
+            const int row_ = in_ * KROWS + lane / KCOLS;
+            const int swz_ = KCOLS == 16 ? (row_ & 15) : ((row_ >> 1) & 7);
+            goff[q_] = (int)k_off + row_ * HD + (((lane % KCOLS) ^ swz_) * 8);
+        } else {
+            const int row_ = (in_ - KINSTR) * 8 + (lane >> 3);
+            goff[q_] = (int)v_off + row_ * PAGE + (((lane & 7) ^ ((row_ >> 1) & 7)) * 8);
+        }
+    }
+#define PF_ISSUE(I)                                                                                          \
+    do {                                                                                                     \
+        const bf16* pg_ = cache + (size_t)bts[I] * page_elems;                                               \
+        _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                \
+            const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + ((I) & 1) * STAGE + (wave * NDMA + q_) * 1024); \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(pg_ + goff[q_]) : "m0"); \
+        }                                                                                                    \
+    } while (0)
+
+    PF_ISSUE(0);
+    for (int i = 0; i < n_run; ++i) {
+        const int pi = pg_first + i;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                 // every wave's part of page i is there; page i - 1 is done with
+        asm volatile("" ::: "memory");
+        if (i + 1 < n_run) PF_ISSUE(i + 1);
+        const unsigned char* st = dsm + (i & 1) * STAGE;
+        const bool tail_page = (pi + 1) * PAGE > ctx;      // values beyond the context are stale: read them as zero
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int kl = half * 32, kb = pi * PAGE + kl;
+            // blocks no row of this wave can see are skipped
+            if (!wave_ok || kb > pq_max_w || (window > 0 && kb + 31 <= pq_min_w - window)) continue;
+            const int krow = kl + key_of_row32(c);
+            const int kswz_ = KCOLS == 16 ? (krow & 15) : ((krow >> 1) & 7);
+            const unsigned char* kp = st + krow * KROWB;
+            f32x16 s_acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < 2 * NB; ++s) {
+                const bf16x8 kf = *(const bf16x8*)(kp + (((2 * s + g) ^ kswz_) * 16));
+                s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+            }
+            float sv[16];
+            float mx = -INFINITY;
+            const bool whole = row0 + 31 < rows_total && kb + 31 <= pq_min_w &&
+                               (window <= 0 || kb > pq_max_w - window);
+            if (whole) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { sv[r] = s_acc[r]; mx = fmaxf(mx, sv[r]); }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+                    const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
+                    sv[r] = ok ? s_acc[r] : -INFINITY;
+                    mx = fmaxf(mx, sv[r]);
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;      // the scale is positive
+            const float m_new = fmaxf(m, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const bool moved = __any(m_new > m);
+            if (moved) {
+                const float corr = fast_exp2(m - m_use);
+                lsum *= corr;
+#pragma unroll
+                for (int i2 = 0; i2 < NB; ++i2)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc_o[i2][r] *= corr;
+            }
+            float psum = 0.f;
+            bf16x8 p1, p2;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = fast_exp2(fmaf(sv[r], scale2, -m_use));
+                psum += p;
+                if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
+            }
+            lsum += psum;
+            m = m_new;
+#pragma unroll
+            for (int i2 = 0; i2 < NB; ++i2) {
+                const int vrow = i2 * 32 + c;
+                const unsigned char* vp = st + KB + vrow * 128;
+                const int vswz = (vrow >> 1) & 7;
+                bf16x8 v1 = *(const bf16x8*)(vp + (((kl / 8 + g) ^ vswz) * 16));
+                bf16x8 v2 = *(const bf16x8*)(vp + (((kl / 8 + g + 2) ^ vswz) * 16));
+                if (tail_page) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (kb + 8 * g + e >= ctx) v1[e] = (bf16)0.f;
+                        if (kb + 16 + 8 * g + e >= ctx) v2[e] = (bf16)0.f;
+                    }
+                }
+                acc_o[i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i2], 0, 0, 0);
+                acc_o[i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i2], 0, 0, 0);
+            }
+        }
+    }
+#undef PF_ISSUE
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (!row_ok) return;
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int d = i * 32 + 8 * r4 + 4 * g;
+            bf16x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (bf16)(acc_o[i][4 * r4 + e] * inv);
+            *(bf16x4*)(orow + d) = o;
+        }
+}
+
 // ---------------------------------------------------------------------- decode ------
 // One token per sequence.  grid = (splits, nkv * head blocks, sequences), block = 256.
 // The pages a query sees are cut into `nsplit` runs; the 4 waves of a workgroup take a
@@ -832,10 +1029,35 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
         return BR_BAD_ARG;
     const int G = nq / nkv;
     // variant 0: choose; 1: fragments straight from the cache; 2: pages staged in LDS by workgroups of
-    // 8 waves; 3: the same by workgroups of 4 waves
+    // 8 waves; 3: the same by workgroups of 4 waves; 4: pages brought into an LDS ring by direct loads
+    // (head sizes 64 and 128, block tables of at most PF_MAX_RUN pages)
+    const bool dma_ok = (hd == 64 || hd == 128) && table_stride <= PF_MAX_RUN && (uintptr_t)cache % 16 == 0;
+    if (variant < 0 || variant > 4 || (variant == 4 && !dma_ok)) return BR_BAD_ARG;
     // (up to head size 128 two such workgroups fit a compute unit and fill each other's gaps between the
     // page barriers: 18 to 21 % faster at 8,192 tokens; beyond 128 four waves spill registers, beyond 192 eight do)
-    if (variant == 0) variant = ((size_t)max_new * G >= 256 && hd <= 192) ? (hd <= 128 ? 3 : 2) : 1;
+    if (variant == 0) variant = ((size_t)max_new * G >= 256 && hd <= 192) ? (dma_ok ? 4 : hd <= 128 ? 3 : 2) : 1;
+    if (variant == 4) {
+        dim3 grid4(((size_t)max_new * G + 127) / 128, nkv, B);
+        const int cus = br_device_cus();
+        const int pair = cus > 0 && (long long)grid4.x * nkv * B <= 2LL * cus;
+#define BR_PREFILL_DMA(HD_)                                                                                \
+    do {                                                                                                   \
+        auto kern = attn_prefill_dma_kernel<HD_>;                                                          \
+        constexpr size_t lds4 = (size_t)2 * 2 * PAGE * HD_ * 2 + PF_MAX_RUN * sizeof(int);                 \
+        static bool set = false;                                                                           \
+        if (!set) {                                                                                        \
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds4) != hipSuccess) \
+                return BR_LAUNCH_FAILED;                                                                   \
+            set = true;                                                                                    \
+        }                                                                                                  \
+        kern<<<grid4, 256, lds4, s>>>((const bf16*)q, q_stride, (bf16*)out, cu_seqlens, slots, ctx_lens,  \
+                                      block_table, table_stride, (const bf16*)cache, nq, nkv, window,      \
+                                      scale, pair);                                                        \
+    } while (0)
+        if (hd == 128) BR_PREFILL_DMA(128); else BR_PREFILL_DMA(64);
+#undef BR_PREFILL_DMA
+        return br_check_launch();
+    }
     if (variant == 2 || variant == 3) {
         const int variant_waves = variant == 3 ? 4 : 8;
         const int nw = variant_waves;
