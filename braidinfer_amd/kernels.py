@@ -381,13 +381,16 @@ def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu
                            cache: torch.Tensor, B: int, max_new: int, nq: int, nkv: int, hd: int, page: int,
                            window: Optional[int], scale: float, variant: int = 0) -> None:
     """Flash attention on the matrix cores for steps with several tokens per sequence.
-    `variant` 1 reads operand fragments straight from the cache, 2 stages pages in LDS
-    (for long prompts), 0 chooses by the step's longest sequence."""
+    `variant` 1 reads operand fragments straight from the cache, 2 and 3 stage pages in LDS
+    through registers (workgroups of 8 and of 4 waves), 4 brings them into an LDS ring by
+    direct loads (head sizes 64 and 128), 0 chooses by the step's longest sequence and the
+    head size."""
     _dev("attention_prefill_bf16", out, cu_seqlens, slots, ctx_lens, block_table, cache)
     _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
          "attention_prefill_bf16: bfloat16 only")
     _req(hd % 16 == 0 and hd <= 256, f"attention_prefill_bf16: head_dim {hd} must be a multiple of 16, at most 256")
     _req(page == 64, "attention_prefill_bf16: pages of 64 tokens")
+    _req(scale > 0, f"attention_prefill_bf16: the score scale must be positive, not {scale} (the kernels take the row maximum before scaling)")
     _req(cache.shape[1:] == (2, nkv, page, hd), "attention_prefill_bf16: cache unit must be [pages, 2, nkv, page, hd]")
     _req(out.shape[1] == nq * hd and nq % nkv == 0, "attention_prefill_bf16: out must be [T, nq * hd]")
     f = _fn("attention_bf16", "br_attn_prefill_bf16",

@@ -51,6 +51,8 @@ class GQAAttention(Mixer):
         self.window = None if window is None else int(window)
         self.position = position
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        if not self.scale > 0:
+            raise ConfigError(f"attention: the score scale must be positive, not {self.scale}")
         self.w_qkv = self.w_o = None
         self.force_simple = False          # tests set it to run the one-wave-per-query kernel in bf16
 
