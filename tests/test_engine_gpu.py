@@ -461,3 +461,34 @@ def test_serving_sizes_random_schedule(serving, dtype, layout, monkeypatch):
     for i in range(0, len(seqs), 3):                     # every third request against the plain implementation
         close(np.concatenate(got[i]), P.forward(cfg, w, seqs[i]), dtype, f"request {i} of {len(seqs[i])} tokens")
     assert [g.pool.free_count for g in eng.cache.groups] == free_before
+
+
+def test_wide_matrices_take_the_blocked_layout_by_themselves(tmp_path):
+    """Matrices of 8,192 rows and more (here gate/up and the head) are laid out in blocks at load
+    without being asked; the others keep their rows.  Whole, the last tokens one by one, and a batch."""
+    cfg_d = dict(SERVING, num_hidden_layers=1, intermediate_size=4096, vocab_size=8200, layer_types=["full_attention"])
+    folder = str(tmp_path / "wide")
+    B.Engine.write_random_folder(folder, B.MistralConfig.from_dict(cfg_d), seed=4, std=0.03, vector_jitter=0.3)
+    cfg, w = P.read_folder(folder)
+    eng = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=8192)
+    layer = eng.model.layers[0]
+    assert layer.feed_forward.w_gu.dim() == 4 and eng.model.lm_head.weight.dim() == 4
+    assert layer.feed_forward.w_d.dim() == 2 and layer.mixer.w_qkv.dim() == 2 and layer.mixer.w_o.dim() == 2
+    toks = tokens(cfg, 150, 3)
+    ref = P.forward(cfg, w, toks)
+    close(whole(eng, toks), ref, "bfloat16", "wide matrices, whole")
+    s = eng.alloc_slot()
+    parts = [eng.step([StepEntry(s, toks[:140], list(range(140)))]).cpu().numpy()]
+    for t in toks[140:]:
+        parts.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    eng.free_slot(s)
+    close(np.concatenate(parts), ref, "bfloat16", "wide matrices, last 10 one by one")
+    seqs = [tokens(cfg, 20 + 3 * i, 80 + i) for i in range(24)]               # 24 rows: the wide streaming product
+    slots = [eng.alloc_slot() for _ in seqs]
+    out = eng.step([StepEntry(sl, q[:-1], [len(q) - 2]) for sl, q in zip(slots, seqs)]).cpu().numpy()
+    out2 = eng.step([StepEntry(sl, [q[-1]], [0]) for sl, q in zip(slots, seqs)]).cpu().numpy()
+    for sl in slots:
+        eng.free_slot(sl)
+    for i in (0, 11, 23):
+        r = P.forward(cfg, w, seqs[i])
+        close(np.stack([out[i], out2[i]]), r[-2:], "bfloat16", f"wide matrices, request {i} of 24")
