@@ -492,3 +492,45 @@ def test_wide_matrices_take_the_blocked_layout_by_themselves(tmp_path):
     for i in (0, 11, 23):
         r = P.forward(cfg, w, seqs[i])
         close(np.stack([out[i], out2[i]]), r[-2:], "bfloat16", f"wide matrices, request {i} of 24")
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Sizes drawn at random (head sizes in steps of 16, groups of 1 to 6 heads, widths and vocabularies
+    that are no powers of two, windows, tied heads, 1 to 3 layers): a prompt whole, its last 8 tokens
+    one by one, and 20 requests of unequal lengths in one step and one token each, in both precisions."""
+    rng = np.random.default_rng(1000 + seed)
+    hd = int(rng.choice([16, 32, 48, 64, 80, 96, 128]))
+    nkv = int(rng.choice([1, 2, 3, 4]))
+    nq = nkv * int(rng.choice([1, 2, 3, 4, 6]))
+    window = None if rng.random() < 0.4 else int(rng.choice([4, 17, 64, 100]))
+    L = int(rng.integers(1, 4))
+    cfg_d = dict(num_hidden_layers=L, hidden_size=int(rng.choice([64, 96, 200, 264, 520, 1024, 1152])),
+                 num_attention_heads=nq, num_key_value_heads=nkv, head_dim=hd,
+                 intermediate_size=int(rng.choice([96, 192, 328, 520, 1024, 1536, 2048])),
+                 vocab_size=int(rng.choice([100, 257, 1000, 4100, 9000])), rope_theta=float(rng.choice([1e4, 1e6])),
+                 rms_norm_eps=float(rng.choice([1e-5, 1e-6])), sliding_window=window, max_position_embeddings=4096,
+                 tie_word_embeddings=bool(rng.random() < 0.3),
+                 layer_types=[str(rng.choice(["full_attention", "sliding_attention"])) if window else "full_attention"
+                              for _ in range(L)])
+    folder = str(tmp_path / "drawn")
+    B.Engine.write_random_folder(folder, B.MistralConfig.from_dict(cfg_d), seed=seed, std=0.03, vector_jitter=0.3)
+    cfg, w = P.read_folder(folder)
+    n = int(rng.choice([30, 90, 150, 300]))
+    toks = tokens(cfg, n, seed)
+    ref = P.forward(cfg, w, toks)
+    for dtype in ("float32", "bfloat16"):
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=2048)
+        s = eng.alloc_slot()
+        parts = [eng.step([StepEntry(s, toks[:n - 8], list(range(n - 8)))]).cpu().numpy()]
+        for t in toks[n - 8:]:
+            parts.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+        eng.free_slot(s)
+        close(np.concatenate(parts), ref, dtype, f"{cfg_d}: whole, then 8 one by one")
+        slots = [eng.alloc_slot() for _ in range(20)]
+        first = eng.step([StepEntry(sl, toks[:10 + i], [9 + i]) for i, sl in enumerate(slots)]).cpu().numpy()
+        then = eng.step([StepEntry(sl, [toks[10 + i]], [0]) for i, sl in enumerate(slots)]).cpu().numpy()
+        for sl in slots:
+            eng.free_slot(sl)
+        close(first, ref[9:29], dtype, f"{cfg_d}: 20 prompts of 10 to 29 tokens in one step")
+        close(then, ref[10:30], dtype, f"{cfg_d}: one token each after them")
