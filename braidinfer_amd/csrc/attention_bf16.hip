@@ -490,11 +490,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             f32x16 s_acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int s = 0; s < 2 * NB; ++s) {
                 const bf16x8 kf = *(const bf16x8*)(kp + (((2 * s + g) ^ kswz_) * 16));
                 s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
             }
+            __builtin_amdgcn_s_setprio(0);
             float sv[16];
             float mx = -INFINITY;
             const bool whole = row0 + 31 < rows_total && kb + 31 <= pq_min_w &&
@@ -533,6 +535,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             lsum += psum;
             m = m_new;
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int i2 = 0; i2 < NB; ++i2) {
                 const int vrow = i2 * 32 + c;
@@ -550,6 +553,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 acc_o[i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i2], 0, 0, 0);
                 acc_o[i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i2], 0, 0, 0);
             }
+            __builtin_amdgcn_s_setprio(0);
         }
     }
 #undef PF_ISSUE
