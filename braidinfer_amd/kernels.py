@@ -383,8 +383,7 @@ def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu
     """Flash attention on the matrix cores for steps with several tokens per sequence.
     `variant` 1 reads operand fragments straight from the cache, 2 and 3 stage pages in LDS
     through registers (workgroups of 8 and of 4 waves), 4 brings them into an LDS ring by
-    direct loads (head sizes 64 and 128), 0 chooses by the step's longest sequence and the
-    head size."""
+    direct loads (head sizes 64 and 128), 0 chooses by the head size."""
     _dev("attention_prefill_bf16", out, cu_seqlens, slots, ctx_lens, block_table, cache)
     _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
          "attention_prefill_bf16: bfloat16 only")
