@@ -476,16 +476,23 @@ static int launch_tile_dma(const bf16* A, const bf16* W, void* C, int M, int N, 
     return br_check_launch();
 }
 
-// Which direct-to-LDS tile (5: 128x256, one workgroup per CU; 6: 128x128, two) and how many
-// runs of k-tiles for a product of more than 64 rows: the least time by a rough count in
-// microseconds (rounds of workgroups over the chip times k-tiles times 1.0-1.3 us a k-tile,
-// plus, when split, a launch and the traffic of the partial sums), runs of at least 4
-// k-tiles that fit the scratch memory.
+// Which direct-to-LDS tile (5: 128x256, one workgroup per CU; 6: 128x128, two; 10: 256x192, one, two
+// stages, not split) and how many runs of k-tiles for a product of more than 64 rows: the least time by
+// a rough count in microseconds (rounds of workgroups over the chip times k-tiles times 1.0-1.7 us a
+// k-tile, plus, when split, a launch and the traffic of the partial sums), runs of at least 4 k-tiles
+// that fit the scratch memory.  The 256x192 tile is there for shapes that it covers in fewer rounds:
+// 2,048 x 6,144 is 256 of them, one round, against 384 tiles of 128x256 (measured 103-118 against
+// 129-134 us); with equal rounds it loses (two stages, 1.5 times the work a k-tile for 1.5 times the time).
 static void choose_tile(int M, int N, int K, int cus, size_t scratch_bytes, int* kernel, int* parts) {
     const int nk = K / DMA_BK;
     double best = 1e30;
     *kernel = 5;
     *parts = 1;
+    {
+        const long long tiles = (long long)((M + 255) / 256) * ((N + 191) / 192);
+        const double t = (double)((tiles + cus - 1) / cus) * nk * 1.72;
+        if (tiles > cus / 2) { best = t; *kernel = 10; }             // with fewer tiles a split product fills the chip better
+    }
     for (int k = 5; k <= 6; ++k) {
         const long long tiles = (long long)((M + 127) / 128) * ((N + (k == 5 ? 255 : 127)) / (k == 5 ? 256 : 128));
         const long long slots = (long long)cus * (k == 5 ? 1 : 2);
@@ -1408,7 +1415,7 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
 // rows), 8 = stream wide (16 < M <= 64, K a multiple of 128), 9 = direct-to-LDS tile 64x128
-// (M <= 64); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out of registers in
+// (M <= 64), 10 = direct-to-LDS tile 256x192; tests force one.  (A 256x256 tile of 8 waves was tried: it runs out of registers in
 // three of the four epilogues and was no faster in the fourth.)
 // `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 9).
 // `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
@@ -1432,7 +1439,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
     const bool wide_ok = aligned && M > 16 && M <= 64 && K % 128 == 0 && K >= 256 &&
                          (!scratch || (uintptr_t)scratch % 16 == 0);
-    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 9 || kernel < 0 ||
+    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 10 || kernel < 0 || (kernel == 10 && !dma_ok) ||
         (kernel == 9 && (!dma_ok || M > 64)))
         return BR_BAD_ARG;
     if (wl != WL_ROWS) {
@@ -1459,6 +1466,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
         const int cus = br_device_cus();
         if (cus > 0) choose_tile(M, N, K, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
     }
+    if (kernel == 10) return launch_tile_dma<256, 192, 4, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
     if (forced_parts > 1 && (kernel == 5 || kernel == 6)) {
         if (!scratch || (uintptr_t)scratch % 16 || (size_t)forced_parts * M * N * sizeof(float) > scratch_bytes ||
             forced_parts > K / DMA_BK)
