@@ -483,7 +483,7 @@ static int launch_tile_dma(const bf16* A, const bf16* W, void* C, int M, int N, 
 // that fit the scratch memory.  The 256x192 tile is there for shapes that it covers in fewer rounds:
 // 2,048 x 6,144 is 256 of them, one round, against 384 tiles of 128x256 (measured 103-118 against
 // 129-134 us); with equal rounds it loses (two stages, 1.5 times the work a k-tile for 1.5 times the time).
-static void choose_tile(int M, int N, int K, int cus, size_t scratch_bytes, int* kernel, int* parts) {
+static void choose_tile(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* kernel, int* parts) {
     const int nk = K / DMA_BK;
     double best = 1e30;
     *kernel = 5;
@@ -492,6 +492,13 @@ static void choose_tile(int M, int N, int K, int cus, size_t scratch_bytes, int*
         const long long tiles = (long long)((M + 255) / 256) * ((N + 191) / 192);
         const double t = (double)((tiles + cus - 1) / cus) * nk * 1.72;
         if (tiles > cus / 2) { best = t; *kernel = 10; }             // with fewer tiles a split product fills the chip better
+    }
+    if (mode == OUT_SWIGLU) {
+        // 256x256, SwiGLU epilogue only (the other epilogues run out of registers around its 128 accumulators a
+        // wave): 8 % faster than 128x256 where its rounds fit (4,096 x 28,672: 920 against 1,000 us)
+        const long long tiles = (long long)((M + 255) / 256) * ((N + 255) / 256);
+        const double t = (double)((tiles + cus - 1) / cus) * nk * 2.1;
+        if (tiles > cus / 2 && t < best - 1e-9) { best = t; *kernel = 11; }
     }
     for (int k = 5; k <= 6; ++k) {
         const long long tiles = (long long)((M + 127) / 128) * ((N + (k == 5 ? 255 : 127)) / (k == 5 ? 256 : 128));
@@ -1415,7 +1422,7 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
 // rows), 8 = stream wide (16 < M <= 64, K a multiple of 128), 9 = direct-to-LDS tile 64x128
-// (M <= 64), 10 = direct-to-LDS tile 256x192; tests force one.  (A 256x256 tile of 8 waves was tried: it runs out of registers in
+// (M <= 64), 10 = direct-to-LDS tile 256x192, 11 = the same 256x256 (SwiGLU epilogue only); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out of registers in
 // three of the four epilogues and was no faster in the fourth.)
 // `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 9).
 // `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
@@ -1439,7 +1446,8 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
     const bool wide_ok = aligned && M > 16 && M <= 64 && K % 128 == 0 && K >= 256 &&
                          (!scratch || (uintptr_t)scratch % 16 == 0);
-    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 10 || kernel < 0 || (kernel == 10 && !dma_ok) ||
+    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 11 || kernel < 0 || (kernel >= 10 && !dma_ok) ||
+        (kernel == 11 && mode != OUT_SWIGLU) ||
         (kernel == 9 && (!dma_ok || M > 64)))
         return BR_BAD_ARG;
     if (wl != WL_ROWS) {
@@ -1464,9 +1472,14 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     int parts = 1;
     if (chosen && (kernel == 5 || kernel == 6)) {
         const int cus = br_device_cus();
-        if (cus > 0) choose_tile(M, N, K, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
+        if (cus > 0) choose_tile(M, N, K, mode, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
     }
     if (kernel == 10) return launch_tile_dma<256, 192, 4, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
+    if (kernel == 11) {
+        gemm_tile_dma_kernel<256, 256, 2, 4, 2, OUT_SWIGLU><<<(unsigned)(((M + 255) / 256) * ((N + 255) / 256)), 512, 0, s>>>(
+            A, W, C, M, N, K, lda, ldc, (M + 255) / 256, (N + 255) / 256, K / DMA_BK, 0, wl);
+        return br_check_launch();
+    }
     if (forced_parts > 1 && (kernel == 5 || kernel == 6)) {
         if (!scratch || (uintptr_t)scratch % 16 || (size_t)forced_parts * M * N * sizeof(float) > scratch_bytes ||
             forced_parts > K / DMA_BK)
@@ -1505,7 +1518,7 @@ extern "C" int br_gemm_bf16(const void* A, const void* W, void* C, int M, int N,
 extern "C" int br_gemm_bf16_tile_choice(int M, int N, int K, size_t scratch_bytes, int* kernel, int* parts) {
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
-    choose_tile(M, N, K, cus, scratch_bytes, kernel, parts);
+    choose_tile(M, N, K, OUT_BF16, cus, scratch_bytes, kernel, parts);
     return BR_OK;
 }
 

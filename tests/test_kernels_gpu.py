@@ -75,7 +75,7 @@ SHAPES = [(1, 64, 64), (5, 100, 96), (17, 192, 320), (64, 301, 100), (33, 1000, 
 def _skip_unless_kernel_takes(kernel, M, Kd):
     if kernel == 3 and (Kd % 8 or M > 64):
         pytest.skip("the skinny kernels take M <= 64 and K in steps of 8")
-    if (4 <= kernel <= 6 or kernel == 10) and Kd % 64:
+    if (4 <= kernel <= 6 or kernel in (10, 11)) and Kd % 64:
         pytest.skip("the direct-to-LDS tile kernels take K in steps of 64")
     if kernel == 7 and (M > 16 or Kd % 128 or Kd < 1024):
         pytest.skip("the streaming kernel takes M <= 16 and K in steps of 128 from 1024")
@@ -659,7 +659,7 @@ def test_attention_kernels_refuse_what_they_do_not_take():
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11])
 @pytest.mark.parametrize("M,I,Kd", [(40, 8264, 256), (64, 328, 1152), (1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
                                     (300, 512, 1024), (129, 200, 192), (1, 2056, 1024), (8, 328, 1152), (13, 4400, 1280),
                                     (100, 264, 4096), (260, 520, 2048)])
