@@ -1474,6 +1474,31 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
         const int cus = br_device_cus();
         if (cus > 0) choose_tile(M, N, K, mode, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
     }
+    if (chosen && mode == OUT_SWIGLU && kernel == 5 && parts == 1) {
+        // The 256x256 tile over as many weight rows as make whole rounds of it, the 128x256 tile over the rest,
+        // where the count says that this is faster than 128x256 over all of them (2,048 x 28,672: three
+        // rounds of 256x256 over 24,576 rows and one round of 128x256 over 4,096, instead of seven of 128x256).
+        const int cus = br_device_cus();
+        const int tm11 = (M + 255) / 256, nk = K / DMA_BK;
+        const int cols = cus > 0 ? cus / tm11 : 0;                   // tile columns of one round
+        if (cols > 0) {
+            const long long n_round = (long long)cols * 256;
+            const long long r11 = N / n_round, n1 = r11 * n_round, n2 = N - n1;
+            const long long t5_all = ((long long)((M + 127) / 128) * ((N + 255) / 256) + cus - 1) / cus;
+            const long long t5_rest = ((long long)((M + 127) / 128) * ((n2 + 255) / 256) + cus - 1) / cus;
+            const double whole = (double)t5_all * nk * 1.14;
+            const double split = (double)r11 * nk * 2.05 + (double)t5_rest * nk * 1.14 + 5.0;
+            if (r11 >= 1 && n2 > 0 && n2 % 16 == 0 && split < 0.97 * whole) {
+                gemm_tile_dma_kernel<256, 256, 2, 4, 2, OUT_SWIGLU><<<(unsigned)(tm11 * (int)(n1 / 256)), 512, 0, s>>>(
+                    A, W, C, M, (int)n1, K, lda, ldc, tm11, (int)(n1 / 256), nk, 0, wl);
+                int rc = br_check_launch();
+                if (rc != BR_OK) return rc;
+                // n1 rows on: the same number of elements in either weight layout (n1 is a multiple of 16)
+                return launch_tile_dma<128, 256, 2, 4, 3>(A, W + (size_t)n1 * K, (bf16*)C + n1 / 2, M, (int)n2, K, lda, ldc,
+                                                          mode, s, 1, nullptr, wl);
+            }
+        }
+    }
     if (kernel == 10) return launch_tile_dma<256, 192, 4, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
     if (kernel == 11) {
         gemm_tile_dma_kernel<256, 256, 2, 4, 2, OUT_SWIGLU><<<(unsigned)(((M + 255) / 256) * ((N + 255) / 256)), 512, 0, s>>>(

@@ -677,3 +677,24 @@ def test_gemm_with_swiglu_epilogue(M, I, Kd, kernel):
         out2 = torch.empty_like(out)
         K.gemm_swiglu(a, K.interleave_gate_up(wg, wu), out2, scratch=torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV))
         assert (out2.double() - want).abs().max() < 1e-2 * want.abs().max()
+
+
+@pytest.mark.parametrize("blocked", [False, True])
+def test_gemm_swiglu_over_two_tile_shapes(blocked):
+    # 2,048 x 28,672: the chooser covers 24,576 weight rows with 256x256 tiles (whole rounds of them) and the
+    # other 4,096 with 128x256 tiles, in two launches; every tile kernel sums k in the same order, so the
+    # result equals that of one tile shape bit for bit
+    M, I, Kd = 2048, 14336, 1024
+    a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
+    wg, wu = rnd(I, Kd, seed=2, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=3, scale=0.3, dtype=torch.bfloat16)
+    w = K.interleave_gate_up(wg, wu)
+    if blocked:
+        w = K.block_weight(w)
+    out = torch.full((M, I), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K.gemm_swiglu(a, w, out)
+    one = torch.empty_like(out)
+    K.gemm_swiglu(a, w, one, kernel=5)
+    assert torch.equal(out, one)
+    g, u = a.float() @ wg.float().T, a.float() @ wu.float().T
+    want = g / (1 + torch.exp(-g)) * u
+    assert (out.float() - want).abs().max() < 1e-2 * want.abs().max()
