@@ -35,6 +35,7 @@ MODULES: Dict[str, List[str]] = {
     "sampling": ["sampling.hip"],
     "gemm_bf16": ["gemm_bf16.hip"],
     "attention_bf16": ["attention_bf16.hip"],
+    "random_weights": ["random_weights.hip"],
 }
 HEADERS = ["common.h"]
 
@@ -163,7 +164,7 @@ def compile_module(name: str, force: bool = False) -> str:
 
 
 def build_all(force: bool = True, names: Optional[Iterable[str]] = None, jobs: int = 4) -> List[str]:
-    """Compile every module (the round's build check calls this with force=True)."""
+    """Compile every module, by default also those already built for the current sources."""
     names = [n for n in (names or MODULES) if all(os.path.isfile(os.path.join(HERE, f)) for f in MODULES[n])]
     results: Dict[str, str] = {}
     errors: List[str] = []

@@ -20,6 +20,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 #define BR_OK 0
 #define BR_BAD_ARG 1
 #define BR_LAUNCH_FAILED 2
+#define BR_TOO_LARGE 3
 
 static inline int br_check_launch() {
     hipError_t e = hipGetLastError();

@@ -19,7 +19,7 @@ from ..cache import SequenceCache
 from ..config import config_from_folder, spec_of
 from ..errors import BraidError, CacheError, ConfigError, KernelError, StepError
 from ..parts import Runtime
-from ..weights import load_tensors, random_tensors, write_model_folder
+from ..weights import FolderTensors, RandomTensors, write_model_folder
 from .model import DecoderModel
 from .step import StepBatch, Workspace, pack_step
 
@@ -59,56 +59,66 @@ class Engine:
         self.device = rt.device
         self.ws = Workspace(rt.device)
         if max_seq_len is None:
-            # the block tables are [slots, pages of the longest sequence]: bound the longest
-            # sequence by the model's positions (at least 32k) rather than by the whole cache
-            max_seq_len = min(max(int(max_tokens), 64), max(int(model.spec.max_position_embeddings), 32768))
+            # the block tables are [slots, pages of the longest sequence]: the longest sequence is
+            # what the cache holds, but no longer than the positions the model was made for
+            # (a caller who wants more says so with max_seq_len)
+            max_seq_len = min(max(int(max_tokens), 64), int(model.spec.max_position_embeddings))
         self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens=max_tokens,
                                    max_seq_len=max_seq_len, n_slots=n_slots, dtype=rt.dtype, device=rt.device)
         self.vocab_size = self.spec.vocab_size
         # single-token steps are replayed from HIP graphs when every part allows it
         self.use_graphs = bool(use_graphs) and model.graph_safe()
         self._graphs = None
+        self.load_profile = None
 
     # ---- construction ------------------------------------------------------------------
+    @classmethod
+    def _from_source(cls, config, make_source, dtype, device, max_tokens, max_seq_len, n_slots, use_graphs) -> "Engine":
+        """Build the model of `config`, size one arena for what its parts keep, and let the
+        parts pull their tensors from the source `make_source(specs, allowed, device, dtype)` makes."""
+        from ..weights import WeightArena
+        device = torch.device(device)
+        _require_gpu(device)
+        model = DecoderModel(spec_of(config))
+        rt = Runtime(device=device, dtype=parse_dtype(dtype))
+        source = make_source(model.weight_specs(), model.optional_names(), device, rt.dtype)
+        rt.arena = WeightArena(device, source.resident_bytes())
+        model.load(source, rt)
+        profile = source.finish(rt.arena)
+        eng = cls(config, model, rt, max_tokens, max_seq_len, n_slots, use_graphs)
+        eng.load_profile = profile
+        return eng
+
     @classmethod
     def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
                     max_seq_len: Optional[int] = None, n_slots: Optional[int] = None,
                     use_graphs: bool = True) -> "Engine":
-        device = torch.device(device)
-        _require_gpu(device)
+        """A model folder (config.json and model.safetensors, or shards with their index).
+        `engine.load_profile.line()` says how the load went (the reference prints a
+        `LOAD PROFILE` line, bin/generate.rs:62-68)."""
         config = config_from_folder(folder)
-        model = DecoderModel(spec_of(config))
-        rt = Runtime(device=device, dtype=parse_dtype(dtype))
-        tensors = load_tensors(folder, model.weight_specs(), device, rt.dtype,
-                               allow_unexpected=model.optional_names())
-        model.load(tensors, rt)
-        return cls(config, model, rt, max_tokens, max_seq_len, n_slots, use_graphs)
+        return cls._from_source(config, lambda specs, allowed, dev, dt: FolderTensors(folder, specs, dev, dt, allowed),
+                                dtype, device, max_tokens, max_seq_len, n_slots, use_graphs)
 
     @classmethod
     def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
                max_seq_len: Optional[int] = None, n_slots: Optional[int] = None, std: float = 0.02,
-               use_graphs: bool = True) -> "Engine":
-        """Seeded random weights made on the device (no folder): bf16 N(0, std) matrices,
-        norm weights 1, as the random-weights folder mode makes them."""
-        device = torch.device(device)
-        _require_gpu(device)
-        model = DecoderModel(spec_of(config))
-        rt = Runtime(device=device, dtype=parse_dtype(dtype))
-        tensors = {}
-        specs = model.weight_specs()
-        kinds = {sp.name: sp.kind for sp in specs}
-        for name, t in random_tensors(specs, seed, device, torch.bfloat16, std):
-            widen = kinds[name] == "vector" or rt.dtype == torch.float32
-            tensors[name] = t.to(torch.float32) if (widen and kinds[name] != "int") else t
-        model.load(tensors, rt)
-        return cls(config, model, rt, max_tokens, max_seq_len, n_slots, use_graphs)
+               use_graphs: bool = True, vector_jitter: float = 0.0) -> "Engine":
+        """Seeded random weights made on the device (no folder): the same bits a
+        random-weights folder of that configuration, seed and std holds (bfloat16 N(0, std)
+        matrices, norm weights 1), widened for the 32-bit path."""
+        return cls._from_source(config, lambda specs, allowed, dev, dt: RandomTensors(specs, seed, dev, dt, std, vector_jitter),
+                                dtype, device, max_tokens, max_seq_len, n_slots, use_graphs)
 
     @staticmethod
     def write_random_folder(folder: str, config, seed: int = 0, std: float = 0.02,
-                            vector_jitter: float = 0.0) -> str:
-        """Random-weights mode: a model folder (config.json, model.safetensors)."""
+                            vector_jitter: float = 0.0, device="cpu", shard_bytes: Optional[int] = None) -> str:
+        """Random-weights mode: a model folder (config.json, model.safetensors; with
+        `shard_bytes` several files and their index).  `device` is where the values are
+        made: the bits are the same everywhere, a GPU is faster for large shapes."""
         model = DecoderModel(spec_of(config))
-        return write_model_folder(folder, config, model.weight_specs(), seed, std, vector_jitter)
+        return write_model_folder(folder, config, model.weight_specs(), seed, std, vector_jitter, device=device,
+                                  shard_bytes=shard_bytes)
 
     # ---- slots -----------------------------------------------------------------------
     def alloc_slot(self) -> int:

@@ -54,7 +54,7 @@ def _check(rc: int, name: str) -> None:
     if rc == 0:
         return
     raise KernelError(f"{name}: " + {1: "arguments outside what the kernel takes",
-                                     2: "launch failed"}.get(rc, f"error {rc}"))
+                                     2: "launch failed", 3: "sizes beyond the entry point's fixed scratch"}.get(rc, f"error {rc}"))
 
 
 _sigs_done = set()
@@ -164,6 +164,26 @@ def convert(a: torch.Tensor, out: torch.Tensor) -> None:
     _check(f(_ptr(a), _ptr(out), to_bf16, a.numel(), _stream()), "convert")
 
 
+# -------------------------------------------------------------- random weights -----
+def _random_fill(fn_name: str, out: torch.Tensor, key: int, param: float, first: int) -> None:
+    _dev(fn_name, out)
+    f = _fn("random_weights", "br_" + fn_name, [_P, c_int, c_size_t, c_size_t, ctypes.c_uint64, c_float, _P])
+    _check(f(_ptr(out), _is_bf16(out, fn_name), out.numel(), int(first), int(key) & ((1 << 64) - 1), param, _stream()),
+           fn_name)
+
+
+def random_normal(out: torch.Tensor, key: int, std: float, first: int = 0) -> None:
+    """out (flat order) = elements first.. of the normal tensor with this key (see
+    weights/random_weights.py for the generator); the scale is float32(std) * 2^-16."""
+    import numpy as np
+    _random_fill("random_normal", out, key, float(np.float32(std) * np.float32(2.0 ** -16)), first)
+
+
+def random_ones(out: torch.Tensor, key: int, jitter: float, first: int = 0) -> None:
+    """out = 1 + (2u - 1) * jitter with u the generator's uniform number of each element."""
+    _random_fill("random_ones", out, key, float(jitter), first)
+
+
 # ------------------------------------------------------------------------ GEMM ------
 GEMM_SCRATCH_FLOATS = 16 * 1024 * 1024   # 64 MB: room for the partial sums of the products that the bf16 kernels split along k
 
@@ -179,21 +199,28 @@ def weight_block_rows() -> int:
     return int(_fn("gemm_bf16", "br_gemm_bf16_block_rows", [])())
 
 
-def block_weight(w: torch.Tensor) -> torch.Tensor:
+def block_weight(w: torch.Tensor, alloc=None) -> torch.Tensor:
     """The matrix [N, K] as blocks [ceil(N / R), K / 128, R, 128], R = `weight_block_rows()` = 16:
     R rows by 128 k are contiguous and a strip of R rows is one run along k; rows are padded
     with zeros to a multiple of R.  The products that stream a weight matrix once per step
     read it faster in this order than 256 bytes from every row.  `gemm`, `gemm_swiglu`,
     `gemm_norm_prepare` and `gemm_norm_scaled` take either form and tell them apart by the
-    number of dimensions; N is then the output's width."""
+    number of dimensions; N is then the output's width.  `alloc(shape, dtype)` gives the
+    memory of the result (default: a new tensor)."""
     if not weight_blockable(w):
         raise KernelError(f"block_weight: {tuple(w.shape)} {w.dtype} on {w.device} is not taken")
     N, K = w.shape
     R = weight_block_rows()
     nb = -(-N // R)
-    if nb * R != N:
-        w = torch.cat([w, torch.zeros(nb * R - N, K, dtype=w.dtype, device=w.device)], dim=0)
-    return w.view(nb, R, K // 128, 128).permute(0, 2, 1, 3).contiguous()
+    shape = (nb, K // 128, R, 128)
+    out = alloc(shape, w.dtype) if alloc is not None else torch.empty(shape, dtype=w.dtype, device=w.device)
+    full = N // R
+    if full:
+        out[:full].copy_(w[:full * R].view(full, R, K // 128, 128).permute(0, 2, 1, 3))
+    if full != nb:
+        out[full].zero_()
+        out[full, :, :N - full * R].copy_(w[full * R:].view(N - full * R, K // 128, 128).permute(1, 0, 2))
+    return out
 
 
 def unblock_weight(wb: torch.Tensor, N: int) -> torch.Tensor:
@@ -351,12 +378,17 @@ def gemm_norm_scaled(xg: torch.Tensor, ssq: torch.Tensor, tiles: int, eps: float
              wl, _stream()), "gemm_norm_scaled")
 
 
-def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:
-    """[2 I, K]: blocks of 8 gate rows followed by the 8 up rows of the same outputs."""
+def interleave_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor, alloc=None) -> torch.Tensor:
+    """[2 I, K]: blocks of 8 gate rows followed by the 8 up rows of the same outputs.
+    `alloc(shape, dtype)` gives the memory of the result (default: a new tensor)."""
     I, K = w_gate.shape
     if I % 8:
         raise KernelError(f"interleave_gate_up: intermediate size {I} is not a multiple of 8")
-    return torch.stack([w_gate.view(I // 8, 8, K), w_up.view(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
+    out = alloc((2 * I, K), w_gate.dtype) if alloc is not None else torch.empty((2 * I, K), dtype=w_gate.dtype, device=w_gate.device)
+    o = out.view(I // 8, 2, 8, K)
+    o[:, 0].copy_(w_gate.view(I // 8, 8, K))
+    o[:, 1].copy_(w_up.view(I // 8, 8, K))
+    return out
 
 
 # ------------------------------------------------------------------- attention -----

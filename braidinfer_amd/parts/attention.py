@@ -21,7 +21,7 @@ from ..cache import CacheNeed
 from ..errors import ConfigError
 from ..weights import TensorSpec
 from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
-from .linear import fuse_rows, linear, stream_layout
+from .linear import fused_layout, linear, stream_layout
 
 
 def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
@@ -66,8 +66,8 @@ class GQAAttention(Mixer):
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.w_qkv = stream_layout(fuse_rows([tensors[prefix + n + "_proj.weight"] for n in ("q", "k", "v")]), rt)
-        self.w_o = stream_layout(tensors[prefix + "o_proj.weight"].contiguous(), rt)
+        self.w_qkv = fused_layout([tensors[prefix + n + "_proj.weight"] for n in ("q", "k", "v")], rt)
+        self.w_o = stream_layout(tensors[prefix + "o_proj.weight"], rt)
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv_heads=self.nkv, head_dim=self.hd, window=self.window)

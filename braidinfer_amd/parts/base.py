@@ -29,14 +29,36 @@ from ..weights import TensorSpec
 
 @dataclass
 class Runtime:
-    """Where and in which precision a model runs."""
+    """Where and in which precision a model runs, and where its parts keep their weights.
+
+    `arena`: when set (anything with `empty(shape, dtype)` and `holds(tensor)`, e.g.
+    `weights.WeightArena`), `empty` and `own` place what a part keeps inside it, so a
+    loaded model is one device allocation.  `published`: tensors a part offers to parts
+    loaded after it, by tensor name (a tied output head finds the embedding table there)."""
 
     device: torch.device
     dtype: torch.dtype            # torch.float32 (true 32-bit path) or torch.bfloat16
+    arena: Any = None
+    published: Dict[str, torch.Tensor] = field(default_factory=dict)
 
     @property
     def is_bf16(self) -> bool:
         return self.dtype == torch.bfloat16
+
+    def empty(self, shape, dtype: torch.dtype) -> torch.Tensor:
+        """Uninitialised memory for a tensor the part keeps."""
+        if self.arena is not None:
+            return self.arena.empty(shape, dtype)
+        return torch.empty(tuple(shape), dtype=dtype, device=self.device)
+
+    def own(self, t: torch.Tensor) -> torch.Tensor:
+        """`t` as the part keeps it: dense, on the device, inside the arena when there is one
+        (a copy unless it already is all that)."""
+        if t.device == self.device and t.is_contiguous() and (self.arena is None or self.arena.holds(t)):
+            return t
+        out = self.empty(t.shape, t.dtype)
+        out.copy_(t)
+        return out
 
 
 class Part:

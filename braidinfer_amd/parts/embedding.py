@@ -29,7 +29,8 @@ class TokenEmbedding(Embedding):
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = tensors[prefix + "weight"].contiguous()
+        self.weight = rt.own(tensors[prefix + "weight"])
+        rt.published[prefix + "weight"] = self.weight      # a tied output head reads the same table
 
     def forward(self, tokens, out) -> None:
         K.embedding(self.weight, tokens, out)
@@ -51,12 +52,18 @@ class LMHead(OutputHead):
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        name = self.tied_to or prefix + "weight"
+        if self.tied_to:                           # a tied table is also read row by row by the embedding
+            if self.tied_to in rt.published:
+                self.weight = rt.published[self.tied_to]
+            elif self.tied_to in tensors:
+                self.weight = rt.own(tensors[self.tied_to])
+            else:
+                raise WeightError(f"output head: tensor {self.tied_to} is missing", missing=[self.tied_to])
+            return
+        name = prefix + "weight"
         if name not in tensors:
             raise WeightError(f"output head: tensor {name} is missing", missing=[name])
-        self.weight = tensors[name].contiguous()
-        if not self.tied_to:                       # a tied table is also read row by row by the embedding
-            self.weight = stream_layout(self.weight, rt)
+        self.weight = stream_layout(tensors[name], rt)
 
     def forward(self, h, out, ws=None) -> None:
         linear(h, self.weight, out, ws)

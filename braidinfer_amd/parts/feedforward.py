@@ -10,7 +10,7 @@ import torch
 from .. import kernels as K
 from ..weights import TensorSpec
 from .base import FeedForward, NormedInput, Runtime, register_part
-from .linear import fuse_rows, linear, stream_layout
+from .linear import fused_layout, linear, stream_layout
 
 
 class SwiGLU(FeedForward):
@@ -34,8 +34,8 @@ class SwiGLU(FeedForward):
         # bf16: gate and up rows interleaved so that the product's epilogue applies silu * up
         # and the [T, 2 I] intermediate is never written
         self.fused = g.dtype == u.dtype == torch.bfloat16 and rt.is_bf16 and self.I % 8 == 0
-        self.w_gu = stream_layout(K.interleave_gate_up(g, u) if self.fused else fuse_rows([g, u]), rt)
-        self.w_d = stream_layout(tensors[prefix + "down_proj.weight"].contiguous(), rt)
+        self.w_gu = fused_layout([g, u], rt, interleave=self.fused)
+        self.w_d = stream_layout(tensors[prefix + "down_proj.weight"], rt)
 
     def forward(self, h, x, step) -> None:
         T = step.n_tokens

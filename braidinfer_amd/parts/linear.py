@@ -62,23 +62,51 @@ def linear(a, w: torch.Tensor, out, ws, accumulate: bool = False) -> None:
 BLOCK_FROM_ROWS = 8192
 
 
-def stream_layout(w: torch.Tensor, rt) -> torch.Tensor:
-    """The weight as the bf16 products read it fastest.  Parts call it once at load on every
-    matrix that only `linear` and the fused products read.  Wide matrices (from 8,192 rows:
-    gate/up, the head) become blocks of 16 rows x 128 k (`kernels.block_weight`) where the
-    runtime allows it: measured on a 28,672 x 4,096 matrix, products of 17 to 128 rows gain 10 to
-    15 %, others nothing, while matrices of 4,096 to 6,144 rows lose up to 4 % in blocks and keep
-    their rows.  BRAIDINFER_WEIGHT_LAYOUT=rows or =blocks in the environment forces one
-    (measurements and tests)."""
+def blocks_at_load(rows: int, k: int, dtype: torch.dtype, rt) -> bool:
+    """Whether `stream_layout` turns a [rows, k] matrix of this dtype into blocks."""
     want = os.environ.get("BRAIDINFER_WEIGHT_LAYOUT", "")
-    if rt.is_bf16 and K.weight_blockable(w) and want != "rows" and (w.shape[0] >= BLOCK_FROM_ROWS or want == "blocks"):
-        return K.block_weight(w)
-    return w
+    return (rt.is_bf16 and dtype == torch.bfloat16 and rt.device.type == "cuda" and k % 128 == 0 and k >= 1024
+            and want != "rows" and (rows >= BLOCK_FROM_ROWS or want == "blocks"))
 
 
-def fuse_rows(mats):
+def stream_layout(w: torch.Tensor, rt) -> torch.Tensor:
+    """The weight as the part keeps it and as the bf16 products read it fastest.  Parts call
+    it once at load on every matrix that only `linear` and the fused products read.  Wide
+    matrices (from 8,192 rows: gate/up, the head) become blocks of 16 rows x 128 k
+    (`kernels.block_weight`) where the runtime allows it: measured on a 28,672 x 4,096 matrix,
+    products of 17 to 128 rows gain 10 to 15 %, others nothing, while matrices of 4,096 to 6,144
+    rows lose up to 4 % in blocks and keep their rows.  BRAIDINFER_WEIGHT_LAYOUT=rows or =blocks
+    in the environment forces one (measurements and tests).  The result lies in the
+    runtime's arena when it has one."""
+    if w.dim() == 2 and blocks_at_load(w.shape[0], w.shape[1], w.dtype, rt) and K.weight_blockable(w):
+        return K.block_weight(w, rt.empty)
+    return rt.own(w)
+
+
+def fused_layout(mats, rt, interleave: bool = False) -> torch.Tensor:
+    """`stream_layout` of the matrices stacked along the output dimension (`fuse_rows`), or
+    of gate and up rows interleaved for the SwiGLU epilogue (`kernels.interleave_gate_up`):
+    what is kept is written once, into the runtime's memory; a stack that becomes blocks is
+    put together in a transient tensor first."""
+    rows = sum(m.shape[0] for m in mats)
+    dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+    transient = blocks_at_load(rows, mats[0].shape[1], dt, rt)
+    alloc = None if transient else rt.empty
+    w = K.interleave_gate_up(mats[0], mats[1], alloc) if interleave else fuse_rows(mats, None if transient else rt)
+    return stream_layout(w, rt)
+
+
+def fuse_rows(mats, rt=None):
     """Stack weight matrices along the output dimension so that one product serves all
     (the reference keeps q/k/v and gate/up separate: three and two launches,
-    megakernel/compile_attention.rs:82-85).  Mixed precisions widen to float32."""
+    megakernel/compile_attention.rs:82-85).  Mixed precisions widen to float32.  With a
+    runtime the result is memory of its own (`rt.empty`), else a new tensor."""
     dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
-    return torch.cat([m.to(dt) for m in mats], dim=0).contiguous()
+    rows = sum(m.shape[0] for m in mats)
+    shape = (rows,) + tuple(mats[0].shape[1:])
+    out = rt.empty(shape, dt) if rt is not None else torch.empty(shape, dtype=dt, device=mats[0].device)
+    r = 0
+    for m in mats:
+        out[r:r + m.shape[0]].copy_(m)
+        r += m.shape[0]
+    return out

@@ -23,7 +23,7 @@ class RMSNorm(Norm):
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = tensors[prefix + "weight"].to(torch.float32).contiguous()
+        self.weight = rt.own(tensors[prefix + "weight"].to(torch.float32))
 
     def forward(self, x, out, rows=None):
         K.rmsnorm(x, self.weight, out, self.eps, rows)

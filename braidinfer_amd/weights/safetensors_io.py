@@ -11,7 +11,7 @@ import mmap
 import os
 import struct
 import warnings
-from typing import Dict, Iterable, List, Tuple
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -23,6 +23,7 @@ _DTYPES = {
     "I16": (torch.int16, 2), "I8": (torch.int8, 1), "U8": (torch.uint8, 1), "BOOL": (torch.bool, 1),
 }
 _NAMES = {v[0]: k for k, v in _DTYPES.items()}
+INDEX_NAME = "model.safetensors.index.json"
 
 
 class SafetensorsFile:
@@ -76,35 +77,58 @@ class SafetensorsFile:
             t = torch.frombuffer(self._mm, dtype=tdt, count=(e - b) // _DTYPES[dt][1], offset=self._base + b)
         return t.reshape(shape)
 
+    def byte_range(self, name: str) -> Tuple[int, int, int]:
+        """(file descriptor, offset in the file, bytes) of a tensor's data, for readers that
+        bring the bytes into memory of their own."""
+        _, _, b, e = self.entries[name]
+        return self._f.fileno(), self._base + b, e - b
+
     def close(self):
         # tensors handed out keep the map alive through the buffer protocol
         self._f.close()
 
 
 class SafetensorsFolder:
-    """All tensors of a model folder: `model.safetensors`, or the shards an index names."""
+    """All tensors of a model folder: `model.safetensors`, or the shards an index names
+    (`model.safetensors.index.json` -> `weight_map`: tensor name -> file)."""
 
     def __init__(self, folder: str):
         self.folder = folder
         single = os.path.join(folder, "model.safetensors")
-        index = os.path.join(folder, "model.safetensors.index.json")
+        index = os.path.join(folder, INDEX_NAME)
         self.files: List[SafetensorsFile] = []
         self.where: Dict[str, SafetensorsFile] = {}
+        weight_map: Optional[Dict[str, str]] = None
         if os.path.isfile(single):
             paths = [single]
         elif os.path.isfile(index):
-            with open(index) as f:
-                wm = json.load(f).get("weight_map", {})
-            paths = sorted({os.path.join(folder, v) for v in wm.values()})
+            try:
+                with open(index, "r", encoding="utf-8") as f:
+                    weight_map = json.load(f).get("weight_map")
+            except (OSError, json.JSONDecodeError, AttributeError) as e:
+                raise WeightError(f"{index}: cannot read the index ({e})") from None
+            if not isinstance(weight_map, dict) or not weight_map or \
+                    not all(isinstance(k, str) and isinstance(v, str) for k, v in weight_map.items()):
+                raise WeightError(f"{index}: 'weight_map' must map tensor names to file names")
+            paths = [os.path.join(folder, v) for v in sorted(set(weight_map.values()))]
+            absent = [os.path.basename(p) for p in paths if not os.path.isfile(p)]
+            if absent:
+                raise WeightError(f"{folder}: the index names files that are not there: {', '.join(absent)}")
         else:
-            raise WeightError(f"{folder}: neither model.safetensors nor model.safetensors.index.json")
+            raise WeightError(f"{folder}: neither model.safetensors nor {INDEX_NAME}")
         for p in paths:
             sf = SafetensorsFile(p)
             self.files.append(sf)
             for n in sf.names():
                 if n in self.where:
-                    raise WeightError(f"{folder}: tensor {n} appears in two files")
+                    raise WeightError(f"{folder}: tensor {n} appears in two files "
+                                      f"({os.path.basename(self.where[n].path)} and {os.path.basename(p)})")
                 self.where[n] = sf
+        if weight_map is not None:
+            wrong = sorted(n for n, v in weight_map.items()
+                           if n not in self.where or os.path.basename(self.where[n].path) != os.path.basename(v))
+            if wrong:
+                raise WeightError(f"{folder}: the index places tensors in files that do not hold them: {', '.join(wrong)}")
 
     def names(self) -> List[str]:
         return list(self.where)
@@ -115,26 +139,98 @@ class SafetensorsFolder:
     def tensor(self, name):
         return self.where[name].tensor(name)
 
+    def byte_range(self, name):
+        return self.where[name].byte_range(name)
+
+
+
+class SafetensorsWriter:
+    """Writes one file tensor by tensor: the header comes first, from the names, dtypes and
+    shapes given up front; `write` then takes the tensors in that order and appends their
+    bytes, so no more than one tensor is held at a time."""
+
+    def __init__(self, path: str, layout: Sequence[Tuple[str, torch.dtype, Tuple[int, ...]]], metadata=None):
+        header = {}
+        if metadata:
+            header["__metadata__"] = {str(k): str(v) for k, v in metadata.items()}
+        off = 0
+        self._expect: List[Tuple[str, torch.dtype, Tuple[int, ...], int]] = []
+        for name, dtype, shape in layout:
+            if dtype not in _NAMES:
+                raise WeightError(f"cannot store dtype {dtype} of {name}")
+            if name in header:
+                raise WeightError(f"{path}: tensor {name} is named twice")
+            n = _DTYPES[_NAMES[dtype]][1]
+            for s in shape:
+                n *= int(s)
+            header[name] = {"dtype": _NAMES[dtype], "shape": [int(s) for s in shape], "data_offsets": [off, off + n]}
+            self._expect.append((name, dtype, tuple(int(s) for s in shape), n))
+            off += n
+        self.data_bytes = off
+        hj = json.dumps(header, separators=(",", ":")).encode("utf-8")
+        hj += b" " * ((8 - len(hj) % 8) % 8)
+        self.path = path
+        self._f = open(path, "wb")
+        self._f.write(struct.pack("<Q", len(hj)))
+        self._f.write(hj)
+        self._next = 0
+
+    def write(self, name: str, t: torch.Tensor) -> None:
+        if self._next >= len(self._expect):
+            raise WeightError(f"{self.path}: tensor {name} is one more than the header names")
+        want, dtype, shape, n = self._expect[self._next]
+        if name != want or t.dtype != dtype or tuple(t.shape) != shape:
+            raise WeightError(f"{self.path}: expected {want} {dtype} {list(shape)} next, "
+                              f"got {name} {t.dtype} {list(t.shape)}")
+        t = t.detach().cpu().contiguous()
+        if n:
+            self._f.write(memoryview(t.view(torch.uint8).reshape(-1).numpy()))
+        self._next += 1
+
+    def close(self) -> None:
+        self._f.close()
+        if self._next != len(self._expect):
+            raise WeightError(f"{self.path}: {len(self._expect) - self._next} tensors of the header were never written")
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, et, ev, tb):
+        if et is None:
+            self.close()
+        else:
+            self._f.close()
+
 
 def write_safetensors(path: str, tensors: Iterable[Tuple[str, torch.Tensor]], metadata=None) -> None:
-    """Write CPU tensors in the given order."""
-    header = {}
-    if metadata:
-        header["__metadata__"] = {str(k): str(v) for k, v in metadata.items()}
-    blobs = []
-    off = 0
-    for name, t in tensors:
-        t = t.detach().cpu().contiguous()
-        if t.dtype not in _NAMES:
-            raise WeightError(f"cannot store dtype {t.dtype} of {name}")
-        raw = t.view(torch.uint8).reshape(-1).numpy().tobytes() if t.numel() else b""
-        header[name] = {"dtype": _NAMES[t.dtype], "shape": list(t.shape), "data_offsets": [off, off + len(raw)]}
-        off += len(raw)
-        blobs.append(raw)
-    hj = json.dumps(header, separators=(",", ":")).encode("utf-8")
-    hj += b" " * ((8 - len(hj) % 8) % 8)
-    with open(path, "wb") as f:
-        f.write(struct.pack("<Q", len(hj)))
-        f.write(hj)
-        for b in blobs:
-            f.write(b)
+    """Write tensors that are all at hand, in the given order."""
+    items = [(n, t.detach()) for n, t in tensors]
+    with SafetensorsWriter(path, [(n, t.dtype, tuple(t.shape)) for n, t in items], metadata) as w:
+        for n, t in items:
+            w.write(n, t)
+
+
+def plan_shards(layout: Sequence[Tuple[str, torch.dtype, Tuple[int, ...]]], shard_bytes: Optional[int]) -> List[List[int]]:
+    """Indices of `layout` per file: in order, a new file whenever the next tensor would
+    take the current one beyond `shard_bytes` (None: one file)."""
+    shards: List[List[int]] = [[]]
+    used = 0
+    for i, (name, dtype, shape) in enumerate(layout):
+        n = _DTYPES[_NAMES[dtype]][1]
+        for s in shape:
+            n *= int(s)
+        if shard_bytes and shards[-1] and used + n > shard_bytes:
+            shards.append([])
+            used = 0
+        shards[-1].append(i)
+        used += n
+    return shards
+
+
+def shard_file_name(i: int, n: int) -> str:
+    return "model.safetensors" if n == 1 else f"model-{i + 1:05d}-of-{n:05d}.safetensors"
+
+
+def write_index(folder: str, weight_map: Dict[str, str], total_size: int) -> None:
+    with open(os.path.join(folder, INDEX_NAME), "w", encoding="utf-8") as f:
+        json.dump({"metadata": {"total_size": int(total_size)}, "weight_map": weight_map}, f, indent=2)

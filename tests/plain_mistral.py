@@ -25,12 +25,11 @@ def bf16_bytes_to_f32(raw):
     return (u16 << 16).view(np.float32)
 
 
-def read_folder(folder):
-    """config.json as a dict and every tensor of model.safetensors as float32 arrays
-    (container layout: braidinfer-core/src/safetensors.rs:71-80)."""
-    with open(os.path.join(folder, "config.json")) as f:
-        cfg = json.load(f)
-    with open(os.path.join(folder, "model.safetensors"), "rb") as f:
+def read_safetensors(path):
+    """Every tensor of one safetensors file as float32 arrays: 8 bytes header length, a JSON
+    header {name: {dtype, shape, data_offsets}}, then the data
+    (braidinfer-core/src/safetensors.rs:71-80)."""
+    with open(path, "rb") as f:
         (hlen,) = struct.unpack("<Q", f.read(8))
         header = json.loads(f.read(hlen))
         data = f.read()
@@ -47,7 +46,91 @@ def read_folder(folder):
         else:
             raise ValueError(f"dtype {e['dtype']} of {name}")
         tensors[name] = a.reshape(e["shape"]).astype(F)
+    return tensors
+
+
+def read_folder(folder):
+    """config.json as a dict and every tensor as float32 arrays, from model.safetensors or
+    from the files that model.safetensors.index.json's weight_map names
+    (braidinfer-core/src/safetensors.rs:102-159)."""
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    single = os.path.join(folder, "model.safetensors")
+    if os.path.isfile(single):
+        return cfg, read_safetensors(single)
+    with open(os.path.join(folder, "model.safetensors.index.json")) as f:
+        weight_map = json.load(f)["weight_map"]
+    tensors = {}
+    for fname in sorted(set(weight_map.values())):
+        part = read_safetensors(os.path.join(folder, fname))
+        for name, a in part.items():
+            if weight_map.get(name) != fname or name in tensors:
+                raise ValueError(f"{name} in {fname} disagrees with the index")
+            tensors[name] = a
     return cfg, tensors
+
+
+# ------------------------------------------------------------------ random weights ----
+_M64 = (1 << 64) - 1
+_GOLDEN = 0x9E3779B97F4A7C15
+
+
+def _mix64(z):
+    z &= _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def tensor_names(cfg):
+    """The name table of a Mistral folder, in the order the random generator numbers the
+    tensors: embedding; per layer the attention norm, q, k, v, o, the feed-forward norm,
+    gate, up, down; the final norm; the head unless tied."""
+    sz = sizes(cfg)
+    H, I, V, nq, nkv, hd = sz["H"], sz["I"], sz["V"], sz["nq"], sz["nkv"], sz["hd"]
+    out = [("model.embed_tokens.weight", (V, H))]
+    for i in range(sz["L"]):
+        p = f"model.layers.{i}."
+        out += [(p + "input_layernorm.weight", (H,)),
+                (p + "self_attn.q_proj.weight", (nq * hd, H)), (p + "self_attn.k_proj.weight", (nkv * hd, H)),
+                (p + "self_attn.v_proj.weight", (nkv * hd, H)), (p + "self_attn.o_proj.weight", (H, nq * hd)),
+                (p + "post_attention_layernorm.weight", (H,)),
+                (p + "mlp.gate_proj.weight", (I, H)), (p + "mlp.up_proj.weight", (I, H)),
+                (p + "mlp.down_proj.weight", (H, I))]
+    out.append(("model.norm.weight", (H,)))
+    if not sz["tied"]:
+        out.append(("lm_head.weight", (V, H)))
+    return out
+
+
+def random_weights(cfg, seed, std=0.02, vector_jitter=0.0):
+    """The random-weights mode's tensors as float32 arrays holding bfloat16 values, written
+    with Python integers from the generator's definition (ours; the reference has no random
+    weights): key = mix(mix(seed + G) + (t + 1) G) for tensor t of the name table;
+    word(c) = mix(key + (c + 1) G); a matrix element i is (the twelve 16-bit fields of
+    word(3i), word(3i+1), word(3i+2) added up, minus 393210) * (float32(std) * 2^-16); a norm
+    weight is 1 + (2 u - 1) * jitter with u = (word(i) >> 40) * 2^-24; float32 is rounded to
+    bfloat16 to nearest even (quant.rs:203-207)."""
+    scale = F(F(std) * F(2.0 ** -16))
+    out = {}
+    for t, (name, shape) in enumerate(tensor_names(cfg)):
+        key = _mix64(_mix64(seed + _GOLDEN) + (t + 1) * _GOLDEN)
+        n = int(np.prod(shape))
+        vals = np.empty(n, dtype=F)
+        for i in range(n):
+            if len(shape) == 1:
+                u = F(_mix64(key + (i + 1) * _GOLDEN) >> 40) * F(2.0 ** -24)
+                vals[i] = F(F(1.0) + F(F(F(u + u) - F(1.0)) * F(vector_jitter)))
+            else:
+                s = 0
+                for c in (3 * i, 3 * i + 1, 3 * i + 2):
+                    w = _mix64(key + (c + 1) * _GOLDEN)
+                    s += (w & 0xFFFF) + ((w >> 16) & 0xFFFF) + ((w >> 32) & 0xFFFF) + (w >> 48)
+                vals[i] = F(s - 393210) * scale
+        bits = vals.view(np.uint32)
+        rounded = ((bits + (((bits >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF))) >> np.uint32(16)) << np.uint32(16)
+        out[name] = rounded.astype(np.uint32).view(F).reshape(shape)
+    return out
 
 
 def sizes(cfg):
