@@ -15,6 +15,7 @@
 // so that the accumulator registers of a lane hold 8 consecutive keys: then the k-slots of
 // the second product are in key order and V^T is read 16 contiguous bytes at a time.
 #include "common.h"
+#include "no_alloc.h"
 
 #define PAGE 64
 #define LOG2E 1.4426950408889634f
@@ -1202,4 +1203,57 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
     if (rc != BR_OK || nsplit == 1) return rc;
     attn_decode_combine_kernel<<<dim3(nq, B), 256, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
     return br_check_launch();
+}
+
+
+// ------------------------------------------------ an entry point that allocates nothing ----
+// See no_alloc.h.  The scratch of the split runs lives in a device array of this file; host
+// code never uses the array's name as an address (on the host it is a stand-in, not device
+// memory): the address is asked for once per device and kept.
+static __device__ __align__(256) float scratch[BR_NO_ALLOC_SCRATCH_FLOATS];
+static float* scratch_of_device[64];
+
+static float* no_alloc_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        fprintf(stderr, "braidinfer_amd: br_attn_decode_bf16_no_alloc: no current device\n");
+        return nullptr;
+    }
+    if (!scratch_of_device[dev]) {
+        float* p = nullptr;
+        hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            fprintf(stderr, "braidinfer_amd: br_attn_decode_bf16_no_alloc: hipGetSymbolAddress failed: %s\n",
+                    hipGetErrorString(e));
+            return nullptr;
+        }
+        scratch_of_device[dev] = p;
+    }
+    return scratch_of_device[dev];
+}
+
+extern "C" int br_attn_decode_bf16_no_alloc(const void* q, size_t q_stride, void* out, const int* slots,
+                                            const int* ctx_lens, const int* block_table, int table_stride,
+                                            void* cache, int B, int nq, int nkv, int hd, int page, int window,
+                                            float scale, int nsplit, int variant, int fuse, const float* cs,
+                                            const float* sn, int write_cache, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (nq <= 0 || hd <= 0 || nsplit < 1) return BR_BAD_ARG;
+    float *part_o = nullptr, *part_ml = nullptr;
+    if (nsplit > 1) {
+        const unsigned long long rows = (unsigned long long)B * nq * nsplit;
+        const unsigned long long o_floats = (rows * hd + 63) / 64 * 64, need = o_floats + rows * 2;
+        if (need > BR_NO_ALLOC_SCRATCH_FLOATS) {
+            fprintf(stderr, "braidinfer_amd: br_attn_decode_bf16_no_alloc: %d sequences x %d heads x %d runs x head size %d "
+                            "need %llu floats of scratch, the array holds %u\n", B, nq, nsplit, hd, need,
+                    (unsigned)BR_NO_ALLOC_SCRATCH_FLOATS);
+            return BR_TOO_LARGE;
+        }
+        float* base = no_alloc_scratch();
+        if (!base) return BR_LAUNCH_FAILED;
+        part_o = base;
+        part_ml = base + o_floats;
+    }
+    return br_attn_decode_bf16(q, q_stride, out, slots, ctx_lens, block_table, table_stride, cache, B, nq, nkv, hd,
+                               page, window, scale, nsplit, part_o, part_ml, variant, fuse, cs, sn, write_cache, s);
 }

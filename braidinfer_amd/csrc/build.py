@@ -37,7 +37,7 @@ MODULES: Dict[str, List[str]] = {
     "attention_bf16": ["attention_bf16.hip"],
     "random_weights": ["random_weights.hip"],
 }
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
