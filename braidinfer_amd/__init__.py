@@ -9,7 +9,7 @@ replay.  Every device operation is a hand-written HIP kernel under `csrc/`.
 from .errors import BraidError, ConfigError, WeightError, CacheError, KernelError, StepError
 from .config import (MistralConfig, preset, PRESETS, config_from_folder, config_from_dict, spec_of,
                      register_architecture, registered_architectures, PartSpec, LayerSpec, ScheduleEntry,
-                     ModelSpec)
+                     ModelSpec, prenorm_layer)
 from .parts import register_part
 from .engine import Engine, StepEntry, DecoderModel, generate, GenerationResult, GenerationStats
 from .sampling import SamplingParams, Sampler
@@ -19,5 +19,5 @@ __version__ = "0.1.0"
 __all__ = ["BraidError", "ConfigError", "WeightError", "CacheError", "KernelError", "StepError",
            "MistralConfig", "preset", "PRESETS", "config_from_folder", "config_from_dict", "spec_of",
            "register_architecture", "registered_architectures", "PartSpec", "LayerSpec", "ScheduleEntry",
-           "ModelSpec", "register_part", "Engine", "StepEntry", "DecoderModel", "generate", "GenerationResult",
+           "ModelSpec", "prenorm_layer", "register_part", "Engine", "StepEntry", "DecoderModel", "generate", "GenerationResult",
            "GenerationStats", "SamplingParams", "Sampler"]

@@ -4,13 +4,16 @@ and a fixed-size state area per sequence.
 Layout (decided for the attention kernels of this library, not taken from the
 reference, whose page holds all layers of 64 tokens as f32,
 crates/braidinfer-runtime/src/paged_kv.rs:17-21): a *group* gathers the cache units
-whose needs are equal (kv heads, head size, full or windowed).  A group owns one page
-pool and one block table `[slot, page index in sequence] -> page`; every unit of the
-group owns storage `[n_pages, 2 (K|V), kv_heads, page_tokens * head_dim]` indexed by the
-same page numbers: keys as `[token, head_dim]` after rotation, values transposed as
-`[head_dim, token]` (the operand layout of the matrix-core attention kernels; the tensor's
-last two dimensions are declared `[page_tokens, head_dim]` for both).  A windowed
-group returns pages that lie wholly before the window to its pool after every step.
+whose needs are equal (kv heads, widths of what is kept per token, full or windowed).  A
+group owns one page pool and one block table `[slot, page index in sequence] -> page`;
+every unit of the group owns storage `[n_pages, elements of a page]` indexed by the same
+page numbers.  A page holds, for its 64 tokens, first the keys of every kv head
+(`[kv_heads, 64 * key_dim]`), then the values (`[kv_heads, 64 * value_dim]`); the two widths
+may differ and the second may be zero (a mixer that keeps one row per token).  What lies
+inside a head's block is the mixer's business: the attention part of this library keeps
+keys as `[token, head_dim]` after rotation and values transposed as `[head_dim, token]`
+(the operand layout of the matrix-core attention kernels).  A windowed group returns pages
+that lie wholly before the window to its pool after every step.
 """
 from __future__ import annotations
 
@@ -27,11 +30,22 @@ PAGE_TOKENS = 64
 
 @dataclass(frozen=True)
 class CacheNeed:
-    """What a mixer asks of the cache for one unit: growing keys/values."""
+    """What a mixer asks of the cache for one unit: rows that grow with the sequence.
+    Per token and kv head it keeps `head_dim` elements of keys and `value_dim` elements of
+    values (None: as many as of keys; 0: none)."""
 
     kv_heads: int
     head_dim: int
     window: Optional[int] = None      # None: all keys; W: the last W positions
+    value_dim: Optional[int] = None
+
+    @property
+    def key_dim(self) -> int:
+        return self.head_dim
+
+    @property
+    def val_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -56,11 +70,31 @@ class CacheGroup:
         self.table_cpu = torch.full((n_slots, max_pages_per_seq), -1, dtype=torch.int32)
         self.table_dev = self.table_cpu.to(self.device) if self.device.type != "cpu" else self.table_cpu
         self._dirty: Dict[int, Tuple[int, int]] = {}
+        if need.kv_heads <= 0 or need.key_dim <= 0 or need.val_dim < 0:
+            raise CacheError(f"a cache unit needs kv heads and a key width above zero, got {need}")
+        self.key_elems = need.kv_heads * page_tokens * need.key_dim        # of one page
+        self.page_elems = self.key_elems + need.kv_heads * page_tokens * need.val_dim
         self.storage: Dict[int, torch.Tensor] = {}
         if dtype is not None:
             for u in self.unit_ids:
-                self.storage[u] = torch.zeros((n_pages, 2, need.kv_heads, page_tokens, need.head_dim),
-                                              dtype=dtype, device=self.device)
+                self.storage[u] = torch.zeros((n_pages, self.page_elems), dtype=dtype, device=self.device)
+
+    # -- views of a unit's storage ----------------------------------------------------------
+    def keys(self, unit: int) -> torch.Tensor:
+        """[pages, kv_heads, page_tokens * key_dim]: every head's block of keys, page by page."""
+        return self.storage[unit][:, :self.key_elems].view(-1, self.need.kv_heads, self.page_tokens * self.need.key_dim)
+
+    def values(self, unit: int) -> torch.Tensor:
+        """[pages, kv_heads, page_tokens * value_dim]."""
+        return self.storage[unit][:, self.key_elems:].view(-1, self.need.kv_heads, self.page_tokens * self.need.val_dim)
+
+    def storage_view(self, unit: int) -> torch.Tensor:
+        """Keys and values of equal width as one tensor [pages, 2, kv_heads, page_tokens, head_dim]
+        (what this library's attention kernels take); the flat [pages, page elements] otherwise."""
+        n = self.need
+        if n.val_dim == n.key_dim:
+            return self.storage[unit].view(-1, 2, n.kv_heads, self.page_tokens, n.key_dim)
+        return self.storage[unit]
 
     # -- bookkeeping, all on the host ------------------------------------------------
     def pages_needed(self, slot: int, new_len: int) -> int:
@@ -202,6 +236,24 @@ class SequenceCache:
                 g.grow(s, self.lengths[s] + n)
             g.sync()
 
+    def pages_held(self) -> List[List[int]]:
+        """Per group and slot the number of page entries a sequence has now (what
+        `release_reserved` rolls back to)."""
+        return [[len(p) for p in g.pages] for g in self.groups]
+
+    def release_reserved(self, slots: Sequence[int], held: List[List[int]]) -> None:
+        """Undo a `reserve` that no `commit` follows: pages the slots took since `held` was
+        read go back to their pools."""
+        for g, before in zip(self.groups, held):
+            for s in slots:
+                extra = g.pages[s][before[s]:]
+                if extra:
+                    g.pool.free([p for p in extra if p >= 0])
+                    g.table_cpu[s, before[s]:len(g.pages[s])] = -1
+                    g._mark(s, before[s], len(g.pages[s]))
+                    del g.pages[s][before[s]:]
+            g.sync()
+
     def commit(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         for s, n in zip(slots, new_tokens):
             self.lengths[s] += n
@@ -210,7 +262,7 @@ class SequenceCache:
 
     # -- views for parts ---------------------------------------------------------------
     def unit_storage(self, unit: int) -> torch.Tensor:
-        return self.group_of_unit[unit].storage[unit]
+        return self.group_of_unit[unit].storage_view(unit)
 
     def unit_group(self, unit: int) -> CacheGroup:
         return self.group_of_unit[unit]

@@ -14,8 +14,8 @@ Output: the generated text on standard output (token ids when the folder has no
 tokenizer), statistics on standard error, including the reference's `PPTG` line.
 
 Flags beyond the reference: --prompt-ids, --batch-file, --temperature, --top-k, --top-p,
---min-p, --repetition-penalty, --seed, --dtype, --random-weights SEED --preset NAME,
---list-weights.
+--min-p, --repetition-penalty, --seed, --dtype, --random-weights SEED --preset NAME
+(--save-folder DIR, --shard-bytes N), --list-weights.
 """
 from __future__ import annotations
 
@@ -67,6 +67,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--random-weights", type=int, metavar="SEED", default=None,
                     help="make a model folder of random weights for --preset instead of reading MODEL")
     ap.add_argument("--preset", default="tiny-a")
+    ap.add_argument("--save-folder", metavar="DIR", default=None,
+                    help="with --random-weights: write the model folder here and keep it (default: a temporary folder)")
+    ap.add_argument("--shard-bytes", type=int, default=None,
+                    help="with --random-weights: cut the folder into files of about this size with an index")
     ap.add_argument("--list-weights", action="store_true", help="print the tensor names and shapes the model needs")
     ap.add_argument("--max-seq-len", type=int, default=None)
     ap.add_argument("rest", nargs="*")
@@ -84,9 +88,18 @@ def main(argv: Optional[List[str]] = None) -> int:
     tmp = None
     try:
         if args.random_weights is not None:
+            import torch
             cfg = B.preset(args.preset)
-            tmp = tempfile.mkdtemp(prefix="braidinfer_random_")
-            model_dir = B.Engine.write_random_folder(tmp, cfg, seed=args.random_weights)
+            if args.save_folder:
+                where = args.save_folder
+            else:
+                where = tmp = tempfile.mkdtemp(prefix="braidinfer_random_")
+            t0 = time.perf_counter()
+            # the values are the same bits wherever they are made; the GPU makes them faster
+            model_dir = B.Engine.write_random_folder(where, cfg, seed=args.random_weights, shard_bytes=args.shard_bytes,
+                                                     device="cuda:0" if torch.cuda.is_available() else "cpu")
+            print(f"random weights of {args.preset} (seed {args.random_weights}) written to {model_dir} in "
+                  f"{time.perf_counter() - t0:.1f} s", file=sys.stderr)
         if model_dir is None:
             print("generate: no model: set MODEL, pass a folder, or use --random-weights SEED --preset NAME",
                   file=sys.stderr)
@@ -127,8 +140,13 @@ def main(argv: Optional[List[str]] = None) -> int:
         t0 = time.perf_counter()
         engine = B.Engine.from_folder(model_dir, dtype=args.dtype, max_tokens=max(room, 64), max_seq_len=cap_seq)
         print(f"LOAD PROFILE: Engine.from_folder = {(time.perf_counter() - t0) * 1e3:.0f} ms", file=sys.stderr)
+        if engine.load_profile is not None:
+            print(engine.load_profile.line(), file=sys.stderr)
+        import resource
+        print(f"host memory at its peak: {resource.getrusage(resource.RUSAGE_SELF).ru_maxrss / 1e6:.2f} GB",
+              file=sys.stderr)
         print(f"max_seq_len: {engine.cache.max_seq_len}", file=sys.stderr)
-        print(f"stop tokens: {list(engine.spec.stop_token_ids)}", file=sys.stderr)
+        print(f"stop tokens: {list(engine.stop_token_ids)}", file=sys.stderr)
         t0 = time.perf_counter()
         outs, stats = engine.generate(prompts, max_new_tokens=max_tokens, temperature=args.temperature,
                                       seed=args.seed, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,

@@ -15,7 +15,7 @@ from dataclasses import dataclass, field, asdict
 from typing import Any, Dict, List, Optional, Tuple
 
 from ..errors import ConfigError
-from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, default_schedule
+from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, default_schedule, prenorm_layer
 
 ARCHITECTURE = "MistralForCausalLM"
 
@@ -132,6 +132,10 @@ class MistralConfig:
                 f"of num_key_value_heads {self.num_key_value_heads}")
         if self.head_dim % 2:
             raise ConfigError(f"config.json: head_dim {self.head_dim} must be even for rotary pairs")
+        from ..parts.attention import MAX_HEAD_DIM      # the attention part's own limit, refused here already
+        if self.head_dim > MAX_HEAD_DIM:
+            raise ConfigError(f"config.json: head_dim {self.head_dim} is beyond the largest head size any attention "
+                              f"kernel of this library takes ({MAX_HEAD_DIM})")
         if self.sliding_window is not None and self.sliding_window <= 0:
             raise ConfigError(f"config.json: sliding_window must be positive or null, found {self.sliding_window}")
         if self.rope_pairing not in ("half", "adjacent"):
@@ -209,8 +213,11 @@ def build_spec(cfg: MistralConfig) -> ModelSpec:
             "hidden_size": cfg.hidden_size,
             "intermediate_size": cfg.intermediate_size,
         })
-        layers.append(LayerSpec(prefix=f"model.layers.{i}.", mixer=mixer, feed_forward=ffn,
-                                mixer_norm=norm, ffn_norm=norm))
+        # tensor names of MistralForCausalLM checkpoints (the reference looks the same ones up,
+        # model_load.rs:624-744)
+        layers.append(prenorm_layer(f"model.layers.{i}.", mixer, ffn, norm, norm, mixer_name="self_attn.",
+                                    feed_forward_name="mlp.", mixer_norm_name="input_layernorm.",
+                                    ffn_norm_name="post_attention_layernorm."))
     return ModelSpec(
         architecture=ARCHITECTURE,
         hidden_size=cfg.hidden_size,
@@ -224,6 +231,7 @@ def build_spec(cfg: MistralConfig) -> ModelSpec:
         positions={"rope": PartSpec("rope", {"rotary_dim": cfg.head_dim, "theta": cfg.rope_theta,
                                              "pairing": cfg.rope_pairing})},
         max_position_embeddings=cfg.max_position_embeddings,
+        embedding_prefix="model.embed_tokens.", final_norm_prefix="model.norm.", lm_head_prefix="lm_head.",
         stop_token_ids=list(cfg.eos_token_id),
         bos_token_id=cfg.bos_token_id,
     )

@@ -89,6 +89,29 @@ def read_config_json(folder: str) -> Dict[str, Any]:
     return d
 
 
+def generation_stop_tokens(folder: str):
+    """`eos_token_id` (an integer or a list) of the folder's generation_config.json, [] when
+    the file or the key is absent.  The reference gathers its stop set from the tokenizer's
+    end markers and config.json's `text_config.eos_token_id`
+    (crates/braidinfer-runtime/src/generate.rs:34-68); checkpoints of this architecture
+    carry theirs in config.json and in generation_config.json, and both are read."""
+    path = os.path.join(folder, "generation_config.json")
+    if not os.path.isfile(path):
+        return []
+    try:
+        with open(path, "r", encoding="utf-8") as f:
+            d = json.load(f)
+    except json.JSONDecodeError as e:
+        raise ConfigError(f"{path}: not valid JSON ({e})") from None
+    eos = d.get("eos_token_id") if isinstance(d, dict) else None
+    if eos is None:
+        return []
+    ids = [eos] if isinstance(eos, int) and not isinstance(eos, bool) else eos
+    if not isinstance(ids, (list, tuple)) or not all(isinstance(e, int) and not isinstance(e, bool) and e >= 0 for e in ids):
+        raise ConfigError(f"{path}: eos_token_id must be a token id or a list of them, found {eos!r}")
+    return list(ids)
+
+
 def config_from_dict(d: Dict[str, Any]):
     arch = architecture_of(d)
     return arch.config_class.from_dict(d)

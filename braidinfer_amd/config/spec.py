@@ -30,24 +30,48 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a mixer and a feed-forward, each behind its norm, arranged by `block`.
+    """One layer: a mixer, a feed-forward and any number of norms, arranged by `block`.
 
     `mixer` or `feed_forward` may be None (a layer with only the other half, as the
-    reference's `LayerType::Ffn` / `FfnType::None`, config.rs:26-37).  `prefix` is the
-    tensor-name prefix of the layer's weights, e.g. ``model.layers.3.``.
+    reference's `LayerType::Ffn` / `FfnType::None`, config.rs:26-37).  `norms` maps a role
+    to a norm; which roles exist is between the architecture's builder and the block
+    arrangement it names (`prenorm_residual` reads "mixer" and "feed_forward", the norms in
+    front of the two halves; an arrangement with norms behind the halves too would read two
+    more roles).  `prefix` is the tensor-name prefix of the layer's weights, e.g.
+    ``model.layers.3.``; `names` gives the piece under it for "mixer", "feed_forward" and
+    every role of `norms` as "norm.<role>" (the names of the architecture's checkpoints: the
+    builder supplies them, nothing here knows any).
     """
 
     prefix: str
-    mixer: Optional[PartSpec]
-    feed_forward: Optional[PartSpec]
-    mixer_norm: Optional[PartSpec]
-    ffn_norm: Optional[PartSpec]
+    mixer: Optional[PartSpec] = None
+    feed_forward: Optional[PartSpec] = None
+    norms: Dict[str, PartSpec] = field(default_factory=dict)
     block: str = "prenorm_residual"
-    # tensor-name pieces under `prefix` (the names of the architecture's checkpoints)
-    mixer_name: str = "self_attn."
-    feed_forward_name: str = "mlp."
-    mixer_norm_name: str = "input_layernorm."
-    ffn_norm_name: str = "post_attention_layernorm."
+    names: Dict[str, str] = field(default_factory=dict)
+
+    def name_of(self, what: str) -> str:
+        if what not in self.names:
+            raise KeyError(f"layer {self.prefix!r}: no tensor-name piece for {what!r} (names: {sorted(self.names)})")
+        return self.prefix + self.names[what]
+
+
+def prenorm_layer(prefix: str, mixer: Optional[PartSpec], feed_forward: Optional[PartSpec],
+                  mixer_norm: Optional[PartSpec], ffn_norm: Optional[PartSpec], mixer_name: str,
+                  feed_forward_name: str, mixer_norm_name: str, ffn_norm_name: str) -> LayerSpec:
+    """The common layer: x += mixer(norm(x)); x += feed_forward(norm(x)), with the four
+    tensor-name pieces of the architecture's checkpoints."""
+    norms, names = {}, {}
+    if mixer is not None:
+        if mixer_norm is not None:
+            norms["mixer"], names["norm.mixer"] = mixer_norm, mixer_norm_name
+        names["mixer"] = mixer_name
+    if feed_forward is not None:
+        if ffn_norm is not None:
+            norms["feed_forward"], names["norm.feed_forward"] = ffn_norm, ffn_norm_name
+        names["feed_forward"] = feed_forward_name
+    return LayerSpec(prefix=prefix, mixer=mixer, feed_forward=feed_forward, norms=norms, block="prenorm_residual",
+                     names=names)
 
 
 @dataclass(frozen=True)
@@ -78,11 +102,12 @@ class ModelSpec:
     # position encodings by name; mixers refer to them by that name
     positions: Dict[str, PartSpec]
     max_position_embeddings: int
+    # tensor-name prefixes of the parts outside the layers, as the architecture's checkpoints name them
+    embedding_prefix: str
+    final_norm_prefix: str
+    lm_head_prefix: str
     stop_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
-    embedding_prefix: str = "model.embed_tokens."
-    final_norm_prefix: str = "model.norm."
-    lm_head_prefix: str = "lm_head."
 
 
 def default_schedule(n_layers: int) -> List[ScheduleEntry]:

@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..cache import SequenceCache
-from ..config import config_from_folder, spec_of
+from ..config import config_from_folder, generation_stop_tokens, spec_of
 from ..errors import BraidError, CacheError, ConfigError, KernelError, StepError
 from ..parts import Runtime
 from ..weights import FolderTensors, RandomTensors, write_model_folder
@@ -40,6 +40,9 @@ class StepEntry:
     slot: int
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    # position numbers for the position encodings, one integer or k integers per token; None: the
+    # tokens' places in the sequence.  All entries of a step give them, or none does.
+    position_ids: Optional[Sequence] = None
 
 
 def _require_gpu(device: torch.device) -> None:
@@ -70,6 +73,8 @@ class Engine:
         self.use_graphs = bool(use_graphs) and model.graph_safe()
         self._graphs = None
         self.load_profile = None
+        # tokens that end a sequence: the configuration's, and for a folder also its generation_config.json's
+        self.stop_token_ids: List[int] = list(self.spec.stop_token_ids)
 
     # ---- construction ------------------------------------------------------------------
     @classmethod
@@ -97,8 +102,11 @@ class Engine:
         `engine.load_profile.line()` says how the load went (the reference prints a
         `LOAD PROFILE` line, bin/generate.rs:62-68)."""
         config = config_from_folder(folder)
-        return cls._from_source(config, lambda specs, allowed, dev, dt: FolderTensors(folder, specs, dev, dt, allowed),
-                                dtype, device, max_tokens, max_seq_len, n_slots, use_graphs)
+        more_stops = generation_stop_tokens(folder)
+        eng = cls._from_source(config, lambda specs, allowed, dev, dt: FolderTensors(folder, specs, dev, dt, allowed),
+                               dtype, device, max_tokens, max_seq_len, n_slots, use_graphs)
+        eng.stop_token_ids += [t for t in more_stops if t not in eng.stop_token_ids]
+        return eng
 
     @classmethod
     def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192,
@@ -131,13 +139,17 @@ class Engine:
         return self.cache.length(slot)
 
     # ---- the step function -------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], probe=None) -> torch.Tensor:
         """Run the given tokens of each entry's sequence as one batch, from the cache
         earlier steps left; return float32 logits `[number of wanted places, vocab]` on the
         device, in the order of the entries and of each entry's `want`, in a tensor of
         their own (later steps do not touch it).
 
-        Nothing is changed if the step cannot be run (bad entry, no room in the cache)."""
+        `probe(name, tensor)` is handed to the model (see `DecoderModel.forward`); a probed
+        step runs its kernels one by one, never from a recorded graph.
+
+        Nothing is changed if the step cannot be run (bad entry, no room in the cache, a size
+        no kernel takes): the sequences keep their lengths and pages taken for the step go back."""
         if not entries:
             raise StepError("a step needs at least one entry")
         slots = [e.slot for e in entries]
@@ -161,23 +173,42 @@ class Engine:
                     raise StepError(f"slot {e.slot}: wanted place {w!r} is outside its {len(tl)} tokens")
                 rows.append(base + int(w))
             base += len(tl)
+        with_ids = [e.position_ids is not None for e in entries]
+        if any(with_ids) and not all(with_ids):
+            raise StepError("position_ids: given for some entries of the step and not for others")
+        position_ids = None
+        if all(with_ids):
+            position_ids = [e.position_ids for e in entries]
+            for e, tl in zip(entries, token_lists):
+                if len(e.position_ids) != len(tl):
+                    raise StepError(f"slot {e.slot}: {len(e.position_ids)} position numbers for {len(tl)} tokens")
         new = [len(tl) for tl in token_lists]
+        held = self.cache.pages_held()
         self.cache.reserve(slots, new)          # all or nothing
-        starts = [self.cache.lengths[s] for s in slots]
-        n_want = len(rows)
-        if self.use_graphs and all(n == 1 for n in new) and len(slots) <= 256:
-            if self._graphs is None:
-                from .graph import DecodeGraphs
-                self._graphs = DecodeGraphs(self.model, self.cache, self.device)
-            all_logits = self._graphs.run(slots, [tl[0] for tl in token_lists], starts)
-            self.cache.commit(slots, new)
-            if rows == list(range(len(slots))):
-                return all_logits.clone()          # the graph's buffer is overwritten by the next step
-            return all_logits[torch.tensor(rows, dtype=torch.long, device=self.device)]
-        step = pack_step(slots, token_lists, starts, self.device, self.ws)
-        want_rows = (torch.tensor(rows, dtype=torch.int32).to(self.device) if n_want
-                     else torch.empty(0, dtype=torch.int32, device=self.device))
-        logits = self.model.forward(step, self.cache, want_rows, n_want)
+        try:
+            starts = [self.cache.lengths[s] for s in slots]
+            n_want = len(rows)
+            if (self.use_graphs and probe is None and position_ids is None and all(n == 1 for n in new)
+                    and len(slots) <= 256):
+                if self._graphs is None:
+                    from .graph import DecodeGraphs
+                    self._graphs = DecodeGraphs(self.model, self.cache, self.device)
+                all_logits = self._graphs.run(slots, [tl[0] for tl in token_lists], starts)
+                if rows == list(range(len(slots))):
+                    logits = all_logits.clone()          # the graph's buffer is overwritten by the next step
+                else:
+                    logits = all_logits[torch.tensor(rows, dtype=torch.long, device=self.device)]
+            else:
+                try:
+                    step = pack_step(slots, token_lists, starts, self.device, self.ws, position_ids=position_ids)
+                except ValueError as e:
+                    raise StepError(str(e)) from None
+                want_rows = (torch.tensor(rows, dtype=torch.int32).to(self.device) if n_want
+                             else torch.empty(0, dtype=torch.int32, device=self.device))
+                logits = self.model.forward(step, self.cache, want_rows, n_want, probe=probe)
+        except BaseException:
+            self.cache.release_reserved(slots, held)
+            raise
         self.cache.commit(slots, new)
         return logits
 

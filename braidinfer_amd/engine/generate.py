@@ -83,7 +83,8 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
     """Generate for every prompt; returns (results in request order, stats).
 
     `params`: one `SamplingParams` for all or one per request; None is greedy.
-    `stop_token_ids`: None takes the model's (config.json `eos_token_id`)."""
+    `stop_token_ids`: None takes the engine's (`eos_token_id` of config.json and of
+    generation_config.json)."""
     n = len(prompts)
     if params is None:
         plist = [SamplingParams.greedy() for _ in range(n)]
@@ -97,7 +98,7 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
         p.validate()
     if max_new_tokens < 0:
         raise StepError(f"max_new_tokens must be >= 0, got {max_new_tokens}")
-    stops = set(engine.spec.stop_token_ids if stop_token_ids is None else stop_token_ids)
+    stops = set(engine.stop_token_ids if stop_token_ids is None else stop_token_ids)
     seeds = [resolve_seed(p.seed) for p in plist]
     if sampler is None:
         sampler = Sampler(engine.device, engine.vocab_size)

@@ -29,17 +29,47 @@ class Layer:
         self.spec = spec
         self.mixer = build_part("mixer", spec.mixer) if spec.mixer else None
         self.feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward else None
-        self.mixer_norm = build_part("norm", spec.mixer_norm) if (spec.mixer and spec.mixer_norm) else None
-        self.ffn_norm = build_part("norm", spec.ffn_norm) if (spec.feed_forward and spec.ffn_norm) else None
-        self.run = block_arrangement(spec.block)
+        self.norms: Dict[str, object] = {role: build_part("norm", ns) for role, ns in spec.norms.items()}
+        arrangement = block_arrangement(spec.block)
+        # an arrangement is an object with `run` (and optionally `first_norm`), or a plain function
+        self.run = getattr(arrangement, "run", arrangement)
+        self._first_norm = getattr(arrangement, "first_norm", None)
         self.rt: Optional[Runtime] = None
 
+    # the two norms of the common arrangement, by their roles
+    @property
+    def mixer_norm(self):
+        return self.norms.get("mixer")
+
+    @property
+    def ffn_norm(self):
+        return self.norms.get("feed_forward")
+
+    def first_norm(self):
+        """The norm that reads the residual rows first when this layer runs, if its
+        arrangement says."""
+        return self._first_norm(self) if self._first_norm is not None else None
+
     def named_parts(self):
+        """(part, tensor-name prefix) in the order of the spec's `names`, which is the order
+        of the layer's tensors in the model's name table."""
         s = self.spec
-        for part, name in ((self.mixer_norm, s.mixer_norm_name), (self.mixer, s.mixer_name),
-                           (self.ffn_norm, s.ffn_norm_name), (self.feed_forward, s.feed_forward_name)):
+        for what in s.names:
+            if what == "mixer":
+                part = self.mixer
+            elif what == "feed_forward":
+                part = self.feed_forward
+            elif what.startswith("norm."):
+                part = self.norms.get(what[5:])
+            else:
+                raise ConfigError(f"layer {s.prefix!r}: names has {what!r}; known: mixer, feed_forward, norm.<role>")
             if part is not None:
-                yield part, s.prefix + name
+                yield part, s.name_of(what)
+        named = set(s.names)
+        missing = [w for w, p in [("mixer", self.mixer), ("feed_forward", self.feed_forward)]
+                   + [("norm." + r, n) for r, n in self.norms.items()] if p is not None and w not in named]
+        if missing:
+            raise ConfigError(f"layer {s.prefix!r}: no tensor-name piece for {missing}")
 
 
 class DecoderModel:
@@ -61,6 +91,9 @@ class DecoderModel:
                     written.add(e.cache)
                 elif e.cache not in written:
                     raise ConfigError(f"schedule entry reads cache {e.cache} before any entry writes it")
+        for layer in self.layers:
+            if layer.mixer is not None:
+                layer.mixer.check_positions(self.positions)
         self.rt: Optional[Runtime] = None
 
     # ---- weights -------------------------------------------------------------------
@@ -132,33 +165,44 @@ class DecoderModel:
 
     # ---- one step ----------------------------------------------------------------------
     def forward(self, step: StepBatch, cache: SequenceCache, want_rows: torch.Tensor, n_want: int,
-                logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                logits_out: Optional[torch.Tensor] = None, probe=None) -> torch.Tensor:
         """Run the step's tokens through every scheduled layer; return float32 logits
         `[n_want, vocab]` of the rows `want_rows` (indices into the packed tokens), in
-        `logits_out` when given, else in a tensor of their own."""
+        `logits_out` when given, else in a tensor of their own.
+
+        `probe(name, tensor)`, when given, is called with the residual rows after the
+        embedding ("embed"), after each scheduled layer's mixer and feed-forward
+        ("L{i}.post_mixer", "L{i}.post_ffn", i the place in the run order), and with the
+        normed wanted rows ("final_norm") and the logits ("logits"): the reference's probe
+        names (crates/braidinfer-runtime/src/tracer.rs:94-160).  The tensors are the
+        step's own buffers: a probe that keeps one copies it."""
         rt = self.rt
         T, H = step.n_tokens, self.spec.hidden_size
         ws = step.ws
+        step.probe = probe
         x = ws.get("residual", (T, H), torch.float32)
         self.embedding.forward(step.tokens, x)
         step.position_data = {}
         for name, enc in self.positions.items():
             step.position_data[name] = enc.prepare(step)
             enc.add_to_embedding(x, step)
+        if probe is not None:
+            probe("embed", x)
         step.prepared_norm = None
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
+            step.schedule_index = i
             # the norm that reads the residual rows after this layer: the next scheduled layer's first
             # (the final norm reads chosen rows only and is left alone)
             step.norm_after_layer = None
             if i + 1 < len(self.schedule):
-                nxt = self.layers[self.schedule[i + 1].layer]
-                step.norm_after_layer = nxt.mixer_norm if nxt.mixer is not None else nxt.ffn_norm
+                step.norm_after_layer = self.layers[self.schedule[i + 1].layer].first_norm()
             ctx = MixerContext(unit=e.cache, writes_cache=e.writes_cache)
             if layer.mixer is not None:
                 if e.cache is not None and e.cache in cache.group_of_unit:
                     g = cache.unit_group(e.cache)
-                    ctx.storage, ctx.block_table, ctx.page_tokens = g.storage[e.cache], g.table_dev, g.page_tokens
+                    ctx.storage, ctx.block_table, ctx.page_tokens = g.storage_view(e.cache), g.table_dev, g.page_tokens
+                    ctx.keys, ctx.values = g.keys(e.cache), g.values(e.cache)
                 ctx.state = cache.state(("entry", i))
             layer.run(layer, x, step, ctx)
         if logits_out is None:
@@ -169,5 +213,9 @@ class DecoderModel:
             return logits
         hn = ws.get("final_h", (n_want, H), rt.dtype)
         self.final_norm.forward(x, hn, rows=want_rows)
+        if probe is not None:
+            probe("final_norm", hn)
         self.lm_head.forward(hn, logits, ws)
+        if probe is not None:
+            probe("logits", logits)
         return logits

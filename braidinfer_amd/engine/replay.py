@@ -10,7 +10,10 @@ Input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
 For a step with wanted places, `<out>/<step>.f32` holds float32 little-endian logits
 [wanted, vocab] in the order of the entries and of `want`.  After every step a line
-`done <step>` is printed and flushed.
+`done <step>` is printed and flushed.  With `--probes` a step also leaves
+`<out>/<step>.probes.json`, statistics of the activations at the reference's probe points
+(crates/braidinfer-runtime/src/tracer.rs:94-160: embed, L{i}.post_mixer, L{i}.post_ffn,
+final_norm, logits).
 """
 from __future__ import annotations
 
@@ -26,12 +29,24 @@ from ..errors import BraidError, StepError
 from .engine import Engine, StepEntry
 
 
+def probe_stats(t) -> dict:
+    """What the reference's `trace_dump` prints of a probed tensor (bin/trace_dump.rs:49-117):
+    its size, mean, root mean square, largest magnitude and first values."""
+    f = t.detach().float()
+    n = f.numel()
+    if n == 0:
+        return {"shape": list(t.shape), "mean": 0.0, "rms": 0.0, "absmax": 0.0, "head": []}
+    return {"shape": list(t.shape), "mean": float(f.mean()), "rms": float(f.pow(2).mean().sqrt()),
+            "absmax": float(f.abs().max()), "head": [float(v) for v in f.reshape(-1)[:8].tolist()]}
+
+
 class Replayer:
-    def __init__(self, engine: Engine, out_dir: str):
+    def __init__(self, engine: Engine, out_dir: str, probes: bool = False):
         self.engine = engine
         self.out_dir = out_dir
         os.makedirs(out_dir, exist_ok=True)
         self.slot_of: Dict[str, int] = {}
+        self.probes = probes
 
     def run_step(self, obj: dict) -> None:
         step_no = obj["step"]
@@ -45,7 +60,12 @@ class Replayer:
                     fresh.append(rid)
                 entries.append(StepEntry(self.slot_of[rid], e["tokens"], e.get("want", [])))
             if entries:
-                logits = self.engine.step(entries)
+                stats = {}
+                logits = self.engine.step(entries, probe=(lambda name, t: stats.__setitem__(name, probe_stats(t)))
+                                          if self.probes else None)
+                if self.probes:
+                    with open(os.path.join(self.out_dir, f"{step_no}.probes.json"), "w") as f:
+                        json.dump(stats, f, indent=1)
                 if logits.shape[0] > 0:
                     arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                     tmp = os.path.join(self.out_dir, f".{step_no}.f32.tmp")
@@ -80,11 +100,14 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--probes", action="store_true",
+                    help="also write <step>.probes.json: statistics of the residual rows after the embedding, after "
+                         "every layer's mixer and feed-forward, of the final norm and the logits")
     args = ap.parse_args(argv)
     try:
         engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device,
                                     max_tokens=max(args.max_tokens, 64))
-        Replayer(engine, args.out).run(sys.stdin, sys.stdout)
+        Replayer(engine, args.out, probes=args.probes).run(sys.stdin, sys.stdout)
     except BraidError as e:
         print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr, flush=True)
         return 1

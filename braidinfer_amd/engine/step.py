@@ -40,7 +40,7 @@ class StepBatch:
     n_tokens: int                    # T: tokens in this step (padding included)
     n_seqs: int                      # B: sequences (padding included)
     tokens: torch.Tensor             # [T] token ids
-    positions: torch.Tensor          # [T] position of each token in its sequence
+    positions: torch.Tensor          # [T] place of each token in its sequence (its index in the cache)
     seq_of_token: torch.Tensor       # [T] index into the batch
     cu_seqlens: torch.Tensor         # [B + 1] offsets of the sequences' tokens
     slots: torch.Tensor              # [B] cache slot of each sequence, -1 = padding
@@ -60,12 +60,24 @@ class StepBatch:
     norm_after_layer: Any = None
     prepared_norm: Any = None
     extras: Dict[str, Any] = field(default_factory=dict)     # per-step scratch of parts (keyed by them)
+    # what the position encodings read: [T], the same tensor as `positions` unless the caller gave
+    # position numbers of its own, which may be k per token: [T, k]
+    position_ids: Optional[torch.Tensor] = None
+    probe: Any = None                # probe(name, tensor) of the running step, or None
+    schedule_index: int = 0          # place in the run order of the layer that is running
+
+    def __post_init__(self):
+        if self.position_ids is None:
+            self.position_ids = self.positions
 
 
 def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts: Sequence[int],
-              device, ws: Workspace, pad_seqs: int = 0) -> StepBatch:
+              device, ws: Workspace, pad_seqs: int = 0, position_ids: Optional[Sequence] = None) -> StepBatch:
     """Build the device arrays of a step in one host-to-device copy.  `pad_seqs` extra
-    sequences of one dummy token (slot -1, position 0) may follow the real ones."""
+    sequences of one dummy token (slot -1, position 0) may follow the real ones.
+    `position_ids`: per sequence the position numbers of its tokens for the position
+    encodings, one integer or k integers per token (the same k for all); None: each token's
+    place in its sequence."""
     B = len(slots) + pad_seqs
     new = [len(t) for t in token_lists] + [1] * pad_seqs
     T = sum(new)
@@ -79,8 +91,16 @@ def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts
     pos = np.arange(T, dtype=np.int64) - cu[sot] + starts_a[sot]
     toks = np.concatenate([np.asarray(t, dtype=np.int64) for t in token_lists] + [np.zeros(pad_seqs, dtype=np.int64)])
     ctx = np.where(np.asarray(all_slots) >= 0, starts_a + new_a, 0)
-    # layout of the one int32 staging array: tokens | positions | seq_of_token | cu | slots | ctx
-    flat = np.concatenate([toks, pos, sot, cu, np.asarray(all_slots, dtype=np.int64), ctx]).astype(np.int32)
+    pid = np.zeros(0, dtype=np.int64)
+    k = 0
+    if position_ids is not None:
+        rows = [np.asarray(p, dtype=np.int64).reshape(len(t), -1) for p, t in zip(position_ids, token_lists)]
+        k = rows[0].shape[1]
+        if any(r.shape[1] != k for r in rows) or k == 0:
+            raise ValueError("position_ids: every token needs the same number of position numbers")
+        pid = np.concatenate(rows + [np.zeros((pad_seqs, k), dtype=np.int64)]).reshape(-1)
+    # layout of the one int32 staging array: tokens | positions | seq_of_token | cu | slots | ctx | position ids
+    flat = np.concatenate([toks, pos, sot, cu, np.asarray(all_slots, dtype=np.int64), ctx, pid]).astype(np.int32)
     dev = torch.from_numpy(flat).to(device)
     o = 0
 
@@ -91,9 +111,13 @@ def pack_step(slots: Sequence[int], token_lists: Sequence[Sequence[int]], starts
         return v
     tokens, positions, seq_of_token = take(T), take(T), take(T)
     cu_seqlens, slots_d, ctx_d = take(B + 1), take(B), take(B)
+    pid_d = None
+    if k:
+        pid_d = take(T * k)
+        pid_d = pid_d if k == 1 else pid_d.view(T, k)
     max_ctx = int(ctx.max()) if B else 0
     return StepBatch(
         n_tokens=T, n_seqs=B, tokens=tokens, positions=positions, seq_of_token=seq_of_token,
         cu_seqlens=cu_seqlens, slots=slots_d, ctx_lens=ctx_d, host_slots=all_slots, host_new=new,
         host_start=all_starts, is_decode=all(n == 1 for n in new), max_new=max(new) if new else 0,
-        max_ctx=max_ctx, max_ctx_bound=max_ctx, ws=ws)
+        max_ctx=max_ctx, max_ctx_bound=max_ctx, ws=ws, position_ids=pid_d)

@@ -18,10 +18,13 @@ import torch
 
 from .. import kernels as K
 from ..cache import CacheNeed
-from ..errors import ConfigError
+from ..errors import ConfigError, StepError
 from ..weights import TensorSpec
 from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
 from .linear import fused_layout, linear, stream_layout
+
+
+MAX_HEAD_DIM = 512      # attention_simple's limit; the matrix-core kernels take up to 256 in steps of 16
 
 
 def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
@@ -47,6 +50,9 @@ class GQAAttention(Mixer):
             raise ConfigError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if head_dim <= 0 or head_dim % 2:
             raise ConfigError(f"attention: head_dim {head_dim} must be positive and even")
+        if head_dim > MAX_HEAD_DIM:
+            raise ConfigError(f"attention: head_dim {head_dim} is beyond what any attention kernel of this library "
+                              f"takes ({MAX_HEAD_DIM})")
         self.H, self.nq, self.nkv, self.hd = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
         self.window = None if window is None else int(window)
         self.position = position
@@ -54,6 +60,7 @@ class GQAAttention(Mixer):
         if not self.scale > 0:
             raise ConfigError(f"attention: the score scale must be positive, not {self.scale}")
         self.w_qkv = self.w_o = None
+        self._expects_tables = False       # set by check_positions when the model is put together
         self.force_simple = False          # tests set it to run the one-wave-per-query kernel in bf16
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
@@ -72,6 +79,19 @@ class GQAAttention(Mixer):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv_heads=self.nkv, head_dim=self.hd, window=self.window)
 
+    def check_positions(self, encodings) -> None:
+        if self.position is None:
+            return
+        enc = encodings.get(self.position)
+        if enc is None:
+            raise ConfigError(f"attention asks for the position encoding {self.position!r}, the model has "
+                              f"{sorted(encodings)}; name one of them, or None for attention without positions")
+        if getattr(enc, "gives", None) not in ("rotary", "embedding", "none"):
+            raise ConfigError(f"attention cannot use the position encoding {self.position!r}: it gives "
+                              f"{getattr(enc, 'gives', None)!r}, attention rotates with 'rotary' tables or takes "
+                              "'embedding' / 'none' encodings, which leave queries and keys alone")
+        self._expects_tables = enc.gives == "rotary"
+
     def forward(self, h, x, step, ctx: MixerContext) -> None:
         T = step.n_tokens
         nq, nkv, hd = self.nq, self.nkv, self.hd
@@ -79,8 +99,9 @@ class GQAAttention(Mixer):
         qkv = step.ws.get("attn_qkv", (T, (nq + 2 * nkv) * hd), dt)
         linear(h, self.w_qkv, qkv, step.ws)
         tables = step.position_data.get(self.position) if self.position else None
-        if tables is not None and not isinstance(tables, RotaryTables):
-            tables = None
+        if (tables is None and self._expects_tables) or (tables is not None and not isinstance(tables, RotaryTables)):
+            raise StepError(f"attention: the position encoding {self.position!r} gave {type(tables).__name__}, "
+                            "rotary tables were expected")
         if self._fused_decode(qkv, tables, step, ctx):
             return self._finish(qkv, x, step, ctx, tables, True)
         K.rope_kv_write(qkv, tables.cos if tables else None, tables.sin if tables else None,

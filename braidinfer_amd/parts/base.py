@@ -126,8 +126,13 @@ class NormedInput:
 
 
 class PositionEncoding(Part):
+    # what the encoding gives the mixers that name it: "rotary" (`prepare` returns
+    # `RotaryTables`), "embedding" (it acts on the embeddings only) or "none"
+    gives = "none"
+
     def prepare(self, step) -> Any:
-        """Called once per step before the layers; the result is kept in
+        """Called once per step before the layers, with the step's `position_ids` (int32 [T],
+        or [T, k] when the caller gives k numbers per token); the result is kept in
         `step.position_data[name]` for the mixers."""
         return None
 
@@ -149,6 +154,11 @@ class Mixer(Part):
     def cache_need(self) -> Optional[CacheNeed]:
         return None
 
+    def check_positions(self, encodings: Dict[str, "PositionEncoding"]) -> None:
+        """Called once when the model is put together, with its position encodings by name:
+        a mixer that asks for one raises `ConfigError` here if it is absent or of a kind the
+        mixer cannot use, instead of running without positions later."""
+
     def state_need(self) -> Optional[StateNeed]:
         return None
 
@@ -162,7 +172,9 @@ class MixerContext:
     """What one schedule entry hands its mixer: its cache unit and state, if it asked."""
 
     unit: Optional[int] = None
-    storage: Optional[torch.Tensor] = None        # [pages, 2, kv_heads, page_tokens, head_dim]
+    storage: Optional[torch.Tensor] = None        # [pages, 2, kv_heads, page_tokens, head_dim] (equal key and value widths)
+    keys: Optional[torch.Tensor] = None           # [pages, kv_heads, page_tokens * key width], a view of the same memory
+    values: Optional[torch.Tensor] = None         # [pages, kv_heads, page_tokens * value width]
     block_table: Optional[torch.Tensor] = None    # int32 [slots, pages per sequence], device
     page_tokens: int = 0
     writes_cache: bool = True

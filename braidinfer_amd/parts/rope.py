@@ -14,12 +14,13 @@ from typing import Dict
 import torch
 
 from .. import kernels as K
-from ..errors import ConfigError
+from ..errors import ConfigError, StepError
 from .base import PositionEncoding, RotaryTables, Runtime, register_part
 
 
 class RotaryEncoding(PositionEncoding):
     graph_safe = True
+    gives = "rotary"
 
     def __init__(self, rotary_dim: int, theta: float, pairing: str = "half"):
         if rotary_dim <= 0 or rotary_dim % 2:
@@ -36,10 +37,12 @@ class RotaryEncoding(PositionEncoding):
         self.inv_freq = inv.to(torch.float32).to(rt.device)
 
     def prepare(self, step) -> RotaryTables:
+        if step.position_ids.dim() != 1:
+            raise StepError(f"rotary encoding takes one position per token, the step brings {tuple(step.position_ids.shape)}")
         P = self.rotary_dim // 2
         cos = step.ws.get(f"rope_cos_{id(self)}", (step.n_tokens, P), torch.float32)
         sin = step.ws.get(f"rope_sin_{id(self)}", (step.n_tokens, P), torch.float32)
-        K.rope_table(step.positions, self.inv_freq, cos, sin)
+        K.rope_table(step.position_ids, self.inv_freq, cos, sin)
         return RotaryTables(cos, sin, self.rotary_dim, self.pairing == "adjacent")
 
 

@@ -116,3 +116,39 @@ def test_registering_another_architecture():
     finally:
         unregister_architecture("ToyForCausalLM")
     assert "ToyForCausalLM" not in registered_architectures()
+
+
+def test_a_head_size_no_kernel_takes_is_refused_when_the_configuration_is_read():
+    d = dict(TINY["a"], head_dim=512)
+    assert B.MistralConfig.from_dict(d).head_dim == 512
+    with pytest.raises(B.ConfigError, match="head_dim 514"):
+        B.MistralConfig.from_dict(dict(d, head_dim=514))
+    with pytest.raises(B.ConfigError, match="head_dim 1024"):
+        B.preset("tiny-a", head_dim=1024)
+
+
+def test_stop_tokens_of_generation_config_json(tmp_path):
+    from braidinfer_amd.config import generation_stop_tokens
+    assert generation_stop_tokens(str(tmp_path)) == []
+    (tmp_path / "generation_config.json").write_text('{"bos_token_id": 1, "eos_token_id": 2}')
+    assert generation_stop_tokens(str(tmp_path)) == [2]
+    (tmp_path / "generation_config.json").write_text('{"eos_token_id": [2, 7, 9]}')
+    assert generation_stop_tokens(str(tmp_path)) == [2, 7, 9]
+    (tmp_path / "generation_config.json").write_text('{"temperature": 0.7}')
+    assert generation_stop_tokens(str(tmp_path)) == []
+    (tmp_path / "generation_config.json").write_text('{"eos_token_id": "</s>"}')
+    with pytest.raises(B.ConfigError, match="eos_token_id"):
+        generation_stop_tokens(str(tmp_path))
+
+
+def test_a_layer_names_its_norms_by_role_and_its_tensors_by_the_builder():
+    spec = B.spec_of(B.MistralConfig.from_dict(TINY["a"]))
+    layer = spec.layers[1]
+    assert sorted(layer.norms) == ["feed_forward", "mixer"] and layer.block == "prenorm_residual"
+    assert list(layer.names) == ["norm.mixer", "mixer", "norm.feed_forward", "feed_forward"]
+    assert layer.name_of("norm.feed_forward") == "model.layers.1.post_attention_layernorm."
+    with pytest.raises(KeyError):
+        layer.name_of("norm.post_mixer")
+    # nothing in the neutral description carries a checkpoint's names of its own
+    bare = B.LayerSpec("p.")
+    assert bare.names == {} and bare.norms == {} and bare.mixer is None

@@ -534,3 +534,72 @@ def test_configurations_drawn_at_random(seed, tmp_path):
             eng.free_slot(sl)
         close(first, ref[9:29], dtype, f"{cfg_d}: 20 prompts of 10 to 29 tokens in one step")
         close(then, ref[10:30], dtype, f"{cfg_d}: one token each after them")
+
+
+# ----------------------------------------------------------------- probes, failed steps ----
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_probes_see_the_residual_rows_where_the_plain_implementation_has_them(engines, tiny_folders, dtype):
+    """`step(..., probe=)` hands out the residual rows under the reference's probe names
+    (tracer.rs:94-160), for a whole prompt and for single-token steps (which then run eagerly
+    instead of from a graph), and leaves the logits as they are without a probe."""
+    _, cfg, w = tiny_folders["b"]
+    eng = engines("b", dtype)
+    sz = P.sizes(cfg)
+    toks = tokens(cfg, 21, 50)
+    x = P.embedding(w["model.embed_tokens.weight"], toks)
+    want = {"embed": x}
+    for i in range(sz["L"]):
+        p = f"model.layers.{i}."
+        x = P.attention_block(x, np.arange(len(toks)), w, p, sz, P.layer_window(sz, i))
+        want[f"L{i}.post_mixer"] = x
+        x = P.ffn_block(x, w, p, sz)
+        want[f"L{i}.post_ffn"] = x
+    want["final_norm"] = P.rms_norm(x, w["model.norm.weight"], sz["eps"])
+    want["logits"] = P.forward(cfg, w, toks)
+    seen = {}
+    s = eng.alloc_slot()
+    first = eng.step([StepEntry(s, toks[:20], list(range(20)))], probe=lambda n, t: seen.setdefault(n, t.float().cpu().numpy().copy()))
+    assert list(seen) == list(want)
+    for n in want:
+        close(seen[n], want[n][:20], dtype, n)
+    assert np.array_equal(seen["logits"], first.cpu().numpy())
+    one = {}
+    last = eng.step([StepEntry(s, toks[20:], [0])], probe=lambda n, t: one.setdefault(n, t.float().cpu().numpy().copy()))
+    eng.free_slot(s)
+    for n in want:
+        close(one[n], want[n][20:], dtype, n + " of a single-token step")
+    s = eng.alloc_slot()
+    eng.step([StepEntry(s, toks[:20], [])])
+    plain_last = eng.step([StepEntry(s, toks[20:], [0])])           # no probe: the recorded graph
+    eng.free_slot(s)
+    assert np.abs(plain_last.cpu().numpy() - last.cpu().numpy()).max() <= CUT_TOL[dtype] * np.abs(want["logits"]).max()
+
+
+def test_a_step_that_fails_inside_the_model_leaves_nothing_behind(tiny_folders):
+    folder, cfg, w = tiny_folders["a"]
+    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=512)
+    s1, s2 = eng.alloc_slot(), eng.alloc_slot()
+    toks = tokens(cfg, 130, 3)
+    eng.step([StepEntry(s1, toks[:70], [])])
+    free = [g.pool.free_count for g in eng.cache.groups]
+    real = eng.model.forward
+
+    def broken(*a, **k):
+        raise B.KernelError("a size no kernel takes")
+    eng.model.forward = broken
+    with pytest.raises(B.KernelError):
+        eng.step([StepEntry(s1, toks[70:], [0]), StepEntry(s2, toks[:100], [0])])     # needs three new pages
+    eng.model.forward = real
+    assert [g.pool.free_count for g in eng.cache.groups] == free and eng.length(s1) == 70 and eng.length(s2) == 0
+    got = eng.step([StepEntry(s1, toks[70:], list(range(60)))]).cpu().numpy()         # and the sequence goes on as if nothing happened
+    close(got, P.forward(cfg, w, toks)[70:], "float32", "after a failed step")
+    eng.free_slot(s1); eng.free_slot(s2)
+    assert all(g.pool.held_count == 0 for g in eng.cache.groups)
+
+
+def test_the_longest_sequence_is_the_models_unless_the_caller_says_more(tiny_folders):
+    folder, cfg, _ = tiny_folders["c"]                     # max_position_embeddings 2048
+    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=8192)
+    assert eng.cache.max_seq_len == 2048
+    assert B.Engine.from_folder(folder, dtype="float32", max_tokens=8192, max_seq_len=4096).cache.max_seq_len == 4096
+    assert B.Engine.from_folder(folder, dtype="float32", max_tokens=640).cache.max_seq_len == 640

@@ -88,6 +88,67 @@ def test_command_line(tiny_folders):
     assert r.returncode == 2 and "tokenizer" in r.stderr
 
 
+def _word_tokenizer(folder, vocab_size, bos):
+    """A tokenizer.json made here with the `tokenizers` package: one token per word."""
+    tk = pytest.importorskip("tokenizers")
+    words = {f"w{i}": i for i in range(vocab_size)}
+    words["<s>"] = bos
+    del words[f"w{bos}"]
+    tok = tk.Tokenizer(tk.models.WordLevel(vocab=words, unk_token="w0"))
+    tok.pre_tokenizer = tk.pre_tokenizers.WhitespaceSplit()
+    tok.decoder = tk.decoders.Fuse()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    return tok
+
+
+def test_command_line_with_text_a_tokenizer_and_the_folders_stop_tokens(tmp_path):
+    """The text path: the prompt is tokenized with the folder's tokenizer.json, the BOS of
+    config.json goes in front unless tokenizer_config.json says no (generate.rs:479-489), the
+    stop tokens come from config.json and generation_config.json, the answer is text."""
+    import json
+    import shutil
+    cfg = B.preset("tiny-a", bos_token_id=1, eos_token_id=250)
+    folder = B.Engine.write_random_folder(str(tmp_path / "m"), cfg, seed=31, std=0.08)
+    _word_tokenizer(folder, 256, bos=1)
+    pc, w = P.read_folder(folder)
+    ids = [7, 3, 200, 5]
+    text = " ".join(f"w{i}" for i in ids)
+    free_run = P.greedy_generate(pc, w, [1] + ids, 8)
+    stop = free_run[3]
+    with open(os.path.join(folder, "generation_config.json"), "w") as f:
+        json.dump({"eos_token_id": [stop, 251]}, f)
+    gen = [sys.executable, os.path.join(ROOT, "bin", "generate"), "--dtype", "float32"]
+    env = dict(os.environ, MODEL=folder, MAX_TOKENS="8")
+    r = subprocess.run(gen + [text], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    want = P.greedy_generate(pc, w, [1] + ids, 8, stop_ids=[250, stop, 251])
+    assert 0 < len(want) <= 3 and r.stdout.strip() == "".join(f"w{t}" for t in want)
+    assert f"stop tokens: [250, {stop}, 251]" in r.stderr and "LOAD PROFILE:" in r.stderr and "GB/s" in r.stderr
+    # no BOS when the tokenizer's configuration says so
+    with open(os.path.join(folder, "tokenizer_config.json"), "w") as f:
+        json.dump({"add_bos_token": False}, f)
+    os.remove(os.path.join(folder, "generation_config.json"))
+    r = subprocess.run(gen + [text], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    assert r.stdout.strip() == "".join(f"w{t}" for t in P.greedy_generate(pc, w, ids, 8, stop_ids=[250]))
+    shutil.rmtree(folder)
+
+
+def test_command_line_writes_a_random_folder_in_shards_and_reads_it_again(tmp_path):
+    keep = str(tmp_path / "kept")
+    gen = [sys.executable, os.path.join(ROOT, "bin", "generate"), "--dtype", "float32", "--prompt-ids", "9,8,7"]
+    env = {k: v for k, v in os.environ.items() if k != "MODEL"}
+    env["MAX_TOKENS"] = "5"
+    r1 = subprocess.run(gen + ["--random-weights", "3", "--preset", "tiny-b", "--save-folder", keep, "--shard-bytes", "40000"],
+                        env=env, capture_output=True, text=True)
+    assert r1.returncode == 0, r1.stderr
+    assert os.path.isfile(os.path.join(keep, "model.safetensors.index.json")) and "written to" in r1.stderr
+    r2 = subprocess.run(gen, env=dict(env, MODEL=keep), capture_output=True, text=True)
+    assert r2.returncode == 0 and r2.stdout == r1.stdout
+    pc, w = P.read_folder(keep)
+    assert [int(t) for t in r1.stdout.split()] == P.greedy_generate(pc, w, [9, 8, 7], 5)
+
+
 def test_smoke_entry():
     import __graft_entry__
     __graft_entry__.smoke()

@@ -26,6 +26,7 @@ class FakeEngine:
     def __init__(self, n_pages=32, **kw):
         self.cache = FakeCache(n_pages, **kw)
         self.spec = FakeSpec()
+        self.stop_token_ids = list(self.spec.stop_token_ids)
         self.vocab_size = 50
         self.device = "cpu"
         self.live = {}

@@ -12,14 +12,17 @@ import braidinfer_amd as B
 import plain_mistral as P
 from braidinfer_amd import StepEntry
 from braidinfer_amd.cache import SequenceCache, StateNeed
-from braidinfer_amd.config import (LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture,
+from braidinfer_amd.config import (LayerSpec, ModelSpec, PartSpec, ScheduleEntry, prenorm_layer, register_architecture,
                                    unregister_architecture)
 from braidinfer_amd.engine import Workspace, pack_step
-from braidinfer_amd.parts import (Mixer, MixerContext, Runtime, build_part, register_part, unregister_part)
+from braidinfer_amd.parts import (Mixer, MixerContext, RotaryTables, Runtime, build_part, register_part, unregister_part)
 from braidinfer_amd.weights import TensorSpec
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
+# the tensor-name pieces the toy models below use for the common layer
+NAMES = dict(mixer_name="self_attn.", feed_forward_name="mlp.", mixer_norm_name="input_layernorm.",
+             ffn_norm_name="post_attention_layernorm.")
 
 
 def rt(dtype):
@@ -115,7 +118,7 @@ def test_attention_part_with_its_cache(dtype, window):
         step = pack_step([slot], [[1] * (hi - lo)], [lo], DEV, Workspace(DEV))
         step.position_data = {"rope": rope.prepare(step)}
         g = cache.unit_group(0)
-        ctx = MixerContext(unit=0, storage=g.storage[0], block_table=g.table_dev, page_tokens=g.page_tokens)
+        ctx = MixerContext(unit=0, storage=g.storage_view(0), block_table=g.table_dev, page_tokens=g.page_tokens)
         x = dev(x0[lo:hi])
         part.forward(dev(h[lo:hi], dtype), x, step, ctx)
         cache.commit([slot], [hi - lo])
@@ -191,8 +194,8 @@ def toy_spec(cfg):
     attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
                                       "window": None, "position": "rope"})
     layers = [
-        LayerSpec("toy.layers.0.", PartSpec("running_sum", {"hidden_size": H}), None, norm, None),
-        LayerSpec("toy.layers.1.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 56}), norm, norm),
+        prenorm_layer("toy.layers.0.", PartSpec("running_sum", {"hidden_size": H}), None, norm, None, **NAMES),
+        prenorm_layer("toy.layers.1.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 56}), norm, norm, **NAMES),
     ]
     return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=cfg.vocab_size,
                      embedding=PartSpec("embedding", {"vocab_size": cfg.vocab_size, "hidden_size": H}),
@@ -270,7 +273,7 @@ def loop_spec(cfg):
     norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
     attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 1, "head_dim": 16,
                                       "window": None, "position": "rope"})
-    layers = [LayerSpec(f"m.layers.{i}.", attn, None, norm, None) for i in range(2)]
+    layers = [prenorm_layer(f"m.layers.{i}.", attn, None, norm, None, **NAMES) for i in range(2)]
     if cfg.mode == "twice":       # layer 0, layer 1, layer 0 again with a cache of its own
         schedule = [ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(0, 2)]
     else:                         # layer 1 reads the keys and values layer 0 stored, and stores none
@@ -370,6 +373,7 @@ class Top1Experts(FeedForward):
 
 class LearnedPositions(PositionEncoding):
     """A table of position vectors added to the embeddings (no rotation anywhere)."""
+    gives = "embedding"
 
     def __init__(self, max_positions, hidden_size):
         self.P, self.H = max_positions, hidden_size
@@ -402,8 +406,8 @@ def routed_spec(cfg):
     norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
     attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 3, "head_dim": 16,
                                       "window": None, "position": None})          # attention without rotation
-    layers = [LayerSpec("r.layers.0.", attn, PartSpec("top1_experts", {"hidden_size": H, "expert_size": 24}), norm, norm),
-              LayerSpec("r.layers.1.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 64}), norm, norm)]
+    layers = [prenorm_layer("r.layers.0.", attn, PartSpec("top1_experts", {"hidden_size": H, "expert_size": 24}), norm, norm, **NAMES),
+              prenorm_layer("r.layers.1.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 64}), norm, norm, **NAMES)]
     return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=60,
                      embedding=PartSpec("embedding", {"vocab_size": 60, "hidden_size": H}), layers=layers,
                      schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1)], final_norm=norm,
@@ -465,3 +469,333 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path, dtype):
         unregister_architecture("ToyRoutedForCausalLM")
         unregister_part("feed_forward", "top1_experts")
         unregister_part("position", "learned_positions")
+
+
+# ------------------------------ four norms a layer, arranged by a function from outside ----
+@dataclass(frozen=True)
+class SandwichConfig:
+    architecture = "ToySandwichForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls()
+
+    def to_dict(self):
+        return {"architectures": [self.architecture]}
+
+
+def sandwich(layer, x, step, ctx):
+    """x += post_norm(part(pre_norm(x))) for the mixer, then for the feed-forward: the parts add
+    into a zeroed buffer instead of the residual rows, and a second norm stands behind each."""
+    for part, pre, post, extra in ((layer.mixer, "mixer", "post_mixer", (ctx,)),
+                                   (layer.feed_forward, "feed_forward", "post_feed_forward", ())):
+        h = torch.empty(x.shape, dtype=layer.rt.dtype, device=x.device)
+        layer.norms[pre].forward(x, h)
+        y = torch.zeros_like(x)
+        part.forward(h, y, step, *extra)
+        yn = torch.empty_like(x)
+        layer.norms[post].forward(y, yn)
+        x += yn
+
+
+SANDWICH_NAMES = {"norm.mixer": "ln1.", "mixer": "attn.", "norm.post_mixer": "ln2.", "norm.feed_forward": "ln3.",
+                  "feed_forward": "ffn.", "norm.post_feed_forward": "ln4."}
+
+
+def sandwich_spec(cfg):
+    H = 64
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                      "window": None, "position": "rope"})
+    ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 96})
+    roles = {r: norm for r in ("mixer", "post_mixer", "feed_forward", "post_feed_forward")}
+    layers = [LayerSpec(f"s.layers.{i}.", attn, ffn, norms=roles, block="sandwich", names=SANDWICH_NAMES) for i in range(2)]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=80,
+                     embedding=PartSpec("embedding", {"vocab_size": 80, "hidden_size": H}), layers=layers,
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1)], final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": 80, "hidden_size": H, "tied_to": None}),
+                     positions={"rope": PartSpec("rope", {"rotary_dim": 16, "theta": 1e4, "pairing": "half"})},
+                     max_position_embeddings=256, embedding_prefix="s.embed.", final_norm_prefix="s.norm.",
+                     lm_head_prefix="s.head.")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_with_four_norms_arranged_from_outside(tmp_path, dtype):
+    register_part("block", "sandwich", lambda: sandwich)
+    register_architecture("ToySandwichForCausalLM", SandwichConfig, sandwich_spec)
+    try:
+        folder = B.Engine.write_random_folder(str(tmp_path / "s"), SandwichConfig(), seed=3, std=0.2, vector_jitter=0.3)
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=256)
+        _, w = P.read_folder(folder)
+        assert all(f"s.layers.1.ln{i}.weight" in w for i in (1, 2, 3, 4)) and "s.layers.0.attn.q_proj.weight" in w
+        sz = dict(nq=4, nkv=2, hd=16)
+
+        def plain(toks):
+            T = len(toks)
+            x = P.embedding(w["s.embed.weight"], toks)
+            inv = P.rope_inv_freq(16, 1e4)
+            for l in range(2):
+                p = f"s.layers.{l}."
+                n = P.rms_norm(x, w[p + "ln1.weight"], 1e-5)
+                q, k, v = (P.linear(n, w[p + f"attn.{m}_proj.weight"]).reshape(T, -1, 16) for m in "qkv")
+                q, k = P.rope(q, np.arange(T), inv, "half"), P.rope(k, np.arange(T), inv, "half")
+                a = P.linear(P.attention(q, k, v, 4, 2).reshape(T, 64), w[p + "attn.o_proj.weight"])
+                x = x + P.rms_norm(a, w[p + "ln2.weight"], 1e-5)
+                n = P.rms_norm(x, w[p + "ln3.weight"], 1e-5)
+                f = P.swiglu(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+                x = x + P.rms_norm(f, w[p + "ln4.weight"], 1e-5)
+            return P.linear(P.rms_norm(x, w["s.norm.weight"], 1e-5), w["s.head.weight"])
+
+        toks = [int(t) for t in np.random.default_rng(5).integers(0, 80, 70)]
+        ref = plain(toks)
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, toks[:66], list(range(66)))]).cpu().numpy()]
+        for t in toks[66:]:
+            got.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+        eng.free_slot(s)
+        got = np.concatenate(got)
+        assert np.abs(got - ref).max() < (1e-4 if dtype == "float32" else 4e-2) * np.abs(ref).max()
+    finally:
+        unregister_architecture("ToySandwichForCausalLM")
+        unregister_part("block", "sandwich")
+
+
+# ------------------------------------- a rotary encoding with two position numbers a token ----
+class TwoSectionRotary(B.parts.PositionEncoding):
+    """The lower half of the frequencies turns with a token's first position number, the upper
+    half with its second (as encodings with sectioned positions do)."""
+    gives = "rotary"
+
+    def __init__(self, rotary_dim, theta):
+        self.rd, self.theta = rotary_dim, theta
+
+    def load(self, tensors, prefix, rt):
+        self.rt = rt
+        self.inv = torch.tensor(P.rope_inv_freq(self.rd, self.theta), device=rt.device)
+
+    def prepare(self, step):
+        ids = step.position_ids
+        assert ids.dim() == 2 and ids.shape[1] == 2, "two position numbers per token"
+        half = self.rd // 4
+        which = torch.cat([ids[:, :1].expand(-1, half), ids[:, 1:].expand(-1, self.rd // 2 - half)], 1).float()
+        th = which * self.inv[None, :]
+        return RotaryTables(torch.cos(th).contiguous(), torch.sin(th).contiguous(), self.rd, False)
+
+
+@dataclass(frozen=True)
+class SectionConfig:
+    architecture = "ToySectionForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls()
+
+    def to_dict(self):
+        return {"architectures": [self.architecture]}
+
+
+def section_spec(cfg):
+    H = 48
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 1, "head_dim": 16,
+                                      "window": None, "position": "sections"})
+    layers = [prenorm_layer("t.layers.0.", attn, PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 64}), norm, norm,
+                            **NAMES)]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=70,
+                     embedding=PartSpec("embedding", {"vocab_size": 70, "hidden_size": H}), layers=layers,
+                     schedule=[ScheduleEntry(0, 0)], final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": 70, "hidden_size": H, "tied_to": None}),
+                     positions={"sections": PartSpec("two_section_rotary", {"rotary_dim": 16, "theta": 1e4})},
+                     max_position_embeddings=256, embedding_prefix="t.embed.", final_norm_prefix="t.norm.",
+                     lm_head_prefix="t.head.")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_position_numbers_of_the_callers_own_two_a_token(tmp_path, dtype):
+    register_part("position", "two_section_rotary", TwoSectionRotary)
+    register_architecture("ToySectionForCausalLM", SectionConfig, section_spec)
+    try:
+        folder = B.Engine.write_random_folder(str(tmp_path / "t"), SectionConfig(), seed=9, std=0.2)
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=256)
+        _, w = P.read_folder(folder)
+        toks = [int(t) for t in np.random.default_rng(6).integers(0, 70, 40)]
+        T = len(toks)
+        ids = [(t, 5 + t // 3) for t in range(T)]
+
+        inv = P.rope_inv_freq(16, 1e4)
+        th = np.where(np.arange(8)[None, :] < 4, np.array([i[0] for i in ids], np.float32)[:, None],
+                      np.array([i[1] for i in ids], np.float32)[:, None]).astype(np.float32) * inv[None, :]
+
+        def rot(x):
+            c, s_ = np.cos(th).astype(np.float32)[:, None, :], np.sin(th).astype(np.float32)[:, None, :]
+            a, b = x[..., :8], x[..., 8:]
+            return np.concatenate([a * c - b * s_, a * s_ + b * c], -1).astype(np.float32)
+
+        x = P.embedding(w["t.embed.weight"], toks)
+        p = "t.layers.0."
+        n = P.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+        q, k, v = (P.linear(n, w[p + f"self_attn.{m}_proj.weight"]).reshape(T, -1, 16) for m in "qkv")
+        x = x + P.linear(P.attention(rot(q), rot(k), v, 3, 1).reshape(T, 48), w[p + "self_attn.o_proj.weight"])
+        x = P.ffn_block(x, w, p, dict(eps=1e-5))
+        ref = P.linear(P.rms_norm(x, w["t.norm.weight"], 1e-5), w["t.head.weight"])
+
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, toks[:25], list(range(25)), position_ids=ids[:25])]).cpu().numpy()]
+        for t in range(25, T):
+            got.append(eng.step([StepEntry(s, [toks[t]], [0], position_ids=[ids[t]])]).cpu().numpy())
+        got = np.concatenate(got)
+        assert np.abs(got - ref).max() < (1e-4 if dtype == "float32" else 4e-2) * np.abs(ref).max()
+        # a step must bring position numbers for all of its entries or for none, and one per token
+        s2 = eng.alloc_slot()
+        with pytest.raises(B.StepError, match="position"):
+            eng.step([StepEntry(s, [1], [0], position_ids=[(40, 18)]), StepEntry(s2, [1], [0])])
+        with pytest.raises(B.StepError, match="position numbers"):
+            eng.step([StepEntry(s2, [1, 2], [0], position_ids=[(0, 5)])])
+        assert eng.length(s2) == 0 and eng.length(s) == T
+    finally:
+        unregister_architecture("ToySectionForCausalLM")
+        unregister_part("position", "two_section_rotary")
+
+
+def test_attention_refuses_an_encoding_it_cannot_find_or_use():
+    norm = PartSpec("rmsnorm", {"size": 32, "eps": 1e-5})
+
+    def spec(position, positions):
+        attn = PartSpec("gqa_attention", {"hidden_size": 32, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                          "window": None, "position": position})
+        return ModelSpec(architecture="x", hidden_size=32, vocab_size=50,
+                         embedding=PartSpec("embedding", {"vocab_size": 50, "hidden_size": 32}),
+                         layers=[prenorm_layer("x.0.", attn, None, norm, None, **NAMES)], schedule=[ScheduleEntry(0, 0)],
+                         final_norm=norm, lm_head=PartSpec("lm_head", {"vocab_size": 50, "hidden_size": 32, "tied_to": None}),
+                         positions=positions, max_position_embeddings=64, embedding_prefix="x.e.", final_norm_prefix="x.n.",
+                         lm_head_prefix="x.h.")
+    rope = {"rope": PartSpec("rope", {"rotary_dim": 16, "theta": 1e4, "pairing": "half"})}
+    B.DecoderModel(spec("rope", rope))
+    B.DecoderModel(spec(None, rope))
+    with pytest.raises(B.ConfigError, match="position encoding 'rotary'"):
+        B.DecoderModel(spec("rotary", rope))            # a misspelt name is an error, not attention without positions
+
+    class Odd(B.parts.PositionEncoding):
+        gives = "sinusoid_bias"
+    register_part("position", "odd", Odd)
+    try:
+        with pytest.raises(B.ConfigError, match="cannot use"):
+            B.DecoderModel(spec("p", {"p": PartSpec("odd", {})}))
+    finally:
+        unregister_part("position", "odd")
+
+
+# --------------------- a mixer that keeps rows of two widths per token in the paged cache ----
+class LatentMixer(Mixer):
+    """One head; per token it keeps a 24-wide key and an 8-wide value in the cache (widths
+    that differ), attends over the last `window` of them, and projects the 8-wide result out."""
+
+    def __init__(self, hidden_size, window):
+        self.H, self.window = hidden_size, window
+
+    def weight_specs(self, prefix):
+        return [TensorSpec(prefix + "q.weight", (24, self.H)), TensorSpec(prefix + "k.weight", (24, self.H)),
+                TensorSpec(prefix + "v.weight", (8, self.H)), TensorSpec(prefix + "o.weight", (self.H, 8))]
+
+    def load(self, tensors, prefix, rt):
+        self.rt = rt
+        self.q, self.k, self.v, self.o = (tensors[prefix + n + ".weight"].float() for n in "qkvo")
+
+    def cache_need(self):
+        return B.cache.CacheNeed(kv_heads=1, head_dim=24, window=self.window, value_dim=8)
+
+    def forward(self, h, x, step, ctx):
+        hf = h.float()
+        q, k, v = hf @ self.q.T, hf @ self.k.T, hf @ self.v.T
+        table = ctx.block_table.cpu()
+        o = 0
+        for b, n in enumerate(step.host_new):
+            slot, start = step.host_slots[b], step.host_start[b]
+            for i in range(n):
+                pos = start + i
+                pg = int(table[slot, pos // 64])
+                ctx.keys[pg, 0].view(64, 24)[pos % 64] = k[o + i].to(ctx.keys.dtype)
+                ctx.values[pg, 0].view(64, 8)[pos % 64] = v[o + i].to(ctx.values.dtype)
+                lo = max(0, pos - self.window + 1)
+                ks = torch.stack([ctx.keys[int(table[slot, j // 64]), 0].view(64, 24)[j % 64] for j in range(lo, pos + 1)]).float()
+                vs = torch.stack([ctx.values[int(table[slot, j // 64]), 0].view(64, 8)[j % 64] for j in range(lo, pos + 1)]).float()
+                p = torch.softmax(ks @ q[o + i] / 24 ** 0.5, 0)
+                x[o + i] += (p @ vs) @ self.o.T
+            o += n
+
+
+@dataclass(frozen=True)
+class LatentConfig:
+    architecture = "ToyLatentForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls()
+
+    def to_dict(self):
+        return {"architectures": [self.architecture]}
+
+
+def latent_spec(cfg):
+    H = 40
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    layers = [prenorm_layer(f"l.layers.{i}.", PartSpec("latent", {"hidden_size": H, "window": 70}), None, norm, None, **NAMES)
+              for i in range(2)]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=50,
+                     embedding=PartSpec("embedding", {"vocab_size": 50, "hidden_size": H}), layers=layers,
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1)], final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": 50, "hidden_size": H, "tied_to": None}),
+                     positions={}, max_position_embeddings=512, embedding_prefix="l.embed.", final_norm_prefix="l.norm.",
+                     lm_head_prefix="l.head.")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_whose_keys_and_values_differ_in_width_uses_the_paged_cache(tmp_path, dtype):
+    register_part("mixer", "latent", LatentMixer)
+    register_architecture("ToyLatentForCausalLM", LatentConfig, latent_spec)
+    try:
+        folder = B.Engine.write_random_folder(str(tmp_path / "l"), LatentConfig(), seed=12, std=0.2)
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=512)
+        g = eng.cache.groups[0]
+        assert len(eng.cache.groups) == 1 and g.page_elems == 64 * (24 + 8) and g.keys(0).shape[1:] == (1, 64 * 24)
+        assert g.values(1).shape[1:] == (1, 64 * 8) and g.storage_view(0).dim() == 2
+        _, w = P.read_folder(folder)
+        rd = (lambda a: bf(a)) if dtype == "bfloat16" else (lambda a: a)
+
+        def plain(toks):
+            T = len(toks)
+            x = P.embedding(w["l.embed.weight"], toks)
+            for l in range(2):
+                p = f"l.layers.{l}.self_attn."
+                n = rd(P.rms_norm(x, w[f"l.layers.{l}.input_layernorm.weight"], 1e-5))
+                q, k, v = n @ w[p + "q.weight"].T, rd(n @ w[p + "k.weight"].T), rd(n @ w[p + "v.weight"].T)
+                for t in range(T):
+                    lo = max(0, t - 70 + 1)
+                    sc = k[lo:t + 1] @ q[t] / np.sqrt(24.0)
+                    pr = np.exp(sc - sc.max()); pr /= pr.sum()
+                    x[t] = x[t] + (pr @ v[lo:t + 1]) @ w[p + "o.weight"].T
+            return P.linear(rd(P.rms_norm(x, w["l.norm.weight"], 1e-5)), w["l.head.weight"])
+
+        rng = np.random.default_rng(8)
+        seqs = [[int(t) for t in rng.integers(0, 50, n)] for n in (150, 66)]
+        refs = [plain(s) for s in seqs]
+        for round_ in range(2):                                   # twice: pages come back and are used again
+            slots = [eng.alloc_slot() for _ in seqs]
+            cut = [100, 60]
+            out = eng.step([StepEntry(sl, s[:c], list(range(c))) for sl, s, c in zip(slots, seqs, cut)]).cpu().numpy()
+            got = [[out[:100]], [out[100:]]]
+            pos, live = list(cut), [0, 1]
+            while live:
+                out = eng.step([StepEntry(slots[i], [seqs[i][pos[i]]], [0]) for i in live]).cpu().numpy()
+                for r, i in enumerate(live):
+                    got[i].append(out[r:r + 1]); pos[i] += 1
+                for i in [i for i in live if pos[i] == len(seqs[i])]:
+                    assert g.pool.held_count <= 3 * len(live)     # the window gives pages back while the sequence grows
+                    eng.free_slot(slots[i]); live.remove(i)
+            assert g.pool.held_count == 0
+            for i in range(2):
+                gi = np.concatenate(got[i])
+                assert np.abs(gi - refs[i]).max() < (1e-4 if dtype == "float32" else 3e-2) * np.abs(refs[i]).max(), (round_, i)
+    finally:
+        unregister_architecture("ToyLatentForCausalLM")
+        unregister_part("mixer", "latent")
