@@ -392,3 +392,6 @@ extern "C" int br_convert(const void* a, void* b, int to_bf16, size_t n, hipStre
     else bf16_to_f32_kernel<<<blocks, 256, 0, s>>>((const bf16*)a, (float*)b, n);
     return br_check_launch();
 }
+
+// Compute units of the current device (0 if the runtime does not say).
+extern "C" int br_device_cu_count() { return br_device_cus(); }

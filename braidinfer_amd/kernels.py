@@ -70,6 +70,18 @@ def _fn(module: str, name: str, argtypes):
     return f
 
 
+_device_cus = {}
+
+
+def device_cus() -> int:
+    """Compute units of the current GPU (256 when the runtime does not say)."""
+    dev = torch.cuda.current_device()
+    if dev not in _device_cus:
+        n = int(_fn("elementwise", "br_device_cu_count", [])())
+        _device_cus[dev] = n if n > 0 else 256
+    return _device_cus[dev]
+
+
 # ------------------------------------------------------------------ elementwise -----
 def embedding(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
     _dev("embedding", table, tokens, out)

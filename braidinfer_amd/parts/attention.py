@@ -27,13 +27,14 @@ from .linear import fused_layout, linear, stream_layout
 MAX_HEAD_DIM = 512      # attention_simple's limit; the matrix-core kernels take up to 256 in steps of 16
 
 
-def decode_splits(batch: int, nkv: int, max_ctx: int, page: int) -> int:
+def decode_splits(batch: int, nkv: int, max_ctx: int, page: int, cus: int = 256) -> int:
     """Into how many runs a sequence's pages are cut for single-token steps: about one
-    workgroup per CU (measured: more runs cost more in the combine than they gain) and at
-    least two pages per run; beyond that, runs of at most 64 pages.  It depends on the
-    step's shape only (batch and an upper bound of the context), never on the tokens."""
+    workgroup per compute unit (measured: more runs cost more in the combine than they gain)
+    and at least two pages per run; beyond that, runs of at most 64 pages.  It depends on the
+    step's shape only (batch and an upper bound of the context) and on the device's number
+    of compute units, never on the tokens."""
     pages = max(1, -(-max_ctx // page))
-    want = -(-256 // max(1, batch * nkv))
+    want = -(-max(1, cus) // max(1, batch * nkv))
     n = max(1, min(want, pages // 2 if pages >= 2 else 1, 64))
     while n < 64 and pages > 64 * n:
         n *= 2
@@ -117,7 +118,7 @@ class GQAAttention(Mixer):
             return False
         if tables is not None and (tables.adjacent or tables.rotary_dim != self.hd):
             return False
-        nsplit = decode_splits(step.n_seqs, self.nkv, step.max_ctx_bound, ctx.page_tokens)
+        nsplit = decode_splits(step.n_seqs, self.nkv, step.max_ctx_bound, ctx.page_tokens, K.device_cus())
         return K.attention_decode_fuses_rope(self.hd, self.nq, self.nkv, ctx.page_tokens, ctx.block_table.shape[1], nsplit)
 
     def _finish(self, qkv, x, step, ctx: MixerContext, fused_tables, fused: bool) -> None:
@@ -134,7 +135,7 @@ class GQAAttention(Mixer):
         if qkv.dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and ctx.page_tokens == 64 and not self.force_simple:
             B = step.n_seqs
             if step.is_decode:
-                nsplit = decode_splits(B, nkv, step.max_ctx_bound, ctx.page_tokens)
+                nsplit = decode_splits(B, nkv, step.max_ctx_bound, ctx.page_tokens, K.device_cus())
                 part_o = part_ml = None
                 if nsplit > 1:
                     part_o = step.ws.get("attn_part_o", (B * nq * nsplit * hd,), torch.float32)

@@ -154,18 +154,19 @@ def test_wanted_places_and_chunked_prompts(engines, tiny_folders, dtype):
     eng.free_slot(a); eng.free_slot(b)
 
 
-def _marker_model(tmp_path, sliding_window=None):
+def _marker_model(tmp_path, sliding_window=None, head_dim=16, rope_theta=10000.0, max_positions=4096):
     """A one-layer model in which token 2 (the asker) attends almost only to token 1 (the
     marker), wherever it sits, and copies its content into the logits."""
+    hd = head_dim
     cfg = B.MistralConfig.from_dict(dict(num_hidden_layers=1, hidden_size=32, num_attention_heads=2,
-                                         num_key_value_heads=1, head_dim=16, intermediate_size=16,
-                                         vocab_size=40, rope_theta=10000.0, rms_norm_eps=1e-5,
-                                         max_position_embeddings=4096, sliding_window=sliding_window))
-    folder = B.Engine.write_random_folder(str(tmp_path / "m"), cfg, seed=1, std=0.02)
+                                         num_key_value_heads=1, head_dim=hd, intermediate_size=16,
+                                         vocab_size=40, rope_theta=rope_theta, rms_norm_eps=1e-5,
+                                         max_position_embeddings=max_positions, sliding_window=sliding_window))
+    folder = B.Engine.write_random_folder(str(tmp_path / f"m{hd}"), cfg, seed=1, std=0.02)
     from braidinfer_amd.weights import SafetensorsFolder, write_safetensors
     st = SafetensorsFolder(folder)
     t = {n: st.tensor(n).clone() for n in st.names()}
-    H, hd = 32, 16
+    H = 32
     emb = torch.zeros(40, H)
     content = torch.randn(40, 8, generator=torch.Generator().manual_seed(0))
     emb[:, :8] = content / content.norm(dim=-1, keepdim=True) * 8 ** 0.5              # content, equal norms
@@ -174,8 +175,8 @@ def _marker_model(tmp_path, sliding_window=None):
     t["model.embed_tokens.weight"] = emb.bfloat16()
     q = torch.zeros(2 * hd, H); k = torch.zeros(hd, H); v = torch.zeros(hd, H); o = torch.zeros(H, 2 * hd)
     # rotary leaves the last pair of each half almost unrotated at these positions (lowest
-    # frequency): put the matching direction there (elements 7 and 15 pair up in "half")
-    q[7, 9] = 6.0; k[7, 8] = 6.0
+    # frequency): put the matching direction there (elements hd/2 - 1 and hd - 1 pair up in "half")
+    q[hd // 2 - 1, 9] = 6.0; k[hd // 2 - 1, 8] = 6.0
     v[:8, :8] = torch.eye(8) * 4
     o[10:18, :8] = torch.eye(8)
     for n_, m in (("q", q), ("k", k), ("v", v), ("o", o)):
@@ -603,3 +604,100 @@ def test_the_longest_sequence_is_the_models_unless_the_caller_says_more(tiny_fol
     assert eng.cache.max_seq_len == 2048
     assert B.Engine.from_folder(folder, dtype="float32", max_tokens=8192, max_seq_len=4096).cache.max_seq_len == 4096
     assert B.Engine.from_folder(folder, dtype="float32", max_tokens=640).cache.max_seq_len == 640
+
+
+# ----------------------------------------------- thousands of tokens at the serving head size ----
+def _plain_last_rows(pc, pw, toks, n_last):
+    """The plain implementation's logits of the last rows of a long sequence.  One layer, so
+    only the attention needs the whole sequence: everything row-wise is done on the last rows,
+    the attention with the plain functions on keys and values of all positions."""
+    sz = P.sizes(pc)
+    T = len(toks)
+    p = "model.layers.0."
+    x = P.embedding(pw["model.embed_tokens.weight"], toks)
+    n = P.rms_norm(x, pw[p + "input_layernorm.weight"], sz["eps"])
+    inv = P.rope_inv_freq(sz["hd"], sz["theta"])
+    k = P.rope(P.linear(n, pw[p + "self_attn.k_proj.weight"]).reshape(T, sz["nkv"], sz["hd"]), np.arange(T), inv, sz["pairing"])
+    v = P.linear(n, pw[p + "self_attn.v_proj.weight"]).reshape(T, sz["nkv"], sz["hd"])
+    rows = np.arange(T - n_last, T)
+    q = P.rope(P.linear(n[rows], pw[p + "self_attn.q_proj.weight"]).reshape(n_last, sz["nq"], sz["hd"]), rows, inv, sz["pairing"])
+    out = np.zeros((n_last, sz["nq"], sz["hd"]), np.float32)
+    W = P.layer_window(sz, 0)
+    for r, i in enumerate(rows):                               # P.attention of one query: a 1 x T problem each
+        lo = 0 if W is None else max(0, i - W + 1)
+        for h in range(sz["nq"]):
+            kh = h // (sz["nq"] // sz["nkv"])
+            sc = (k[lo:i + 1, kh] @ q[r, h]) * np.float32(1.0 / np.sqrt(sz["hd"]))
+            e = np.exp(sc - sc.max())
+            out[r, h] = (e / e.sum()) @ v[lo:i + 1, kh]
+    xl = x[rows] + P.linear(out.reshape(n_last, -1), pw[p + "self_attn.o_proj.weight"])
+    xl = P.ffn_block(xl, pw, p, sz)
+    return P.linear(P.rms_norm(xl, pw["model.norm.weight"], sz["eps"]), pw["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [None, 4096])
+def test_a_key_thousands_of_tokens_back_at_head_size_128(tmp_path, dtype, window):
+    """The marker model at the head size of the serving shapes (in bfloat16: the attention kernels that bring
+    pages through LDS rings, the doubling of the decode runs beyond 4,096 tokens) with 9,000
+    tokens: the marker at the start, at the window's edge (seen at distance 4,095, not at
+    4,096), in the last page; the asker as the end of the whole prompt, of a last chunk of 64,
+    and decoded alone, from a graph and eagerly."""
+    folder, pc, pw = _marker_model(tmp_path, sliding_window=window, head_dim=128, rope_theta=1e8, max_positions=16384)
+    small = _plain_last_rows(pc, pw, [5, 1, 7, 2], 1)            # the helper against the whole plain forward
+    assert np.abs(small - P.forward(pc, pw, [5, 1, 7, 2])[-1:]).max() < 1e-5 * np.abs(small).max()
+    T = 9000
+    rng = np.random.default_rng(2)
+    engines_ = [B.Engine.from_folder(folder, dtype=dtype, max_tokens=9216, max_seq_len=9216, use_graphs=g) for g in (True, False)]
+    places = [(0, window is None), (T - 1 - 4095, True), (T - 1 - 4096, window is None), (T - 30, True), (4095, window is None)]
+    for at, seen in places:
+        toks = [int(x) for x in rng.integers(3, 40, T)]
+        toks[at], toks[-1] = 1, 2
+        ref = _plain_last_rows(pc, pw, toks, 1)[0]
+        assert (int(ref.argmax()) == 1) == seen, "the plain implementation must see the marker exactly where the window allows"
+        for eng in engines_:
+            for cut in ((T - 1, 0, T - 64) if eng.use_graphs else (T - 1,)):
+                s = eng.alloc_slot()
+                if cut:
+                    eng.step([StepEntry(s, toks[:cut], [])])
+                got = eng.step([StepEntry(s, toks[cut:], [T - cut - 1])]).cpu().numpy()[0]
+                if window:
+                    assert eng.cache.groups[0].pool.held_count <= 4096 // 64 + 1
+                eng.free_slot(s)
+                assert (int(got.argmax()) == 1) == seen, f"marker at {at}, cut {cut}, graphs {eng.use_graphs}"
+                close(got[None], ref[None], dtype, f"marker at {at}, cut {cut}, graphs {eng.use_graphs}")
+
+
+@pytest.mark.parametrize("live", [65, 100, 130, 200])
+def test_single_token_steps_of_many_requests(serving, live):
+    """65 to 200 requests decode together (graph buckets of 128 and 256 rows with padding
+    sequences, products by tiles cut along k, attention over 128 or 256 rows): every request
+    against the plain forward, graphs against eager steps, requests ending on the way."""
+    folder, cfg, w = serving
+    g = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=live * 128)
+    e = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=live * 128, use_graphs=False)
+    rng = np.random.default_rng(live)
+    lens = [int(n) for n in rng.integers(1, 100, live)]
+    more = [int(n) for n in rng.integers(2, 7, live)]            # tokens decoded after the prompt
+    seqs = [tokens(cfg, n + m, 900 + i) for i, (n, m) in enumerate(zip(lens, more))]
+    got = {}
+    for eng in (g, e):
+        slots = [eng.alloc_slot() for _ in seqs]
+        out = eng.step([StepEntry(sl, q[:n], [n - 1]) for sl, q, n in zip(slots, seqs, lens)]).cpu().numpy()
+        rows = [[out[i:i + 1]] for i in range(live)]
+        alive = list(range(live))
+        k = 0
+        while alive:
+            out = eng.step([StepEntry(slots[i], [seqs[i][lens[i] + k]], [0]) for i in alive]).cpu().numpy()
+            for r, i in enumerate(alive):
+                rows[i].append(out[r:r + 1])
+            k += 1
+            for i in [i for i in alive if lens[i] + k == len(seqs[i])]:
+                eng.free_slot(slots[i]); alive.remove(i)
+        got[eng.use_graphs] = [np.concatenate(r) for r in rows]
+        assert all(gr.pool.held_count == 0 for gr in eng.cache.groups)
+    assert g.use_graphs and (128 if live <= 128 else 256) in g._graphs.graphs and e._graphs is None
+    for i in range(live):
+        ref = P.forward(cfg, w, seqs[i])[lens[i] - 1:]
+        close(got[True][i], ref, "bfloat16", f"request {i} of {live}, graphs")
+        assert np.abs(got[True][i] - got[False][i]).max() <= CUT_TOL["bfloat16"] * np.abs(ref).max()

@@ -698,3 +698,115 @@ def test_gemm_swiglu_over_two_tile_shapes(blocked):
     g, u = a.float() @ wg.float().T, a.float() @ wu.float().T
     want = g / (1 + torch.exp(-g)) * u
     assert (out.float() - want).abs().max() < 1e-2 * want.abs().max()
+
+
+# ------------------------------------------------------- long contexts, serving head size ----
+def _long_cache(lens, nkv, hd, seed, first_live_page=None):
+    """Keys and values of long sequences put into shuffled pages with vector operations:
+    (k, v as float64 CPU tensors per sequence, cache, table).  Slots beyond a sequence's end
+    hold 7.0, so a kernel that reads past the end shows.  `first_live_page[b]`: pages before it
+    are given back (-1 in the table), as the cache does behind a window."""
+    page = 64
+    pages_of = [-(-n // page) for n in lens]
+    n_pages = sum(pages_of) + 5
+    g = torch.Generator().manual_seed(seed)
+    order = torch.randperm(n_pages, generator=g)
+    cache = torch.full((n_pages, 2, nkv, page, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    table = torch.full((len(lens) + 1, max(pages_of) + 2), -1, dtype=torch.int32)
+    ks, vs, used = [], [], 0
+    for b, n in enumerate(lens):
+        np_ = pages_of[b]
+        k = torch.randn(np_ * page, nkv, hd, generator=g).to(torch.bfloat16)
+        v = torch.randn(np_ * page, nkv, hd, generator=g).to(torch.bfloat16)
+        pg = order[used:used + np_]
+        used += np_
+        table[b + 1, :np_] = pg.int()
+        kk, vv = k.clone(), v.clone()
+        kk[n:], vv[n:] = 7.0, 7.0
+        cache[pg.to(DEV), 0] = kk.view(np_, page, nkv, hd).permute(0, 2, 1, 3).to(DEV)
+        cache[pg.to(DEV), 1] = vv.view(np_, page, nkv, hd).permute(0, 2, 3, 1).reshape(np_, nkv, page, hd).to(DEV)   # [hd, token] in memory
+        if first_live_page is not None and first_live_page[b] > 0:
+            table[b + 1, :first_live_page[b]] = -1
+        ks.append(k[:n].double()); vs.append(v[:n].double())
+    return ks, vs, cache, table.to(DEV)
+
+
+def _rows_ref(q_rows, q_pos, k, v, nq, nkv, window):
+    """float64 attention of a few query rows (at positions q_pos) over keys 0..pos."""
+    hd = q_rows.shape[-1]
+    out = torch.zeros(len(q_pos), nq, hd, dtype=torch.float64)
+    j = torch.arange(k.shape[0])
+    for r, p in enumerate(q_pos):
+        see = j <= p
+        if window:
+            see &= j > p - window
+        for h in range(nq):
+            kh = h // (nq // nkv)
+            s = (k[see, kh] @ q_rows[r, h].double()) / math.sqrt(hd)
+            out[r, h] = torch.softmax(s, 0) @ v[see, kh]
+    return out
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("nsplit", [1, 8, 32, 64])
+@pytest.mark.parametrize("window", [None, 4096])
+def test_attention_decode_over_long_contexts(window, nsplit, variant):
+    """Head size 128 and contexts of thousands of tokens: runs of many pages per split, splits
+    that get no page at all, a window of 4,096 far into the sequence with the pages behind it
+    given back."""
+    from braidinfer_amd.parts.attention import decode_splits
+    nq, nkv, hd = 8, 2, 128
+    lens = [5000, 20000, 32768, 4097, 300]
+    first = [max(0, n - window + 1) // 64 if window else 0 for n in lens]
+    ks, vs, cache, table = _long_cache(lens, nkv, hd, seed=3, first_live_page=first)
+    B = len(lens)
+    q = rnd(B, nq, hd, seed=97, dtype=torch.bfloat16)
+    want = [_rows_ref(q[b:b + 1].cpu(), [l - 1], ks[b], vs[b], nq, nkv, window)[0] for b, l in enumerate(lens)]
+    for ns in {nsplit, decode_splits(B, nkv, max(lens), 64)}:
+        out = torch.full((B, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
+        part_o = torch.full((B * nq * ns * hd,), float("nan"), device=DEV)
+        part_ml = torch.full((B * nq * ns * 2,), float("nan"), device=DEV)
+        K.attention_decode_bf16(q.reshape(B, nq * hd), nq * hd, out, i32(list(range(1, B + 1))), i32(lens), table, cache, B,
+                                nq, nkv, hd, 64, window, 1 / math.sqrt(hd), ns, part_o, part_ml, variant)
+        for b in range(B):
+            got = out[b].reshape(nq, hd).cpu().double()
+            assert torch.isfinite(got).all(), (b, ns)
+            assert (got - want[b]).abs().max() < 2e-2 * want[b].abs().max(), f"sequence of {lens[b]}, {ns} splits"
+
+
+def test_decode_splits_double_beyond_64_pages_a_run():
+    from braidinfer_amd.parts.attention import decode_splits
+    assert decode_splits(64, 8, 4096, 64) == 1 and decode_splits(1, 8, 2048, 64) == 16
+    assert decode_splits(64, 8, 20000, 64) == 8 and decode_splits(64, 8, 32768, 64) == 8       # 313 and 512 pages: runs of at most 64
+    assert decode_splits(8, 8, 32768, 64) == 8 and decode_splits(1, 8, 32768, 64) == 32
+    for b in (1, 3, 8, 100):
+        for ctx in (1, 64, 65, 5000, 100000, 1 << 20):
+            n = decode_splits(b, 8, ctx, 64)
+            assert 1 <= n < 128 and (n >= 64 or -(-(-(-ctx // 64)) // n) <= 64)
+    # a chip with other compute units is filled likewise: about one workgroup each
+    assert decode_splits(1, 8, 2048, 64, cus=128) == 16 and decode_splits(1, 8, 4096, 64, cus=304) == 32
+
+
+@pytest.mark.parametrize("variant", [3, 4])
+@pytest.mark.parametrize("window", [None, 4096])
+def test_attention_prefill_chunks_over_long_contexts(window, variant):
+    """Chunks of 64, 1 and 200 new tokens over 8,192, 20,000 and 4,000 earlier ones at head
+    size 128: thousands of earlier keys through the ring, the window's edge inside a page far
+    from the start, pages behind the window given back."""
+    nq, nkv, hd = 8, 2, 128
+    new = [64, 1, 200]
+    lens = [8192 + 64, 20001, 4200]
+    first = [max(0, (l - n) - window + 1) // 64 if window else 0 for l, n in zip(lens, new)]
+    ks, vs, cache, table = _long_cache(lens, nkv, hd, seed=4, first_live_page=first)
+    T = sum(new)
+    q = rnd(T, nq, hd, seed=96, dtype=torch.bfloat16)
+    cu = [0, 64, 65, 265]
+    out = torch.full((T, nq * hd), 5.0, device=DEV, dtype=torch.bfloat16)
+    K.attention_prefill_bf16(q.reshape(T, nq * hd), nq * hd, out, i32(cu), i32([1, 2, 3]), i32(lens), table, cache, 3,
+                             max(new), nq, nkv, hd, 64, window, 1 / math.sqrt(hd), variant)
+    for b, (l, n) in enumerate(zip(lens, new)):
+        rows = sorted({0, n // 2, n - 1})                         # the chunk's first, middle and last query
+        want = _rows_ref(q[cu[b]:cu[b + 1]].cpu()[rows], [l - n + r for r in rows], ks[b], vs[b], nq, nkv, window)
+        got = out[cu[b]:cu[b + 1]].reshape(n, nq, hd).cpu().double()[rows]
+        assert torch.isfinite(out[cu[b]:cu[b + 1]].float()).all()
+        assert (got - want).abs().max() < 2e-2 * want.abs().max(), f"sequence {b}"

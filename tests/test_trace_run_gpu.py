@@ -94,3 +94,27 @@ def test_bad_input_is_an_error_not_a_crash(tiny_folders, tmp_path):
                        input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [1] * 65, "want": []}], "end": []}) + "\n",
                        capture_output=True, text=True)
     assert p.returncode == 1 and "cache" in p.stderr
+
+
+def test_probes_switched_on_leave_statistics_beside_the_logits(tiny_folders, tmp_path):
+    folder, cfg, w = tiny_folders["a"]
+    out = str(tmp_path / "o")
+    toks = [3, 9, 200, 41, 7]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:4], "want": [3]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[4:], "want": [0]}], "end": ["a"]}]
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", out, "--max-tokens", "64", "--probes"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True)
+    assert p.returncode == 0 and p.stdout.split() == ["done", "0", "done", "1"], p.stderr
+    ref = P.forward(cfg, w, toks)
+    for n, row in ((0, 3), (1, 4)):
+        stats = json.load(open(os.path.join(out, f"{n}.probes.json")))
+        assert list(stats) == ["embed", "L0.post_mixer", "L0.post_ffn", "L1.post_mixer", "L1.post_ffn", "final_norm", "logits"]
+        assert stats["logits"]["shape"] == [1, cfg["vocab_size"]]
+        assert abs(stats["logits"]["absmax"] - np.abs(ref[row]).max()) < 1e-4 * np.abs(ref[row]).max()
+        got = np.fromfile(os.path.join(out, f"{n}.f32"), dtype="<f4")
+        assert np.abs(got - ref[row]).max() < 1e-4 * np.abs(ref[row]).max()
+    emb = P.embedding(w["model.embed_tokens.weight"], toks[:4])
+    first = json.load(open(os.path.join(out, "0.probes.json")))["embed"]
+    assert first["shape"] == [4, cfg["hidden_size"]] and np.allclose(first["head"], emb.reshape(-1)[:8], atol=1e-6)
+    assert abs(first["rms"] - np.sqrt((emb ** 2).mean())) < 1e-5
