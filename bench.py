@@ -1,12 +1,20 @@
 #!/usr/bin/env python3
-"""Decode and prefill throughput of the Mistral-7B-v0.3 shape on one MI355X.
+"""Decode and prefill throughput of the Mistral shapes on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|v0.1|24b] [--layers L] [--batch B]
 
 A step is one decode step of the whole batch: the engine's step function over one token
 per sequence, greedy sampling on the GPU, and the token ids read back (what the
-generation loop does per step).  Prompts have lengths uniform in [128, 2048] and random
-token ids; weights are random N(0, 0.02) bf16.  One JSON line goes to standard output.
+generation loop does per step).  Prompts have random token ids and lengths uniform in the
+workload's range; weights are random N(0, 0.02) bf16.  One JSON line goes to standard output.
+
+Workloads (the benchmark description's shapes): `headline` Mistral-7B-v0.3, context 4,096,
+batch 8, prompts in [128, 2048]; `v0.1` Mistral-7B-v0.1 with its window of 4,096, context
+8,192, batch 8, prompts in [4096, 7168]; `24b` Mistral-Small-24B, context 32,768, batch 16,
+prompts in [1024, 16384].  Beside the headline value the line carries: the decode step's
+share of the published memory rate (`roofline`), further batch sizes and prompt lengths
+(`points`), what this GPU delivers to plain streaming and matrix-core kernels of this library
+(`measured_peaks`), and where an eager decode step's kernel time goes (`kernel_share`).
 """
 import argparse
 import json
@@ -18,39 +26,132 @@ import numpy as np
 PEAK_HBM = 8.0e12          # MI355X HBM3E, bytes/s
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
+WORKLOADS = {
+    "headline": dict(preset="mistral-7b-v0.3", context=4096, batch=8, prompt_min=128, prompt_max=2048),
+    "v0.1": dict(preset="mistral-7b-v0.1", context=8192, batch=8, prompt_min=4096, prompt_max=7168),
+    "24b": dict(preset="mistral-small-24b", context=32768, batch=16, prompt_min=1024, prompt_max=16384),
+}
+
+
+def measured_peaks(torch, K):
+    """What plain kernels of this library get out of this GPU: a copy and a pure read of 2 GiB,
+    and a bf16 product of 8,192 cubed on the matrix cores (the tile kernel the prompts use)."""
+    out = {}
+    n = 1 << 31
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+    src.view(torch.int32).fill_(1)
+    sums = torch.empty(64 * 1024, dtype=torch.float32, device="cuda")
+
+    def timed(f, reps=5):
+        f()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            f()
+            b.record()
+            torch.cuda.synchronize()
+            best = min(best, a.elapsed_time(b) * 1e-3)
+        return best
+    out["hbm_copy_GBs"] = round(2 * n / timed(lambda: K.stream_copy(src, dst)) / 1e9, 1)
+    out["hbm_read_GBs"] = round(n / timed(lambda: K.stream_read(src, sums)) / 1e9, 1)
+    del src, dst
+    M = 8192
+    a = torch.randn(M, M, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    w = torch.randn(M, M, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    c = torch.empty(M, M, device="cuda", dtype=torch.bfloat16)
+    out["mfma_bf16_TFLOPs"] = round(2.0 * M ** 3 / timed(lambda: K.gemm(a, w, c)) / 1e12, 1)
+    return out
+
+
+def kernel_share(torch, eng, entries_of, classes):
+    """Where the kernel time of one decode step goes: the step is run eagerly (no graph) with
+    every launcher of `braidinfer_amd.kernels` bracketed by events; shares by class of kernel."""
+    from braidinfer_amd import kernels as K
+    records = []
+    saved = {}
+
+    def wrap(name, f):
+        def g(*a, **k):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            r = f(*a, **k)
+            e.record()
+            records.append((classes(name, a, k), s, e))
+            return r
+        return g
+    names = ["embedding", "rmsnorm", "rope_table", "rope_kv_write", "silu_mul", "residual_add", "gather_rows", "convert",
+             "gemm", "gemm_swiglu", "gemm_norm_prepare", "gemm_norm_scaled", "attention_simple",
+             "attention_prefill_bf16", "attention_decode_bf16", "argmax"]
+    was = eng.use_graphs
+    eng.use_graphs = False
+    try:
+        for n in names:
+            saved[n] = getattr(K, n)
+            setattr(K, n, wrap(n, saved[n]))
+        eng.step(entries_of())           # once to size the workspace
+        records.clear()
+        eng.step(entries_of())
+        torch.cuda.synchronize()
+    finally:
+        for n, f in saved.items():
+            setattr(K, n, f)
+        eng.use_graphs = was
+    total, by = 0.0, {}
+    for cls, s, e in records:
+        ms = s.elapsed_time(e)
+        by[cls] = by.get(cls, 0.0) + ms
+        total += ms
+    share = {k: round(v / total, 4) for k, v in sorted(by.items(), key=lambda kv: -kv[1])}
+    share["kernels_ms"] = round(total, 3)
+    share["launches"] = len(records)
+    return share
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS),
+                    help="which of the benchmark description's shapes (preset, context, batch, prompt lengths)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--preset", default="mistral-7b-v0.3")
+    ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--preset", default=None)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--prompt-min", type=int, default=128)
-    ap.add_argument("--prompt-max", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=None)
+    ap.add_argument("--prompt-min", type=int, default=None)
+    ap.add_argument("--prompt-max", type=int, default=None)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--no-points", action="store_true",
+                    help="skip the further batch sizes and prompt lengths, the measured peaks and the kernel shares")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the prefill of --prefill-tokens (for profiles); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    wl = WORKLOADS[args.workload]
+    for k, v in wl.items():
+        if getattr(args, k) is None:
+            setattr(args, k, v)
+    headline = args.workload == "headline"
 
     import torch
     import braidinfer_amd as B
     from braidinfer_amd import StepEntry
+    from braidinfer_amd import kernels as K
     from braidinfer_amd.sampling import Sampler
 
     full = B.preset(args.preset)
     layers = args.layers or full.num_hidden_layers
     cfg = B.preset(args.preset, num_hidden_layers=layers)
-    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
-    room = max(max(batches) * (-(-(args.prompt_max + args.steps + args.warmup + 1) // 64) * 64),
-               -(-args.prefill_tokens // 64) * 64)
+    points_on = not args.no_points
+    batches = sorted({1, args.batch, 64, 128}) if (points_on and headline) else [args.batch]
+    per_seq = -(-(min(args.prompt_max, args.context) + args.steps + args.warmup + 1) // 64) * 64
+    room = max(max(batches) * per_seq, -(-args.prefill_tokens // 64) * 64)
     t0 = time.time()
     eng = B.Engine.random(cfg, seed=0, dtype=args.dtype, max_tokens=room, max_seq_len=args.context)
     print(f"[bench] engine with {layers} layers ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
@@ -61,29 +162,36 @@ def main() -> int:
     layer_params = (nq + 2 * nkv) * hd * H + H * nq * hd + 3 * H * I
     weight_bytes = (layers * layer_params + V * H) * esz + (2 * layers + 1) * H * 4
     kv_bytes_per_token = 2 * nkv * hd * esz * layers
+    W = cfg.sliding_window
 
-    def prefill(T, reps=4):
+    def prefill(engine, T, reps=4):
         rng = np.random.default_rng(5)
         prompt = [int(t) for t in rng.integers(0, V, T)]
         times = []
         for rep in range(reps):
-            s = eng.alloc_slot()
+            s = engine.alloc_slot()
             torch.cuda.synchronize()
             t = time.perf_counter()
-            eng.step([StepEntry(s, prompt, [T - 1])])
+            engine.step([StepEntry(s, prompt, [T - 1])])
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
-            eng.free_slot(s)
+            engine.free_slot(s)
         pt = min(times[1:])
-        flops = 2.0 * layers * layer_params * T + 2.0 * V * H + 2.0 * T * T * hd * nq * layers
+        # attention counted causally (2 T^2 hd per head), and within the window where the model has one
+        if W:
+            pairs = sum(min(t + 1, W) for t in range(T))
+            attn = 4.0 * pairs * hd * nq * layers
+        else:
+            attn = 2.0 * T * T * hd * nq * layers
+        flops = 2.0 * layers * layer_params * T + 2.0 * V * H + attn
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
         return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3), "frac": round(flops / pt / peak, 4)}
 
     if args.prefill_only:
-        print(json.dumps({"metric": "prefill tok/s", "layers": layers, "prefill": prefill(args.prefill_tokens)}), flush=True)
+        print(json.dumps({"metric": "prefill tok/s", "layers": layers, "prefill": prefill(eng, args.prefill_tokens)}), flush=True)
         return 0
 
-    def decode(batch, steps, warmup, seed):
+    def decode(batch, steps, warmup, seed, share=False):
         rng = np.random.default_rng(seed)
         lens = [int(n) for n in rng.integers(args.prompt_min, args.prompt_max + 1, batch)]
         prompts = [[int(t) for t in rng.integers(0, V, n)] for n in lens]
@@ -109,7 +217,6 @@ def main() -> int:
             one()
         torch.cuda.synchronize()
         # keys a step has to read: the whole context, or the window where the model has one
-        W = cfg.sliding_window
         seen = lambda n: n if W is None else min(n, W)
         ctx0 = sum(seen(eng.length(s)) for s in slots)
         ctx1 = sum(seen(eng.length(s) + steps) for s in slots)
@@ -119,11 +226,29 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t) / steps
         mean_ctx_total = (ctx0 + ctx1) / 2.0
+        shares = None
+        if share:
+            products = {((nq + 2 * nkv) * hd, H): "qkv_product", (H, nq * hd): "o_product", (2 * I, H): "gate_up_product",
+                        (H, I): "down_product", (V, H): "head_product"}
+
+            def classes(name, a, k):
+                if name in ("gemm", "gemm_swiglu", "gemm_norm_prepare"):
+                    w, out, glu = a[1], a[2], name == "gemm_swiglu"
+                elif name == "gemm_norm_scaled":
+                    w, out, glu = a[4], a[5], bool(k.get("swiglu"))
+                elif name.startswith("attention"):
+                    return "attention"
+                else:
+                    return {"rmsnorm": "norm", "rope_table": "rope", "rope_kv_write": "rope", "argmax": "sampling"}.get(name, name)
+                n_out = out.shape[1] * (2 if glu else 1)
+                k_in = w.shape[1] * 128 if w.dim() == 4 else w.shape[1]
+                return products.get((n_out, k_in), "other_product")
+            shares = kernel_share(torch, eng, lambda: [StepEntry(slots[b], [toks[b]], [0]) for b in range(batch)], classes)
         for s in slots:
             eng.free_slot(s)
-        return dt, weight_bytes + mean_ctx_total * kv_bytes_per_token, float(np.mean(lens))
+        return dt, weight_bytes + mean_ctx_total * kv_bytes_per_token, float(np.mean(lens)), shares
 
-    dt, nbytes, mean_len = decode(args.batch, args.steps, args.warmup, seed=1)
+    dt, nbytes, mean_len, shares = decode(args.batch, args.steps, args.warmup, seed=1, share=points_on)
     value = args.batch / dt
     line = {
         "metric": f"decode tok/s (batch {args.batch}, {args.preset} shape, {args.dtype}, prompts uniform in "
@@ -140,18 +265,40 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(nbytes / dt / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(nbytes / dt / PEAK_HBM, 4)},
     }
-    if not args.no_points:
+    if points_on:
         points = {}
-        for b in (1, 64):
-            if b == args.batch:
-                points[f"decode_b{b}"] = round(value, 2)
-                continue
-            k = max(8, args.steps // 2)
-            d, _, _ = decode(b, k, max(2, args.warmup // 2), seed=10 + b)
-            points[f"decode_b{b}"] = round(b / d, 2)
-            print(f"[bench] batch {b}: {d * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
-        line["points"] = points
-        line["prefill"] = prefill(args.prefill_tokens)
+        if headline:
+            for b in (1, 64, 128):
+                if b == args.batch:
+                    points[f"decode_b{b}"] = round(value, 2)
+                    continue
+                k = max(8, args.steps // 2)
+                d, _, _, _ = decode(b, k, max(2, args.warmup // 2), seed=10 + b)
+                points[f"decode_b{b}"] = round(b / d, 2)
+                print(f"[bench] batch {b}: {d * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+        line["prefill"] = prefill(eng, min(args.prefill_tokens, args.context))
+        if headline:
+            for T in (128, 512):
+                points[f"prefill_{T}"] = prefill(eng, T)["value"]
+            # longer prompts than the headline's context: an engine of its own for them
+            del eng
+            torch.cuda.empty_cache()
+            long_eng = B.Engine.random(cfg, seed=0, dtype=args.dtype, max_tokens=32768, max_seq_len=32768)
+            for T in (8192, 32768):
+                r = prefill(long_eng, T, reps=3)
+                points[f"prefill_{T}"] = r["value"]
+                points[f"prefill_{T}_frac"] = r["frac"]
+                print(f"[bench] prefill of {T}: {r['ms']:.1f} ms", file=sys.stderr, flush=True)
+            del long_eng
+            torch.cuda.empty_cache()
+        if points:
+            line["points"] = points
+        line["kernel_share"] = shares
+        peaks = measured_peaks(torch, K)
+        peaks["decode_frac_of_read"] = round(nbytes / dt / 1e9 / peaks["hbm_read_GBs"], 4)
+        peaks["prefill_frac_of_mfma"] = round(line["prefill"]["frac"] * PEAK_FLOPS["bf16"] / 1e12 / peaks["mfma_bf16_TFLOPs"], 4) \
+            if args.dtype == "bfloat16" else None
+        line["measured_peaks"] = peaks
     print(json.dumps(line), flush=True)
     return 0
 

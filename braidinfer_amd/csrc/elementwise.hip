@@ -395,3 +395,46 @@ extern "C" int br_convert(const void* a, void* b, int to_bf16, size_t n, hipStre
 
 // Compute units of the current device (0 if the runtime does not say).
 extern "C" int br_device_cu_count() { return br_device_cus(); }
+
+// ------------------------------------------------------- memory-rate measurements -----
+// Plain streaming kernels that say what this GPU's memory delivers to code like the
+// kernels above: a copy (read + write) and a pure read whose result is one word per
+// workgroup.  16 bytes a lane, consecutive lanes on consecutive addresses, grid-stride.
+__global__ __launch_bounds__(256) void stream_copy_kernel(const f32x4* __restrict__ src, f32x4* __restrict__ dst, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+        dst[i] = __builtin_nontemporal_load(src + i);
+}
+
+__global__ __launch_bounds__(256) void stream_read_kernel(const f32x4* __restrict__ src, float* __restrict__ sums, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 3 * stride < n16; i += 4 * stride) {            // four loads in flight per lane
+        const f32x4 v0 = __builtin_nontemporal_load(src + i), v1 = __builtin_nontemporal_load(src + i + stride);
+        const f32x4 v2 = __builtin_nontemporal_load(src + i + 2 * stride), v3 = __builtin_nontemporal_load(src + i + 3 * stride);
+        a += (v0 + v1) + (v2 + v3);
+    }
+    for (; i < n16; i += stride) a += __builtin_nontemporal_load(src + i);
+    const float t = wave_sum((a[0] + a[1]) + (a[2] + a[3]));
+    if ((threadIdx.x & 63) == 0) sums[blockIdx.x * 4 + (threadIdx.x >> 6)] = t;
+}
+
+// bytes: a multiple of 16; sums: float [4 * blocks] for the read (blocks is returned through *blocks_out)
+extern "C" int br_stream_copy(const void* src, void* dst, size_t bytes, hipStream_t s) {
+    if (bytes == 0) return BR_OK;
+    if (bytes % 16 || ((uintptr_t)src | (uintptr_t)dst) % 16) return BR_BAD_ARG;
+    const int cus = br_device_cus();
+    const unsigned blocks = (unsigned)((cus > 0 ? cus : 256) * 8);
+    stream_copy_kernel<<<blocks, 256, 0, s>>>((const f32x4*)src, (f32x4*)dst, bytes / 16);
+    return br_check_launch();
+}
+
+extern "C" int br_stream_read(const void* src, float* sums, int sums_len, size_t bytes, hipStream_t s) {
+    if (bytes == 0) return BR_OK;
+    const int cus = br_device_cus();
+    const unsigned blocks = (unsigned)((cus > 0 ? cus : 256) * 8);
+    if (bytes % 16 || (uintptr_t)src % 16 || !sums || sums_len < (int)(4 * blocks)) return BR_BAD_ARG;
+    stream_read_kernel<<<blocks, 256, 0, s>>>((const f32x4*)src, sums, bytes / 16);
+    return br_check_launch();
+}

@@ -196,6 +196,28 @@ def random_ones(out: torch.Tensor, key: int, jitter: float, first: int = 0) -> N
     _random_fill("random_ones", out, key, float(jitter), first)
 
 
+# ------------------------------------------------------- memory-rate measurements -----
+def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst = src, 16 bytes a lane: what a plain copy kernel gets out of this GPU's memory
+    (`bench.py` reports it beside the published peak)."""
+    _dev("stream_copy", src, dst)
+    n = src.numel() * src.element_size()
+    _req(n == dst.numel() * dst.element_size() and n % 16 == 0, "stream_copy: equal sizes, a multiple of 16 bytes")
+    f = _fn("elementwise", "br_stream_copy", [_P, _P, c_size_t, _P])
+    _check(f(_ptr(src), _ptr(dst), n, _stream()), "stream_copy")
+
+
+def stream_read(src: torch.Tensor, sums: torch.Tensor) -> None:
+    """Reads all of `src` once (four 16-byte loads in flight per lane) and leaves partial sums
+    of its words in `sums` (float32, at least 32 per compute unit): the read rate of a
+    kernel that only streams."""
+    _dev("stream_read", src, sums)
+    n = src.numel() * src.element_size()
+    _req(n % 16 == 0 and sums.dtype == torch.float32, "stream_read: a multiple of 16 bytes, float32 sums")
+    f = _fn("elementwise", "br_stream_read", [_P, _P, c_int, c_size_t, _P])
+    _check(f(_ptr(src), _ptr(sums), sums.numel(), n, _stream()), "stream_read")
+
+
 # ------------------------------------------------------------------------ GEMM ------
 GEMM_SCRATCH_FLOATS = 16 * 1024 * 1024   # 64 MB: room for the partial sums of the products that the bf16 kernels split along k
 

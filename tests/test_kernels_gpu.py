@@ -810,3 +810,16 @@ def test_attention_prefill_chunks_over_long_contexts(window, variant):
         got = out[cu[b]:cu[b + 1]].reshape(n, nq, hd).cpu().double()[rows]
         assert torch.isfinite(out[cu[b]:cu[b + 1]].float()).all()
         assert (got - want).abs().max() < 2e-2 * want.abs().max(), f"sequence {b}"
+
+
+def test_stream_copy_and_read():
+    n = (1 << 20) + 48
+    src = torch.randint(-1000, 1000, (n // 4,), device=DEV).float()
+    dst = torch.zeros_like(src)
+    K.stream_copy(src, dst)
+    assert torch.equal(src, dst)
+    sums = torch.zeros(K.device_cus() * 32, device=DEV)
+    K.stream_read(src, sums)
+    assert sums.double().sum().item() == src.double().sum().item()         # integers: every word read exactly once
+    with pytest.raises(KernelError):
+        K.stream_copy(src[:-1], dst[:-1])                                    # not a multiple of 16 bytes
