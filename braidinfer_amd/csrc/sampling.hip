@@ -27,7 +27,13 @@ __device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int o
 }
 
 #define ABLOCK 1024
-__global__ __launch_bounds__(ABLOCK) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+// ADVANCE: the row's token also becomes the next single-token step's input, on the device:
+// for a live row (slot >= 0) tokens[b] = the token, and the row's position and length grow
+// by one, so the same recorded step can be replayed without the host writing its arrays.
+template <bool ADVANCE>
+__global__ __launch_bounds__(ABLOCK) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V,
+                                                        int* __restrict__ tokens, int* __restrict__ positions,
+                                                        const int* __restrict__ slots, int* __restrict__ ctx) {
     __shared__ float sv[ABLOCK / 64];
     __shared__ int si[ABLOCK / 64];
     const float* r = logits + (size_t)blockIdx.x * V;
@@ -42,14 +48,29 @@ __global__ __launch_bounds__(ABLOCK) void argmax_kernel(const float* __restrict_
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < ABLOCK / 64; ++w) argmax_combine(bv, bi, sv[w], si[w]);
-        out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+        const int tok = (bi == 0x7fffffff) ? 0 : bi;
+        out[blockIdx.x] = tok;
+        if (ADVANCE && slots[blockIdx.x] >= 0) {
+            tokens[blockIdx.x] = tok;
+            positions[blockIdx.x] += 1;
+            ctx[blockIdx.x] += 1;
+        }
     }
 }
 
 extern "C" int br_argmax(const float* logits, int* out, int B, int V, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0) return BR_BAD_ARG;
-    argmax_kernel<<<B, ABLOCK, 0, s>>>(logits, out, V);
+    argmax_kernel<false><<<B, ABLOCK, 0, s>>>(logits, out, V, nullptr, nullptr, nullptr, nullptr);
+    return br_check_launch();
+}
+
+// argmax of every row, and the rows' step arrays moved on by one token (see ADVANCE)
+extern "C" int br_argmax_advance(const float* logits, int* out, int B, int V, int* tokens, int* positions,
+                                 const int* slots, int* ctx, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0 || !tokens || !positions || !slots || !ctx) return BR_BAD_ARG;
+    argmax_kernel<true><<<B, ABLOCK, 0, s>>>(logits, out, V, tokens, positions, slots, ctx);
     return br_check_launch();
 }
 

@@ -212,6 +212,22 @@ class Engine:
         self.cache.commit(slots, new)
         return logits
 
+    def greedy_chain(self, slots: Sequence[int], tokens: Sequence[int]):
+        """A `GreedyChain` over these sequences, each with the token it takes next, or None when
+        single-token steps of this engine are not replayed from graphs (then `step` and the
+        sampler do the same work one step at a time)."""
+        if not self.use_graphs or len(slots) > 256:
+            return None
+        V = self.vocab_size
+        for t in tokens:
+            if not isinstance(t, (int, np.integer)) or isinstance(t, bool) or not 0 <= t < V:
+                raise StepError(f"token {t!r} is outside the vocabulary of {V}")
+        if self._graphs is None:
+            from .graph import DecodeGraphs
+            self._graphs = DecodeGraphs(self.model, self.cache, self.device)
+        from .graph import GreedyChain
+        return GreedyChain(self._graphs, self.cache, slots, tokens)
+
     # ---- generation (the Python entry point) -----------------------------------------------
     def generate(self, prompts, max_new_tokens: int = 64, temperature: float = 0.0, seed=None,
                  stop_token_ids=None, top_k: int = 0, top_p: float = 1.0, min_p: float = 0.0,

@@ -76,6 +76,57 @@ def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, capacity_token
     return batches
 
 
+def _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0):
+    """Greedy steps of the requests `live` through a chain until one of them ends; returns
+    those that go on.  A second step is launched before the first one's tokens are read
+    whenever no request can end for a reason known beforehand (its budget, the longest
+    sequence the cache takes); a request that meets a stop token has then been given one
+    token too many, which is dropped with its slot."""
+    try:
+        chain.launch()
+        launched, read = 1, 0
+        while True:
+            ahead = launched - read              # steps whose tokens are still to come
+            if ahead < 2 and all(len(out[i]) + ahead + 1 <= max_new_tokens
+                                 and engine.length(slot[i]) + 1 <= cache.max_seq_len for i in live):
+                chain.launch()
+                launched += 1
+            toks = chain.read()
+            read += 1
+            now = time.perf_counter()
+            stats.decode_tokens += len(live)
+            stats.decode_seconds += now - t0
+            t0 = now
+            ended = {}
+            for i, t in zip(live, toks):
+                reason = take(i, t, launched - read)
+                if reason is not None:
+                    ended[i] = reason
+            if not ended and launched == read:
+                chain.launch()
+                launched += 1
+                continue
+            if not ended:
+                continue
+            # someone ended: the tokens of a step launched ahead still belong to the others
+            going = [i for i in live if i not in ended]
+            while launched > read:
+                toks = chain.read()
+                read += 1
+                stats.decode_tokens += len(going)
+                for i, t in zip(live, toks):
+                    if i in going:
+                        reason = take(i, t, launched - read)
+                        if reason is not None:
+                            ended[i] = reason
+                going = [i for i in going if i not in ended]
+            for i, reason in ended.items():
+                finish(i, reason)
+            return going
+    finally:
+        chain.close()
+
+
 def generate(engine: Engine, prompts: Sequence[Sequence[int]],
              params: Union[None, SamplingParams, Sequence[SamplingParams]] = None,
              max_new_tokens: int = 64, stop_token_ids: Optional[Sequence[int]] = None,
@@ -120,45 +171,60 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
         slot = {i: engine.alloc_slot() for i in live}
         out = {i: [] for i in live}
         hist = {i: list(prompts[i]) for i in live}
+
+        def take(i, t, ahead=0):
+            """Book the token request i was given; the reason it ends with, or None.  `ahead`:
+            steps already launched beyond the one this token comes from."""
+            if t in stops:
+                if include_stop:
+                    out[i].append(t)
+                return "stop"
+            out[i].append(t)
+            hist[i].append(t)
+            if len(out[i]) >= max_new_tokens:
+                return "length"
+            if engine.length(slot[i]) - ahead + 1 > cache.max_seq_len:
+                return "context"
+            return None
+
+        def finish(i, reason):
+            results[i] = GenerationResult(out[i], reason, len(prompts[i]))
+            engine.free_slot(slot.pop(i))      # an ended sequence leaves the batch at once
+
+        def sample_and_book(logits, live, prefill):
+            toks = sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live],
+                                  [uniform(seeds[i], i, len(out[i])) for i in live])
+            dt = time.perf_counter() - t0       # sampling returned the tokens: the step is done
+            if prefill:
+                stats.prefill_tokens += sum(len(prompts[i]) for i in live)
+                stats.prefill_seconds += dt
+            else:
+                stats.decode_tokens += len(live)
+                stats.decode_seconds += dt
+            still = []
+            for i, t in zip(live, toks):
+                reason = take(i, t)
+                if reason is None:
+                    still.append(i)
+                else:
+                    finish(i, reason)
+            return still
+
         try:
             t0 = time.perf_counter()
             logits = engine.step([StepEntry(slot[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
-            first = True
-            while True:
-                toks = sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live],
-                                      [uniform(seeds[i], i, len(out[i])) for i in live])
-                dt = time.perf_counter() - t0       # sampling returned the tokens: the step is done
-                if first:
-                    stats.prefill_tokens += sum(len(prompts[i]) for i in live)
-                    stats.prefill_seconds += dt
-                    first = False
-                else:
-                    stats.decode_tokens += len(live)
-                    stats.decode_seconds += dt
-                still = []
-                for i, t in zip(live, toks):
-                    reason = None
-                    if t in stops:
-                        reason = "stop"
-                        if include_stop:
-                            out[i].append(t)
-                    else:
-                        out[i].append(t)
-                        hist[i].append(t)
-                        if len(out[i]) >= max_new_tokens:
-                            reason = "length"
-                        elif engine.length(slot[i]) + 1 > cache.max_seq_len:
-                            reason = "context"
-                    if reason is None:
-                        still.append(i)
-                    else:
-                        results[i] = GenerationResult(out[i], reason, len(prompts[i]))
-                        engine.free_slot(slot.pop(i))      # an ended sequence leaves the batch at once
-                live = still
-                if not live:
-                    break
+            live = sample_and_book(logits, live, True)
+            # plain greedy requests decode through a chain when the engine has one: a step's tokens feed
+            # the next step on the device, and the host reads them one step behind
+            open_chain = getattr(engine, "greedy_chain", None) if all(plist[i].is_plain_greedy for i in live) else None
+            while live:
                 t0 = time.perf_counter()
-                logits = engine.step([StepEntry(slot[i], [out[i][-1]], [0]) for i in live])
+                chain = open_chain([slot[i] for i in live], [out[i][-1] for i in live]) if open_chain else None
+                if chain is not None:
+                    live = _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0)
+                else:
+                    logits = engine.step([StepEntry(slot[i], [out[i][-1]], [0]) for i in live])
+                    live = sample_and_book(logits, live, False)
         finally:
             for s in slot.values():
                 engine.free_slot(s)

@@ -16,6 +16,10 @@ from typing import Dict, List, Sequence
 
 import torch
 
+from collections import deque
+
+from .. import kernels as K
+from ..errors import StepError
 from .step import StepBatch, Workspace
 
 
@@ -64,15 +68,68 @@ class DecodeGraph:
             if gc_was_on:
                 gc.enable()
         torch.cuda.synchronize(dev)
+        self.model, self.cache, self.device = model, cache, dev
+        # the step's arrays on the host, pinned, so that the copy to the device does not wait
+        # (two, used in turn: a buffer is written again only when its last copy has been made)
+        self.host_ints = [torch.zeros(4 * B, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.host_copied = [None, None]
+        self.host_turn = 0
+        self.greedy_graph = None
+        self.next_tokens = torch.zeros(B, dtype=torch.int32, device=dev)
+        self.owner = None                # the chain whose sequences the device arrays describe, if any
+
+    def load(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int]) -> None:
+        """Write the step's arrays: tokens, positions, slots and lengths of the n live rows,
+        padding rows behind them."""
+        B, n = self.B, len(slots)
+        k = self.host_turn
+        self.host_turn ^= 1
+        if self.host_copied[k] is not None:
+            self.host_copied[k].synchronize()
+        h = self.host_ints[k].numpy()
+        h[0:n] = tokens
+        h[B:B + n] = starts
+        h[2 * B:2 * B + n] = slots
+        h[3 * B:3 * B + n] = starts
+        h[3 * B:3 * B + n] += 1
+        if n < B:
+            h[n:B] = 0
+            h[B + n:2 * B] = 0
+            h[2 * B + n:3 * B] = -1
+            h[3 * B + n:4 * B] = 0
+        self.ints.copy_(self.host_ints[k], non_blocking=True)
+        if self.host_copied[k] is None:
+            self.host_copied[k] = torch.cuda.Event()
+        self.host_copied[k].record()
 
     def run(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int]) -> torch.Tensor:
-        B, n = self.B, len(slots)
-        pad = B - n
-        host = (list(tokens) + [0] * pad + list(starts) + [0] * pad + list(slots) + [-1] * pad
-                + [s + 1 for s in starts] + [0] * pad)
-        self.ints.copy_(torch.tensor(host, dtype=torch.int32))
+        self.owner = None
+        self.load(slots, tokens, starts)
         self.graph.replay()
-        return self.logits[:n]
+        return self.logits[:len(slots)]
+
+    def run_greedy(self) -> None:
+        """One more step of the rows the arrays describe: the recorded step, the argmax of
+        every row into `next_tokens`, and the arrays moved on by that token, all on the
+        device (recorded as a second graph over the same buffers when first asked for)."""
+        if self.greedy_graph is None:
+            torch.cuda.synchronize(self.device)
+            saved = self.ints.clone()
+            g = torch.cuda.CUDAGraph()
+            gc_was_on = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(g):
+                    self.model.forward(self.step, self.cache, self.want_rows, self.B, self.logits)
+                    K.argmax_advance(self.logits, self.next_tokens, self.step.tokens, self.step.positions,
+                                     self.step.slots, self.step.ctx_lens)
+            finally:
+                if gc_was_on:
+                    gc.enable()
+            torch.cuda.synchronize(self.device)
+            self.ints.copy_(saved)       # recording runs nothing, but keep the arrays as they were in any case
+            self.greedy_graph = g
+        self.greedy_graph.replay()
 
 
 class DecodeGraphs:
@@ -83,9 +140,71 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self.graphs: Dict[int, DecodeGraph] = {}
 
-    def run(self, slots, tokens, starts) -> torch.Tensor:
-        b = bucket_of(len(slots))
+    def of(self, n: int) -> DecodeGraph:
+        b = bucket_of(n)
         g = self.graphs.get(b)
         if g is None:
             g = self.graphs[b] = DecodeGraph(self.model, self.cache, self.device, b)
-        return g.run(slots, tokens, starts)
+        return g
+
+    def run(self, slots, tokens, starts) -> torch.Tensor:
+        return self.of(len(slots)).run(slots, tokens, starts)
+
+
+class GreedyChain:
+    """Greedy single-token steps of one fixed set of sequences with the host out of the way:
+    a step's tokens go into the next step's input on the device, so a step can be launched
+    before the tokens of the one before have been read.  `launch` runs one step for every
+    sequence (reserving cache pages first, as `Engine.step` does); `read` returns the tokens of
+    the oldest launched step that has not been read.  At most two steps may be unread.
+
+    The chain owns the recorded step of its batch size until it is closed or any other
+    single-token step of that size runs, after which `launch` refuses."""
+
+    def __init__(self, graphs: DecodeGraphs, cache, slots: Sequence[int], tokens: Sequence[int]):
+        if not slots or len(slots) != len(tokens) or len(set(slots)) != len(slots):
+            raise StepError("a chain needs one token for each of its distinct slots")
+        self.cache, self.slots, self.n = cache, list(slots), len(slots)
+        for s in self.slots:
+            cache.slots.check_live(s)
+        self.g = graphs.of(self.n)
+        self.g.load(self.slots, list(tokens), [cache.lengths[s] for s in self.slots])
+        self.g.owner = self
+        self.ones = [1] * self.n
+        self.host = [torch.zeros(self.g.B, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.turn = 0
+        self.pending = deque()
+
+    def launch(self) -> None:
+        if self.g.owner is not self:
+            raise StepError("this chain's recorded step has been used by another step since; open a new chain")
+        if len(self.pending) >= 2:
+            raise StepError("two launched steps are unread; read one first")
+        held = self.cache.pages_held()
+        self.cache.reserve(self.slots, self.ones)
+        try:
+            self.g.run_greedy()
+        except BaseException:
+            self.cache.release_reserved(self.slots, held)
+            raise
+        self.cache.commit(self.slots, self.ones)
+        buf = self.host[self.turn]
+        self.turn ^= 1
+        buf.copy_(self.g.next_tokens, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.pending.append((ev, buf))
+
+    def read(self) -> List[int]:
+        if not self.pending:
+            raise StepError("no launched step is unread")
+        ev, buf = self.pending.popleft()
+        ev.synchronize()
+        return buf[:self.n].tolist()
+
+    def close(self) -> None:
+        """Wait for what was launched and give the recorded step back."""
+        while self.pending:
+            self.pending.popleft()[0].synchronize()
+        if self.g.owner is self:
+            self.g.owner = None

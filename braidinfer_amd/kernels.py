@@ -525,6 +525,20 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _check(f(_ptr(logits), _ptr(out), B, V, _stream()), "argmax")
 
 
+def argmax_advance(logits: torch.Tensor, out: torch.Tensor, tokens: torch.Tensor, positions: torch.Tensor,
+                   slots: torch.Tensor, ctx_lens: torch.Tensor) -> None:
+    """`argmax`, and for every live row (slot >= 0) the step arrays of the next single-token
+    step: tokens[b] = the row's token, positions[b] and ctx_lens[b] one more."""
+    _dev("argmax_advance", logits, out, tokens, positions, slots, ctx_lens)
+    B, V = logits.shape
+    _req(logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= B, "argmax_advance: float32 in, int32 out")
+    _req(all(t.dtype == torch.int32 and t.numel() >= B for t in (tokens, positions, slots, ctx_lens)),
+         "argmax_advance: the step arrays must be int32 [B]")
+    f = _fn("sampling", "br_argmax_advance", [_P, _P, c_int, c_int, _P, _P, _P, _P, _P])
+    _check(f(_ptr(logits), _ptr(out), B, V, _ptr(tokens), _ptr(positions), _ptr(slots), _ptr(ctx_lens), _stream()),
+           "argmax_advance")
+
+
 def sample_prepare(logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature):
     _dev("sample_prepare", logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature)
     B, V = logits.shape

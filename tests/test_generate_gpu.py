@@ -69,6 +69,68 @@ def test_alone_or_in_a_batch_gives_the_same_tokens(engines, tiny_folders):
     assert by_two == together
 
 
+def test_greedy_through_the_chain_equals_greedy_step_by_step(tiny_folders):
+    """Plain greedy requests decode through a chain (a step's tokens feed the next on the
+    device, one step is launched ahead).  In 32-bit that must give the tokens and reasons of
+    single steps, with stop tokens, unequal budgets of context, and page edges on the way."""
+    folder, cfg, w = tiny_folders["b"]
+    with_chain = B.Engine.from_folder(folder, dtype="float32", max_tokens=4096, max_seq_len=160)
+    without = B.Engine.from_folder(folder, dtype="float32", max_tokens=4096, max_seq_len=160, use_graphs=False)
+    assert with_chain.greedy_chain is not None and without.greedy_chain([0], [1]) is None
+    prompts = prompts_of(cfg, [3, 60, 17, 120, 1, 63, 150], 5)
+    free_run = without.generate(prompts, max_new_tokens=70, stop_token_ids=[])
+    stop = free_run[2][9]
+    for kw in (dict(max_new_tokens=70, stop_token_ids=[]), dict(max_new_tokens=70, stop_token_ids=[stop]),
+               dict(max_new_tokens=5, stop_token_ids=[stop], include_stop=True), dict(max_new_tokens=1, stop_token_ids=[])):
+        a, sa = without.generate(prompts, return_stats=True, **kw)
+        b, sb = with_chain.generate(prompts, return_stats=True, **kw)
+        assert a == b, kw
+        assert sb.decode_tokens >= sa.decode_tokens
+        for eng in (with_chain, without):
+            assert all(g.pool.held_count == 0 for g in eng.cache.groups) and eng.cache.slots.free_count == eng.cache.n_slots
+    # the cache's longest sequence is 192 (whole pages): 150 + 42 tokens are fed, the 43rd new token is the last
+    assert with_chain.cache.max_seq_len == 192 and len(free_run[6]) == 43
+    assert free_run[6] == P.greedy_generate(cfg, w, prompts[6], 43)
+    assert free_run[0] == P.greedy_generate(cfg, w, prompts[0], 70)
+
+
+def test_the_chain_by_hand(tiny_folders):
+    folder, cfg, w = tiny_folders["a"]
+    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=1024)
+    prompts = prompts_of(cfg, [5, 70], 8)
+    want = [P.greedy_generate(cfg, w, p, 4) for p in prompts]
+    slots = [eng.alloc_slot() for _ in prompts]
+    logits = eng.step([B.StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
+    first = logits.argmax(-1).tolist()
+    chain = eng.greedy_chain(slots, first)
+    chain.launch()
+    chain.launch()
+    with pytest.raises(B.StepError, match="unread"):
+        chain.launch()
+    got = [first, chain.read(), chain.read()]
+    chain.launch()
+    got.append(chain.read())
+    assert [list(t) for t in zip(*got)] == want and [eng.length(s) for s in slots] == [8, 73]
+    with pytest.raises(B.StepError, match="unread"):
+        chain.read()
+    # any other single-token step of that size takes the recorded step away from the chain
+    other = [eng.alloc_slot(), eng.alloc_slot()]
+    eng.step([B.StepEntry(other[0], [1, 2], []), B.StepEntry(other[1], [3], [])])
+    eng.step([B.StepEntry(other[0], [4], [0]), B.StepEntry(other[1], [5], [0])])
+    with pytest.raises(B.StepError, match="another step"):
+        chain.launch()
+    chain.close()
+    with pytest.raises(B.StepError, match="vocabulary"):
+        eng.greedy_chain(slots, [0, cfg["vocab_size"]])
+    again = eng.greedy_chain(slots, got[-1])       # a new chain goes on where the old one stopped
+    again.launch()
+    more = again.read()
+    again.close()
+    assert more == [P.greedy_generate(cfg, w, p, 5)[-1] for p in prompts]
+    for s in slots + other:
+        eng.free_slot(s)
+
+
 def test_command_line(tiny_folders):
     folder, cfg, w = tiny_folders["a"]
     p = [7, 3, 200, 5]

@@ -162,3 +162,72 @@ def test_uniform_numbers_depend_only_on_seed_sequence_and_draw():
     assert a == [uniform(7, 3, i) for i in range(1000)] and all(0.0 <= x < 1.0 for x in a)
     assert abs(sum(a) / 1000 - 0.5) < 0.05
     assert uniform(7, 3, 0) != uniform(7, 4, 0) != uniform(8, 3, 0)
+
+
+# ---- greedy requests through a chain: the host reads a step behind -------------------------
+class FakeChain:
+    """What `Engine.greedy_chain` hands out, with the stand-in model: every launch feeds each
+    row the token the launch before gave it, whether or not the host has read it yet."""
+
+    def __init__(self, engine, slots, tokens):
+        self.e, self.slots, self.tokens, self.unread, self.closed = engine, list(slots), list(tokens), [], False
+        engine.chains.append(self)
+
+    def launch(self):
+        assert not self.closed and len(self.unread) < 2
+        for s in self.slots:
+            assert s in self.e.live, "a step for a slot that was given back"
+            self.e.live[s] += 1
+            assert self.e.live[s] <= self.e.cache.max_seq_len, "a step beyond the longest sequence"
+        self.tokens = [(t + 1) % 50 for t in self.tokens]
+        self.unread.append(list(self.tokens))
+        self.e.steps.append((list(self.slots), [1] * len(self.slots)))
+        self.e.launched_ahead += len(self.unread) == 2
+
+    def read(self):
+        return self.unread.pop(0)
+
+    def close(self):
+        self.closed = True
+
+
+class ChainEngine(FakeEngine):
+    def __init__(self, *a, **k):
+        super().__init__(*a, **k)
+        self.chains, self.launched_ahead = [], 0
+
+    def greedy_chain(self, slots, tokens):
+        return FakeChain(self, slots, tokens)
+
+
+def test_a_chain_gives_the_tokens_of_single_steps_for_every_way_of_ending():
+    import random
+    rnd = random.Random(3)
+    for trial in range(60):
+        n = rnd.randint(1, 5)
+        prompts = [[rnd.randint(1, 49) for _ in range(rnd.randint(1, 4))] for _ in range(n)]
+        kw = dict(max_new_tokens=rnd.randint(1, 9), stop_token_ids=rnd.choice([[], [0], [rnd.randint(1, 49)]]),
+                  include_stop=rnd.random() < 0.3)
+        limit = rnd.choice([None, 6, 9])
+        plain, chained = FakeEngine(max_seq_len=limit), ChainEngine(max_seq_len=limit)
+        a, sa = run(plain, prompts, **kw)
+        b, sb = run(chained, prompts, **kw)
+        assert [(r.tokens, r.finish_reason) for r in a] == [(r.tokens, r.finish_reason) for r in b], (trial, prompts, kw, limit)
+        assert not chained.live and all(c.closed and not c.unread for c in chained.chains)
+        assert sa.decode_tokens <= sb.decode_tokens <= sa.decode_tokens + n       # at most one token too many per request
+
+
+def test_a_chain_runs_a_step_ahead_only_when_nobody_can_end_for_a_known_reason():
+    e = ChainEngine()
+    res, _ = run(e, [[5], [20]], max_new_tokens=6, stop_token_ids=[])
+    assert [r.tokens for r in res] == [[6, 7, 8, 9, 10, 11], [21, 22, 23, 24, 25, 26]]
+    assert len(e.chains) == 1 and e.launched_ahead == 4       # of 5 chain steps, the last is never launched ahead
+    assert len(e.steps) == 6                                  # and none beyond the budget
+    e = ChainEngine()
+    res, _ = run(e, [[46], [10]], max_new_tokens=8)           # request 0 meets the stop token 0 on its fourth token
+    assert res[0].tokens == [47, 48, 49] and res[0].finish_reason == "stop" and res[1].tokens == list(range(11, 19))
+    assert len(e.chains) == 2 and e.chains[0].slots == [0, 1] and e.chains[1].slots == [1]
+    # sampled requests do not use the chain
+    e = ChainEngine()
+    run(e, [[5]], max_new_tokens=3, stop_token_ids=[], params=SamplingParams(temperature=0.5, seed=1))
+    assert not e.chains
