@@ -105,8 +105,10 @@ def main(argv=None) -> int:
                          "every layer's mixer and feed-forward, of the final norm and the logits")
     args = ap.parse_args(argv)
     try:
-        engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device,
-                                    max_tokens=max(args.max_tokens, 64))
+        # a replay takes any request the cache holds: the longest sequence is the cache's size, whatever
+        # number of positions the model's configuration names (rotary angles are defined for every position)
+        room = max(args.max_tokens, 64)
+        engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device, max_tokens=room, max_seq_len=room)
         Replayer(engine, args.out, probes=args.probes).run(sys.stdin, sys.stdout)
     except BraidError as e:
         print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr, flush=True)

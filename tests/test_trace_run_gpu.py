@@ -118,3 +118,23 @@ def test_probes_switched_on_leave_statistics_beside_the_logits(tiny_folders, tmp
     first = json.load(open(os.path.join(out, "0.probes.json")))["embed"]
     assert first["shape"] == [4, cfg["hidden_size"]] and np.allclose(first["head"], emb.reshape(-1)[:8], atol=1e-6)
     assert abs(first["rms"] - np.sqrt((emb ** 2).mean())) < 1e-5
+
+
+def test_a_replay_is_not_bound_by_the_configurations_positions(tmp_path):
+    """config.json without max_position_embeddings means 2,048 to the engine's own entry
+    points; a replay sized for a longer request still takes it."""
+    import json as _json
+    import braidinfer_amd as B
+    cfg = B.preset("tiny-a")
+    folder = B.Engine.write_random_folder(str(tmp_path / "m"), cfg, seed=3, std=0.08)
+    d = _json.load(open(os.path.join(folder, "config.json")))
+    del d["max_position_embeddings"]
+    _json.dump(d, open(os.path.join(folder, "config.json"), "w"))
+    pc, w = P.read_folder(folder)
+    toks = [int(t) for t in np.random.default_rng(0).integers(0, 256, 2100)]
+    tr = Trace(folder, "float32", str(tmp_path / "o"), max_tokens=2112)
+    assert tr.step([{"id": "a", "tokens": toks[:2090], "want": []}]) is None
+    got = tr.step([{"id": "a", "tokens": toks[2090:], "want": [9]}], end=["a"])
+    tr.close()
+    ref = P.forward(pc, w, toks)[-1]
+    assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
