@@ -95,6 +95,11 @@ class MistralConfig:
             if not isinstance(lt, (list, tuple)) or not all(isinstance(t, str) for t in lt):
                 raise ConfigError("config.json: layer_types must be a list of strings")
             lt = tuple(lt)
+        # rotary frequencies are the plain ones (the reference has no scaling of any kind either,
+        # config.rs:253-272): a configuration that asks for scaled ones is refused, not run unscaled
+        scaling = d.get("rope_scaling")
+        if scaling not in (None, {}) and not (isinstance(scaling, dict) and scaling.get("rope_type", scaling.get("type")) in (None, "default")):
+            raise ConfigError(f"config.json: rope_scaling {scaling!r} is not supported (plain rotary frequencies only)")
         tie = d.get("tie_word_embeddings", False)
         if not isinstance(tie, bool):
             raise ConfigError(f"config.json: tie_word_embeddings must be a boolean, found {tie!r}")

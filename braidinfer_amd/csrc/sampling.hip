@@ -77,14 +77,14 @@ extern "C" int br_argmax_advance(const float* logits, int* out, int B, int V, in
 // --------------------------------------------------- bias, penalty, temperature ----
 // work[b, :] = logits[b, :]; then per row, in the reference's order (sampling.rs:57-87):
 // bias entries (token, delta) are added; every history token's logit is divided by the
-// penalty when positive, multiplied otherwise, once per occurrence (`count` times for a
-// unique token); everything is divided by the temperature when it is not 0.
-// Sparse lists are ragged: entries of row b are [off[b], off[b+1]).
+// penalty when positive, multiplied otherwise, once per occurrence; everything is divided by
+// the temperature when it is not 0.  The bias lists are ragged: entries of row b are
+// [off[b], off[b+1]).  The history is a table counts[B, V] of occurrences per token (null: none),
+// which br_sample_draw_count keeps up to date on the device.
 __global__ __launch_bounds__(SBLOCK) void sample_prepare_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int V,
     const int* __restrict__ bias_off, const int* __restrict__ bias_tok, const float* __restrict__ bias_val,
-    const int* __restrict__ hist_off, const int* __restrict__ hist_tok, const int* __restrict__ hist_cnt,
-    const float* __restrict__ penalty, const float* __restrict__ temperature) {
+    const float* __restrict__ penalty, const float* __restrict__ temperature, const int* __restrict__ counts) {
     const int b = blockIdx.x;
     const float* r = logits + (size_t)b * V;
     float* w = work + (size_t)b * V;
@@ -100,13 +100,15 @@ __global__ __launch_bounds__(SBLOCK) void sample_prepare_kernel(
         __syncthreads();
     }
     const float pen = penalty ? penalty[b] : 1.f;
-    if (hist_off && pen != 1.f) {
-        for (int e = hist_off[b] + threadIdx.x; e < hist_off[b + 1]; e += SBLOCK) {
-            int tk = hist_tok[e];
-            if (tk < 0 || tk >= V) continue;
-            float v = w[tk];
-            for (int c = 0; c < hist_cnt[e]; ++c) v = (v > 0.f) ? v / pen : v * pen;
-            w[tk] = v;
+    if (counts && pen != 1.f) {
+        const int* cn = counts + (size_t)b * V;
+        for (int i = threadIdx.x; i < V; i += SBLOCK) {
+            const int n = cn[i];
+            if (n > 0) {
+                float v = w[i];
+                for (int c = 0; c < n; ++c) v = (v > 0.f) ? v / pen : v * pen;
+                w[i] = v;
+            }
         }
         __syncthreads();
     }
@@ -116,13 +118,26 @@ __global__ __launch_bounds__(SBLOCK) void sample_prepare_kernel(
 }
 
 extern "C" int br_sample_prepare(const float* logits, float* work, int B, int V, const int* bias_off,
-                                 const int* bias_tok, const float* bias_val, const int* hist_off,
-                                 const int* hist_tok, const int* hist_cnt, const float* penalty,
-                                 const float* temperature, hipStream_t s) {
+                                 const int* bias_tok, const float* bias_val, const int* counts,
+                                 const float* penalty, const float* temperature, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0) return BR_BAD_ARG;
-    sample_prepare_kernel<<<B, SBLOCK, 0, s>>>(logits, work, V, bias_off, bias_tok, bias_val, hist_off,
-                                               hist_tok, hist_cnt, penalty, temperature);
+    sample_prepare_kernel<<<B, SBLOCK, 0, s>>>(logits, work, V, bias_off, bias_tok, bias_val, penalty, temperature, counts);
+    return br_check_launch();
+}
+
+// counts[row[e], tok[e]] += cnt[e] for n entries (a history put into the table)
+__global__ void sample_count_add_kernel(int* __restrict__ counts, int V, const int* __restrict__ row,
+                                        const int* __restrict__ tok, const int* __restrict__ cnt, int n) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n && tok[e] >= 0 && tok[e] < V) atomicAdd(counts + (size_t)row[e] * V + tok[e], cnt[e]);
+}
+
+extern "C" int br_sample_count_add(int* counts, int B, int V, const int* row, const int* tok, const int* cnt, int n,
+                                   hipStream_t s) {
+    if (n <= 0) return BR_OK;
+    if (!counts || B <= 0 || V <= 0) return BR_BAD_ARG;
+    sample_count_add_kernel<<<(n + 255) / 256, 256, 0, s>>>(counts, V, row, tok, cnt, n);
     return br_check_launch();
 }
 
@@ -400,7 +415,7 @@ extern "C" int br_sample_filter_sort(float* work, unsigned long long* keys, int 
 // last partial sum (:170).  Sums run over indices in ascending order, SBLOCK at a time.
 __global__ __launch_bounds__(SBLOCK) void sample_draw_kernel(const float* __restrict__ work, int* __restrict__ out,
                                                              int V, const float* __restrict__ temperature,
-                                                             const float* __restrict__ u) {
+                                                             const float* __restrict__ u, int* __restrict__ counts) {
     __shared__ float red[16];
     __shared__ float wsum[SBLOCK / 64];
     __shared__ int found;
@@ -420,19 +435,35 @@ __global__ __launch_bounds__(SBLOCK) void sample_draw_kernel(const float* __rest
     __syncthreads();
     for (int ww = 0; ww < SBLOCK / 64; ++ww) argmax_combine(bv, bi, sv[ww], si[ww]);
     if (bi == 0x7fffffff) bi = 0;
-    if (temperature[b] == 0.f) { if (threadIdx.x == 0) out[b] = bi; return; }
+    if (temperature[b] == 0.f) {
+        if (threadIdx.x == 0) { out[b] = bi; if (counts) counts[(size_t)b * V + bi] += 1; }
+        return;
+    }
     const float vmax = bv;
     float part = 0.f;
     for (int i = threadIdx.x; i < V; i += SBLOCK) part += expf(w[i] - vmax);
     const float sum = block_sum(part, red);
     const int hit = block_first_reach(V, u[b], [&](int i) { return expf(w[i] - vmax) / sum; }, wsum, &found);
-    if (threadIdx.x == 0) out[b] = hit < V ? hit : bi;
+    if (threadIdx.x == 0) {
+        const int tok = hit < V ? hit : bi;
+        out[b] = tok;
+        if (counts) counts[(size_t)b * V + tok] += 1;       // the row's history grows by its new token
+    }
 }
 
 extern "C" int br_sample_draw(const float* work, int* out, int B, int V, const float* temperature,
                               const float* u, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0) return BR_BAD_ARG;
-    sample_draw_kernel<<<B, SBLOCK, 0, s>>>(work, out, V, temperature, u);
+    sample_draw_kernel<<<B, SBLOCK, 0, s>>>(work, out, V, temperature, u, nullptr);
+    return br_check_launch();
+}
+
+// The same, and counts[b, token drawn] += 1 (the dense history of br_sample_prepare_dense; null: none).
+extern "C" int br_sample_draw_count(const float* work, int* out, int B, int V, const float* temperature,
+                                    const float* u, int* counts, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0) return BR_BAD_ARG;
+    sample_draw_kernel<<<B, SBLOCK, 0, s>>>(work, out, V, temperature, u, counts);
     return br_check_launch();
 }

@@ -191,9 +191,26 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
             results[i] = GenerationResult(out[i], reason, len(prompts[i]))
             engine.free_slot(slot.pop(i))      # an ended sequence leaves the batch at once
 
+        # the sampler of the live rows stays on the device from step to step (options, bias lists,
+        # histories); it is cut down to the rows that go on when some end
+        resident = {"rows": None, "state": None}
+
+        def draw(logits, live):
+            us = [uniform(seeds[i], i, len(out[i])) for i in live]
+            make = getattr(sampler, "state", None)
+            if make is None:
+                return sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live], us)
+            if resident["rows"] != live:
+                old = resident["rows"]
+                if old is not None and set(live) <= set(old):
+                    resident["state"] = resident["state"].keep([old.index(i) for i in live])
+                else:
+                    resident["state"] = make([plist[i] for i in live], [hist[i] for i in live])
+                resident["rows"] = list(live)
+            return resident["state"].sample(logits, us)
+
         def sample_and_book(logits, live, prefill):
-            toks = sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live],
-                                  [uniform(seeds[i], i, len(out[i])) for i in live])
+            toks = draw(logits, live)
             dt = time.perf_counter() - t0       # sampling returned the tokens: the step is done
             if prefill:
                 stats.prefill_tokens += sum(len(prompts[i]) for i in live)

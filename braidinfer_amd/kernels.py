@@ -539,13 +539,27 @@ def argmax_advance(logits: torch.Tensor, out: torch.Tensor, tokens: torch.Tensor
            "argmax_advance")
 
 
-def sample_prepare(logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature):
-    _dev("sample_prepare", logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature)
+def sample_prepare(logits, work, bias_off, bias_tok, bias_val, counts, penalty, temperature):
+    """work = logits with bias, repetition penalty and temperature applied.  `counts`: the rows'
+    histories as a table int32 [B, V] of occurrences per token on the device (None: no history)."""
+    _dev("sample_prepare", logits, work, bias_off, bias_tok, bias_val, counts, penalty, temperature)
     B, V = logits.shape
     _req(logits.dtype == torch.float32 and work.dtype == torch.float32 and work.shape == logits.shape, "sample_prepare: float32 [B, V]")
-    f = _fn("sampling", "br_sample_prepare", [_P, _P, c_int, c_int] + [_P] * 9)
-    _check(f(_ptr(logits), _ptr(work), B, V, _ptr(bias_off), _ptr(bias_tok), _ptr(bias_val), _ptr(hist_off),
-             _ptr(hist_tok), _ptr(hist_cnt), _ptr(penalty), _ptr(temperature), _stream()), "sample_prepare")
+    _req(counts is None or (counts.dtype == torch.int32 and counts.dim() == 2 and counts.shape[0] >= B and counts.shape[1] == V
+                            and counts.is_contiguous()), "sample_prepare: counts must be int32 [B, V]")
+    f = _fn("sampling", "br_sample_prepare", [_P, _P, c_int, c_int] + [_P] * 7)
+    _check(f(_ptr(logits), _ptr(work), B, V, _ptr(bias_off), _ptr(bias_tok), _ptr(bias_val), _ptr(counts), _ptr(penalty),
+             _ptr(temperature), _stream()), "sample_prepare")
+
+
+def sample_count_add(counts, rows, toks, cnts):
+    """counts[rows[e], toks[e]] += cnts[e]: puts histories into the table of `sample_prepare`."""
+    _dev("sample_count_add", counts, rows, toks, cnts)
+    n = rows.numel()
+    _req(counts.dtype == torch.int32 and counts.dim() == 2 and all(t.dtype == torch.int32 and t.numel() == n for t in (rows, toks, cnts)),
+         "sample_count_add: int32 counts [B, V] and three int32 lists of one length")
+    f = _fn("sampling", "br_sample_count_add", [_P, c_int, c_int, _P, _P, _P, c_int, _P])
+    _check(f(_ptr(counts), counts.shape[0], counts.shape[1], _ptr(rows), _ptr(toks), _ptr(cnts), n, _stream()), "sample_count_add")
 
 
 FILTER_CANDIDATES = 1024    # CAND in csrc/sampling.hip
@@ -581,9 +595,16 @@ def sample_filter_sort(work, keys, top_k, min_p, top_p, temperature):
            "sample_filter_sort")
 
 
-def sample_draw(work, out, temperature, u):
-    _dev("sample_draw", work, out, temperature, u)
+def sample_draw(work, out, temperature, u, counts=None):
+    """`counts` (int32 [B, V], optional): the table of `sample_prepare`; the token drawn
+    for a row is added to the row's history there."""
+    _dev("sample_draw", work, out, temperature, u, counts)
     B, V = work.shape
     _req(out.dtype == torch.int32 and u.dtype == torch.float32 and temperature.dtype == torch.float32, "sample_draw: dtypes")
-    f = _fn("sampling", "br_sample_draw", [_P, _P, c_int, c_int, _P, _P, _P])
-    _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(u), _stream()), "sample_draw")
+    if counts is None:
+        f = _fn("sampling", "br_sample_draw", [_P, _P, c_int, c_int, _P, _P, _P])
+        _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(u), _stream()), "sample_draw")
+        return
+    _req(counts.dtype == torch.int32 and counts.shape[0] >= B and counts.shape[1] == V, "sample_draw: counts must be int32 [B, V]")
+    f = _fn("sampling", "br_sample_draw_count", [_P, _P, c_int, c_int, _P, _P, _P, _P])
+    _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(u), _ptr(counts), _stream()), "sample_draw")

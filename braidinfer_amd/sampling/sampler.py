@@ -1,6 +1,12 @@
 """The sampler: rows of float logits on the device in, one token per row out, through
 the HIP kernels in csrc/sampling.hip.  Order of operations as the reference's `sample`
-(crates/braidinfer-runtime/src/sampling.rs:49-171)."""
+(crates/braidinfer-runtime/src/sampling.rs:49-171).
+
+`SamplerState` is the sampler of one fixed set of rows over many steps: the rows' options,
+their bias lists and their histories (a table of occurrences per token, for the repetition
+penalty) live on the device; a step brings only its uniform numbers, and the kernel that draws
+a token also adds it to the row's history.  `Sampler.sample` is the same for a single call.
+"""
 from __future__ import annotations
 
 from collections import Counter
@@ -13,22 +19,143 @@ from .. import kernels as K
 from .params import SamplingParams
 
 
-class Sampler:
-    def __init__(self, device, vocab_size: int):
-        self.device = torch.device(device)
-        self.V = int(vocab_size)
-        self._keys = None          # scratch for whole-row sorts, made when first needed
+class SamplerState:
+    def __init__(self, device, vocab_size: int, params: Sequence[SamplingParams],
+                 histories: Optional[Sequence[Sequence[int]]] = None, keys_cache: Optional[dict] = None):
+        self.device, self.V, self.params = torch.device(device), int(vocab_size), list(params)
+        B, V = len(self.params), self.V
+        self.B = B
+        self.greedy = all(p.is_plain_greedy for p in self.params)
+        self._keys_cache = keys_cache if keys_cache is not None else {}
+        self.out = torch.empty(B, dtype=torch.int32, device=self.device)
+        if self.greedy:
+            return
+        # the per-row numbers go over in one copy: four float rows and one int row
+        host = np.empty((5, B), dtype=np.float32)
+        host[0] = [p.temperature for p in self.params]
+        host[1] = [p.repetition_penalty for p in self.params]
+        host[2] = [p.min_p for p in self.params]
+        host[3] = [p.top_p for p in self.params]
+        host[4].view(np.int32)[:] = [p.top_k for p in self.params]
+        dev = torch.from_numpy(host).to(self.device)
+        self.temperature, self.penalty, self.min_p, self.top_p = dev[0], dev[1], dev[2], dev[3]
+        self.top_k = dev[4].view(torch.int32)
+        self.bias_off = self.bias_tok = self.bias_val = None
+        if any(p.logit_bias for p in self.params):
+            off, tok, val = [0], [], []
+            for p in self.params:
+                for t, d in (p.logit_bias or []):
+                    tok.append(int(t))
+                    val.append(float(d))
+                off.append(len(tok))
+            self.bias_off, self.bias_tok = self._i32(off), self._i32(tok or [0])
+            self.bias_val = torch.tensor(val or [0.0], dtype=torch.float32).to(self.device)
+        self.counts = None
+        if any(p.repetition_penalty != 1.0 for p in self.params):
+            self.counts = torch.zeros((B, V), dtype=torch.int32, device=self.device)
+            rows, toks, cnts = [], [], []
+            for b, (p, h) in enumerate(zip(self.params, histories or [[]] * B)):
+                if p.repetition_penalty != 1.0:
+                    for t, c in Counter(int(t) for t in h).items():
+                        rows.append(b)
+                        toks.append(t)
+                        cnts.append(c)
+            if rows:
+                K.sample_count_add(self.counts, self._i32(rows), self._i32(toks), self._i32(cnts))
+        self.filtered = any(p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)
+                            for p in self.params)
+        # rows that the short-list kernel may hand on need room for a sort of the whole row
+        self.needs_keys = any(p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)
+                              and (p.top_k > K.FILTER_CANDIDATES or (not 0 < p.top_k < V and p.top_p < 1.0))
+                              for p in self.params)
+        self.work = torch.empty((B, V), dtype=torch.float32, device=self.device)
+        self.slow = torch.empty(B, dtype=torch.int32, device=self.device)
+        self.u = torch.zeros(B, dtype=torch.float32, device=self.device)
+        self.u_host = torch.zeros(B, dtype=torch.float32, pin_memory=self.device.type == "cuda")
 
     def _i32(self, v):
         return torch.tensor(v, dtype=torch.int32).to(self.device)
 
-    def _f32(self, v):
-        return torch.tensor(v, dtype=torch.float32).to(self.device)
+    def _keys(self):
+        n2 = 1 << (self.V - 1).bit_length()
+        k = self._keys_cache.get("keys")
+        if k is None or k.shape[0] < self.B or k.shape[1] != n2:
+            k = self._keys_cache["keys"] = torch.empty((self.B, n2), dtype=torch.int64, device=self.device)
+        return k
+
+    def launch(self, logits: torch.Tensor, us: Optional[Sequence[float]] = None) -> torch.Tensor:
+        """Enqueue the sampling of one step; returns the device tensor the tokens will stand in
+        (int32 [B], overwritten by the next launch).  `us[b]` is row b's uniform number in [0, 1)."""
+        B, V = logits.shape
+        assert V == self.V and B == self.B
+        if self.greedy:
+            K.argmax(logits, self.out)
+            return self.out
+        if us is not None:
+            self.u_host.numpy()[:] = us
+            self.u.copy_(self.u_host, non_blocking=True)
+        K.sample_prepare(logits, self.work, self.bias_off, self.bias_tok, self.bias_val, self.counts, self.penalty,
+                         self.temperature)
+        if self.filtered:
+            K.sample_filter(self.work, self.top_k, self.min_p, self.top_p, self.temperature, self.slow,
+                            self._keys() if self.needs_keys else None)
+        K.sample_draw(self.work, self.out, self.temperature, self.u, self.counts)
+        return self.out
+
+    def sample(self, logits: torch.Tensor, us: Optional[Sequence[float]] = None) -> List[int]:
+        return self.launch(logits, us).tolist()
+
+    def keep(self, rows: Sequence[int]) -> "SamplerState":
+        """The state of a subset of the rows (those that go on), in the given order; histories
+        stay on the device."""
+        st = SamplerState.__new__(SamplerState)
+        st.device, st.V, st.params = self.device, self.V, [self.params[r] for r in rows]
+        st.B, st.greedy, st._keys_cache = len(rows), self.greedy, self._keys_cache
+        st.out = torch.empty(st.B, dtype=torch.int32, device=self.device)
+        if self.greedy:
+            return st
+        idx = torch.tensor(list(rows), dtype=torch.long, device=self.device)
+        pick = lambda t: t.index_select(0, idx)
+        st.temperature, st.penalty, st.min_p, st.top_p, st.top_k = (pick(t) for t in (
+            self.temperature, self.penalty, self.min_p, self.top_p, self.top_k))
+        st.bias_off = st.bias_tok = st.bias_val = None
+        if self.bias_off is not None:
+            off = self.bias_off.tolist()
+            tok, val = self.bias_tok.tolist(), self.bias_val.tolist()
+            noff, ntok, nval = [0], [], []
+            for r in rows:
+                ntok += tok[off[r]:off[r + 1]]
+                nval += val[off[r]:off[r + 1]]
+                noff.append(len(ntok))
+            st.bias_off, st.bias_tok = st._i32(noff), st._i32(ntok or [0])
+            st.bias_val = torch.tensor(nval or [0.0], dtype=torch.float32).to(self.device)
+        st.counts = pick(self.counts) if self.counts is not None else None
+        V = self.V
+        flt = lambda p: p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)
+        st.filtered = any(flt(p) for p in st.params)
+        st.needs_keys = any(flt(p) and (p.top_k > K.FILTER_CANDIDATES or (not 0 < p.top_k < V and p.top_p < 1.0))
+                            for p in st.params)
+        st.work = self.work[:st.B]
+        st.slow = self.slow[:st.B]
+        st.u = torch.zeros(st.B, dtype=torch.float32, device=self.device)
+        st.u_host = torch.zeros(st.B, dtype=torch.float32, pin_memory=self.device.type == "cuda")
+        return st
+
+
+class Sampler:
+    def __init__(self, device, vocab_size: int):
+        self.device = torch.device(device)
+        self.V = int(vocab_size)
+        self._scratch: dict = {}       # scratch for whole-row sorts, made when first needed and shared by the states
 
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
         K.argmax(logits, out)
         return out
+
+    def state(self, params: Sequence[SamplingParams], histories: Optional[Sequence[Sequence[int]]] = None) -> SamplerState:
+        """The resident sampler of these rows: `state.sample(logits, us)` step after step."""
+        return SamplerState(self.device, self.V, params, histories, self._scratch)
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                histories: Optional[Sequence[Sequence[int]]] = None,
@@ -37,53 +164,4 @@ class Sampler:
         penalty), `us[b]` the row's uniform number in [0, 1)."""
         B, V = logits.shape
         assert V == self.V and len(params) == B
-        if all(p.is_plain_greedy for p in params):
-            return self.argmax(logits).tolist()
-        histories = histories if histories is not None else [[] for _ in range(B)]
-        us = us if us is not None else [0.0] * B
-        work = torch.empty_like(logits)
-        bias_off = bias_tok = bias_val = None
-        if any(p.logit_bias for p in params):
-            off, tok, val = [0], [], []
-            for p in params:
-                for t, d in (p.logit_bias or []):
-                    tok.append(int(t))
-                    val.append(float(d))
-                off.append(len(tok))
-            bias_off, bias_tok, bias_val = self._i32(off), self._i32(tok or [0]), self._f32(val or [0.0])
-        hist_off = hist_tok = hist_cnt = None
-        if any(p.repetition_penalty != 1.0 for p in params):
-            off, tok, cnt = [0], [], []
-            for p, h in zip(params, histories):
-                if p.repetition_penalty != 1.0:
-                    for t, c in Counter(int(t) for t in h).items():
-                        tok.append(t)
-                        cnt.append(c)
-                off.append(len(tok))
-            hist_off, hist_tok, hist_cnt = self._i32(off), self._i32(tok or [0]), self._i32(cnt or [0])
-        # the per-row numbers go over in one copy: five float rows and one int row
-        host = np.empty((6, B), dtype=np.float32)
-        host[0] = [p.temperature for p in params]
-        host[1] = [p.repetition_penalty for p in params]
-        host[2] = [p.min_p for p in params]
-        host[3] = [p.top_p for p in params]
-        host[4] = list(us)
-        host[5].view(np.int32)[:] = [p.top_k for p in params]
-        dev = torch.from_numpy(host).to(self.device)
-        temperature, penalty, min_p, top_p, u = dev[0], dev[1], dev[2], dev[3], dev[4]
-        top_k = dev[5].view(torch.int32)
-        K.sample_prepare(logits, work, bias_off, bias_tok, bias_val, hist_off, hist_tok, hist_cnt, penalty, temperature)
-        filtered = [p for p in params if p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)]
-        if filtered:
-            # rows that the short-list kernel may hand on need room for a sort of the whole row
-            keys = None
-            if any(p.top_k > K.FILTER_CANDIDATES or (not 0 < p.top_k < V and p.top_p < 1.0) for p in filtered):
-                n2 = 1 << (V - 1).bit_length()
-                if self._keys is None or self._keys.shape[0] < B:
-                    self._keys = torch.empty((B, n2), dtype=torch.int64, device=self.device)
-                keys = self._keys
-            slow = torch.empty(B, dtype=torch.int32, device=self.device)
-            K.sample_filter(work, top_k, min_p, top_p, temperature, slow, keys)
-        out = torch.empty(B, dtype=torch.int32, device=self.device)
-        K.sample_draw(work, out, temperature, u)
-        return out.tolist()
+        return self.state(params, histories).sample(logits, us if us is not None else [0.0] * B)

@@ -152,3 +152,10 @@ def test_a_layer_names_its_norms_by_role_and_its_tensors_by_the_builder():
     # nothing in the neutral description carries a checkpoint's names of its own
     bare = B.LayerSpec("p.")
     assert bare.names == {} and bare.norms == {} and bare.mixer is None
+
+
+def test_scaled_rotary_frequencies_are_refused_not_ignored():
+    B.MistralConfig.from_dict(dict(TINY["a"], rope_scaling=None))
+    B.MistralConfig.from_dict(dict(TINY["a"], rope_scaling={"rope_type": "default"}))
+    with pytest.raises(B.ConfigError, match="rope_scaling"):
+        B.MistralConfig.from_dict(dict(TINY["a"], rope_scaling={"rope_type": "yarn", "factor": 4.0}))

@@ -147,3 +147,36 @@ def test_filter_short_list_and_whole_row_sort_agree_with_the_plain_filter(V):
         assert slow[flat_top_p[0]] == 1       # 1024 equal entries of 32773 do not reach 0.9
         peaked_top_p = [b for b, c in enumerate(cases) if c[0].startswith("peaked k=0 min_p=0.0 top_p=0.3")]
         assert slow[peaked_top_p[0]] == 0
+
+
+def test_a_resident_state_keeps_its_rows_histories_on_the_device():
+    """Step after step with only the uniform numbers coming from the host: every drawn token
+    joins its row's history (what the repetition penalty sees), rows that end are dropped with
+    `keep`, and each step equals the plain sampler given the history so far."""
+    V, B = 500, 6
+    rng = np.random.default_rng(3)
+    params = [SamplingParams(temperature=[0.8, 1.0, 0.0][b % 3], top_k=[0, 20][b % 2], top_p=1.0, min_p=0.0,
+                             repetition_penalty=[1.5, 1.0, 1.2][b % 3],
+                             logit_bias=[(b, 1.0), (b + 1, -2.0)] if b in (1, 4) else None) for b in range(B)]
+    hists = [[int(t) for t in rng.integers(0, V, 12)] + [7, 7] for _ in range(B)]
+    state = Sampler(DEV, V).state(params, hists)
+    rows = list(range(B))
+    for step in range(8):
+        logits = rng.normal(size=(len(rows), V)).astype(np.float32) * 2
+        logits[:, 7] += 3.0                                  # a token that is in every history and would win unpenalised
+        us = [float(rng.random()) for _ in rows]
+        got = state.sample(torch.tensor(logits).to(DEV), us)
+        for r, b in enumerate(rows):
+            p = params[b]
+            want = P.sample(logits[r], us[r], p.temperature, p.top_k, p.top_p, p.min_p, p.repetition_penalty, hists[b],
+                            p.logit_bias)
+            near = [P.sample(logits[r], min(max(us[r] + d, 0.0), 0.999999), p.temperature, p.top_k, p.top_p, p.min_p,
+                             p.repetition_penalty, hists[b], p.logit_bias) for d in (-2e-6, 2e-6)]
+            assert got[r] == want or got[r] in near, f"step {step}, row {b}"
+            hists[b].append(got[r])
+        if step == 2:
+            rows = [0, 2, 3, 5]
+            state = state.keep([0, 2, 3, 5])
+        if step == 5:
+            rows = [5, 0]                                    # another order, too
+            state = state.keep([3, 0])
