@@ -701,3 +701,63 @@ def test_single_token_steps_of_many_requests(serving, live):
         ref = P.forward(cfg, w, seqs[i])[lens[i] - 1:]
         close(got[True][i], ref, "bfloat16", f"request {i} of {live}, graphs")
         assert np.abs(got[True][i] - got[False][i]).max() <= CUT_TOL["bfloat16"] * np.abs(ref).max()
+
+
+# ------------------------------------------------- the layer sizes of the benchmark's shape ----
+@pytest.fixture(scope="module")
+def real_sizes(tmp_path_factory):
+    """Two layers of the Mistral-7B-v0.3 shape (hidden 4096, 32 heads over 8 kv heads of 128,
+    intermediate 14336, vocabulary 32768): the matrices that the benchmark's kernels multiply."""
+    folder = str(tmp_path_factory.mktemp("real_sizes"))
+    cfg = B.preset("mistral-7b-v0.3", num_hidden_layers=2)
+    B.Engine.write_random_folder(folder, cfg, seed=17, std=0.02, vector_jitter=0.3, device="cuda:0")
+    pc, w = P.read_folder(folder)
+    return folder, pc, w
+
+
+def test_real_layer_sizes_prompt_single_steps_and_a_batch(real_sizes):
+    """bfloat16 at the sizes the benchmark runs (tiles of 256x256, 256x192 and 128x256 for the
+    prompt, the streaming products over rows and over blocks of 16 rows for 1 to 16 and 17 to
+    64 sequences, attention through the LDS rings): a prompt of 300 tokens whole, its last
+    tokens one by one, and 20 requests of unequal lengths decoding together, all against the
+    plain implementation."""
+    folder, cfg, w = real_sizes
+    eng = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=8192)
+    assert eng.model.layers[0].feed_forward.w_gu.dim() == 4 and eng.model.lm_head.weight.dim() == 4      # blocked layout
+    toks = tokens(cfg, 300, 21)
+    ref = P.forward(cfg, w, toks)
+    close(whole(eng, toks), ref, "bfloat16", "7B sizes, whole prompt")
+    s = eng.alloc_slot()
+    parts = [eng.step([StepEntry(s, toks[:292], [291])]).cpu().numpy()]
+    for t in toks[292:]:
+        parts.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    eng.free_slot(s)
+    close(np.concatenate(parts), ref[291:], "bfloat16", "7B sizes, last tokens one by one")
+    lens = [3 + 9 * i for i in range(20)]
+    seqs = [tokens(cfg, n + 3, 400 + i) for i, n in enumerate(lens)]
+    slots = [eng.alloc_slot() for _ in seqs]
+    got = [[] for _ in seqs]
+    out = eng.step([StepEntry(sl, q[:n], [n - 1]) for sl, q, n in zip(slots, seqs, lens)]).cpu().numpy()
+    for i in range(20):
+        got[i].append(out[i:i + 1])
+    for k in range(3):
+        out = eng.step([StepEntry(sl, [q[n + k]], [0]) for sl, q, n in zip(slots, seqs, lens)]).cpu().numpy()
+        for i in range(20):
+            got[i].append(out[i:i + 1])
+    for sl in slots:
+        eng.free_slot(sl)
+    for i in (0, 11, 19):
+        close(np.concatenate(got[i]), P.forward(cfg, w, seqs[i])[lens[i] - 1:], "bfloat16", f"7B sizes, request {i} of 20")
+
+
+def test_real_layer_sizes_in_32_bit(real_sizes):
+    folder, cfg, w = real_sizes
+    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=1024)
+    toks = tokens(cfg, 70, 22)
+    ref = P.forward(cfg, w, toks)
+    s = eng.alloc_slot()
+    parts = [eng.step([StepEntry(s, toks[:66], list(range(66)))]).cpu().numpy()]
+    for t in toks[66:]:
+        parts.append(eng.step([StepEntry(s, [t], [0])]).cpu().numpy())
+    eng.free_slot(s)
+    close(np.concatenate(parts), ref, "float32", "7B sizes in 32-bit")
