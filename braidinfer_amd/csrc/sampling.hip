@@ -74,6 +74,26 @@ extern "C" int br_argmax_advance(const float* logits, int* out, int B, int V, in
     return br_check_launch();
 }
 
+// The step arrays of n live rows moved on by the tokens a sampler drew for them: tokens[i] =
+// drawn[i], the row's position and length one more (what ADVANCE does for the argmax).
+__global__ void step_advance_kernel(const int* __restrict__ drawn, int* __restrict__ tokens, int* __restrict__ positions,
+                                    const int* __restrict__ slots, int* __restrict__ ctx, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && slots[i] >= 0) {
+        tokens[i] = drawn[i];
+        positions[i] += 1;
+        ctx[i] += 1;
+    }
+}
+
+extern "C" int br_step_advance(const int* drawn, int* tokens, int* positions, const int* slots, int* ctx, int n,
+                               hipStream_t s) {
+    if (n <= 0) return BR_OK;
+    if (!drawn || !tokens || !positions || !slots || !ctx) return BR_BAD_ARG;
+    step_advance_kernel<<<(n + 255) / 256, 256, 0, s>>>(drawn, tokens, positions, slots, ctx, n);
+    return br_check_launch();
+}
+
 // --------------------------------------------------- bias, penalty, temperature ----
 // work[b, :] = logits[b, :]; then per row, in the reference's order (sampling.rs:57-87):
 // bias entries (token, delta) are added; every history token's logit is divided by the

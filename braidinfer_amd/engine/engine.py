@@ -212,10 +212,11 @@ class Engine:
         self.cache.commit(slots, new)
         return logits
 
-    def greedy_chain(self, slots: Sequence[int], tokens: Sequence[int]):
-        """A `GreedyChain` over these sequences, each with the token it takes next, or None when
+    def chain(self, slots: Sequence[int], tokens: Sequence[int], sampler_state=None):
+        """A `DecodeChain` over these sequences, each with the token it takes next, or None when
         single-token steps of this engine are not replayed from graphs (then `step` and the
-        sampler do the same work one step at a time)."""
+        sampler do the same work one step at a time).  Without `sampler_state` the chain is greedy;
+        with one (`Sampler.state` of these rows, in this order) it draws through that state."""
         if not self.use_graphs or len(slots) > 256:
             return None
         V = self.vocab_size
@@ -225,8 +226,11 @@ class Engine:
         if self._graphs is None:
             from .graph import DecodeGraphs
             self._graphs = DecodeGraphs(self.model, self.cache, self.device)
-        from .graph import GreedyChain
-        return GreedyChain(self._graphs, self.cache, slots, tokens)
+        from .graph import DecodeChain
+        return DecodeChain(self._graphs, self.cache, slots, tokens, sampler_state)
+
+    def greedy_chain(self, slots: Sequence[int], tokens: Sequence[int]):
+        return self.chain(slots, tokens)
 
     # ---- generation (the Python entry point) -----------------------------------------------
     def generate(self, prompts, max_new_tokens: int = 64, temperature: float = 0.0, seed=None,

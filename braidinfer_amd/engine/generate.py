@@ -76,20 +76,26 @@ def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, capacity_token
     return batches
 
 
-def _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0):
-    """Greedy steps of the requests `live` through a chain until one of them ends; returns
-    those that go on.  A second step is launched before the first one's tokens are read
-    whenever no request can end for a reason known beforehand (its budget, the longest
-    sequence the cache takes); a request that meets a stop token has then been given one
-    token too many, which is dropped with its slot."""
+def _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0, us_of=None):
+    """Steps of the requests `live` through a chain until one of them ends; returns those
+    that go on.  A second step is launched before the first one's tokens are read whenever
+    no request can end for a reason known beforehand (its budget, the longest sequence the
+    cache takes); a request that meets a stop token has then been given one token too many,
+    which is dropped with its slot.  `us_of(ahead)`: the uniform numbers of a step launched
+    while `ahead` steps are unread (a sampled chain), None for a greedy one."""
+    def launch(ahead):
+        if us_of is None:
+            chain.launch()
+        else:
+            chain.launch(us_of(ahead))
     try:
-        chain.launch()
+        launch(0)
         launched, read = 1, 0
         while True:
             ahead = launched - read              # steps whose tokens are still to come
             if ahead < 2 and all(len(out[i]) + ahead + 1 <= max_new_tokens
                                  and engine.length(slot[i]) + 1 <= cache.max_seq_len for i in live):
-                chain.launch()
+                launch(ahead)
                 launched += 1
             toks = chain.read()
             read += 1
@@ -103,7 +109,7 @@ def _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cac
                 if reason is not None:
                     ended[i] = reason
             if not ended and launched == read:
-                chain.launch()
+                launch(0)
                 launched += 1
                 continue
             if not ended:
@@ -195,19 +201,23 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
         # histories); it is cut down to the rows that go on when some end
         resident = {"rows": None, "state": None}
 
-        def draw(logits, live):
-            us = [uniform(seeds[i], i, len(out[i])) for i in live]
-            make = getattr(sampler, "state", None)
-            if make is None:
-                return sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live], us)
+        make_state = getattr(sampler, "state", None)
+
+        def state_of(live):
             if resident["rows"] != live:
                 old = resident["rows"]
                 if old is not None and set(live) <= set(old):
                     resident["state"] = resident["state"].keep([old.index(i) for i in live])
                 else:
-                    resident["state"] = make([plist[i] for i in live], [hist[i] for i in live])
+                    resident["state"] = make_state([plist[i] for i in live], [hist[i] for i in live])
                 resident["rows"] = list(live)
-            return resident["state"].sample(logits, us)
+            return resident["state"]
+
+        def draw(logits, live):
+            us = [uniform(seeds[i], i, len(out[i])) for i in live]
+            if make_state is None:
+                return sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live], us)
+            return state_of(live).sample(logits, us)
 
         def sample_and_book(logits, live, prefill):
             toks = draw(logits, live)
@@ -231,14 +241,22 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
             t0 = time.perf_counter()
             logits = engine.step([StepEntry(slot[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
             live = sample_and_book(logits, live, True)
-            # plain greedy requests decode through a chain when the engine has one: a step's tokens feed
-            # the next step on the device, and the host reads them one step behind
-            open_chain = getattr(engine, "greedy_chain", None) if all(plist[i].is_plain_greedy for i in live) else None
+            # requests decode through a chain when the engine has one: a step's tokens feed the next
+            # step on the device, and the host reads them one step behind.  Plain greedy requests
+            # take the argmax inside the recorded step; others draw through the resident sampler
+            open_chain = getattr(engine, "chain", None)
             while live:
                 t0 = time.perf_counter()
-                chain = open_chain([slot[i] for i in live], [out[i][-1] for i in live]) if open_chain else None
+                chain = us_of = None
+                if open_chain is not None:
+                    rows = list(live)
+                    if all(plist[i].is_plain_greedy for i in rows):
+                        chain = open_chain([slot[i] for i in rows], [out[i][-1] for i in rows])
+                    elif make_state is not None:
+                        chain = open_chain([slot[i] for i in rows], [out[i][-1] for i in rows], state_of(rows))
+                        us_of = lambda ahead: [uniform(seeds[i], i, len(out[i]) + ahead) for i in rows]
                 if chain is not None:
-                    live = _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0)
+                    live = _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0, us_of)
                 else:
                     logits = engine.step([StepEntry(slot[i], [out[i][-1]], [0]) for i in live])
                     live = sample_and_book(logits, live, False)

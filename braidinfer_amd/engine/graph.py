@@ -151,19 +151,27 @@ class DecodeGraphs:
         return self.of(len(slots)).run(slots, tokens, starts)
 
 
-class GreedyChain:
-    """Greedy single-token steps of one fixed set of sequences with the host out of the way:
-    a step's tokens go into the next step's input on the device, so a step can be launched
+class DecodeChain:
+    """Single-token steps of one fixed set of sequences with the host out of the way: a
+    step's tokens go into the next step's input on the device, so a step can be launched
     before the tokens of the one before have been read.  `launch` runs one step for every
     sequence (reserving cache pages first, as `Engine.step` does); `read` returns the tokens of
     the oldest launched step that has not been read.  At most two steps may be unread.
 
+    Without a sampler state the tokens are the argmax of each row, taken inside the recorded
+    step.  With one (`sampling.SamplerState` of these rows, in the order of `slots`) the recorded
+    step is followed by the state's kernels and by one that moves the step's arrays on by the
+    drawn tokens; `launch(us)` then brings the step's uniform numbers.
+
     The chain owns the recorded step of its batch size until it is closed or any other
     single-token step of that size runs, after which `launch` refuses."""
 
-    def __init__(self, graphs: DecodeGraphs, cache, slots: Sequence[int], tokens: Sequence[int]):
+    def __init__(self, graphs: DecodeGraphs, cache, slots: Sequence[int], tokens: Sequence[int], sampler_state=None):
         if not slots or len(slots) != len(tokens) or len(set(slots)) != len(slots):
             raise StepError("a chain needs one token for each of its distinct slots")
+        if sampler_state is not None and sampler_state.B != len(slots):
+            raise StepError(f"a sampler state of {sampler_state.B} rows for a chain of {len(slots)} sequences")
+        self.state = sampler_state
         self.cache, self.slots, self.n = cache, list(slots), len(slots)
         for s in self.slots:
             cache.slots.check_live(s)
@@ -175,7 +183,17 @@ class GreedyChain:
         self.turn = 0
         self.pending = deque()
 
-    def launch(self) -> None:
+    def _run(self, us) -> torch.Tensor:
+        g, n = self.g, self.n
+        if self.state is None:
+            g.run_greedy()
+            return g.next_tokens[:n]
+        g.graph.replay()
+        drawn = self.state.launch(g.logits[:n], us)
+        K.step_advance(drawn, g.step.tokens, g.step.positions, g.step.slots, g.step.ctx_lens, n)
+        return drawn
+
+    def launch(self, us: Sequence[float] = None) -> None:
         if self.g.owner is not self:
             raise StepError("this chain's recorded step has been used by another step since; open a new chain")
         if len(self.pending) >= 2:
@@ -183,14 +201,14 @@ class GreedyChain:
         held = self.cache.pages_held()
         self.cache.reserve(self.slots, self.ones)
         try:
-            self.g.run_greedy()
+            drawn = self._run(us)
         except BaseException:
             self.cache.release_reserved(self.slots, held)
             raise
         self.cache.commit(self.slots, self.ones)
         buf = self.host[self.turn]
         self.turn ^= 1
-        buf.copy_(self.g.next_tokens, non_blocking=True)
+        buf[:self.n].copy_(drawn, non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
         self.pending.append((ev, buf))
@@ -208,3 +226,6 @@ class GreedyChain:
             self.pending.popleft()[0].synchronize()
         if self.g.owner is self:
             self.g.owner = None
+
+
+GreedyChain = DecodeChain

@@ -539,6 +539,17 @@ def argmax_advance(logits: torch.Tensor, out: torch.Tensor, tokens: torch.Tensor
            "argmax_advance")
 
 
+def step_advance(drawn: torch.Tensor, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                 ctx_lens: torch.Tensor, n: int) -> None:
+    """For the first n rows that are live (slot >= 0): tokens[i] = drawn[i], positions[i] and
+    ctx_lens[i] one more: the next single-token step's arrays from the tokens a sampler drew."""
+    _dev("step_advance", drawn, tokens, positions, slots, ctx_lens)
+    _req(all(t.dtype == torch.int32 and t.numel() >= n for t in (drawn, tokens, positions, slots, ctx_lens)),
+         "step_advance: int32 arrays of at least n entries")
+    f = _fn("sampling", "br_step_advance", [_P, _P, _P, _P, _P, c_int, _P])
+    _check(f(_ptr(drawn), _ptr(tokens), _ptr(positions), _ptr(slots), _ptr(ctx_lens), int(n), _stream()), "step_advance")
+
+
 def sample_prepare(logits, work, bias_off, bias_tok, bias_val, counts, penalty, temperature):
     """work = logits with bias, repetition penalty and temperature applied.  `counts`: the rows'
     histories as a table int32 [B, V] of occurrences per token on the device (None: no history)."""

@@ -70,8 +70,16 @@ class SamplerState:
                               for p in self.params)
         self.work = torch.empty((B, V), dtype=torch.float32, device=self.device)
         self.slow = torch.empty(B, dtype=torch.int32, device=self.device)
-        self.u = torch.zeros(B, dtype=torch.float32, device=self.device)
-        self.u_host = torch.zeros(B, dtype=torch.float32, pin_memory=self.device.type == "cuda")
+        self._make_u()
+
+    def _make_u(self):
+        # the step's uniform numbers: two pinned buffers used in turn, so that a step can be
+        # launched while the copy of the step before may still be waiting in the stream
+        self.u = torch.zeros(self.B, dtype=torch.float32, device=self.device)
+        pinned = self.device.type == "cuda"
+        self.u_host = [torch.zeros(self.B, dtype=torch.float32, pin_memory=pinned) for _ in range(2)]
+        self.u_copied = [None, None]
+        self.u_turn = 0
 
     def _i32(self, v):
         return torch.tensor(v, dtype=torch.int32).to(self.device)
@@ -92,8 +100,16 @@ class SamplerState:
             K.argmax(logits, self.out)
             return self.out
         if us is not None:
-            self.u_host.numpy()[:] = us
-            self.u.copy_(self.u_host, non_blocking=True)
+            k = self.u_turn
+            self.u_turn ^= 1
+            if self.u_copied[k] is not None:
+                self.u_copied[k].synchronize()
+            self.u_host[k].numpy()[:] = us
+            self.u.copy_(self.u_host[k], non_blocking=True)
+            if self.device.type == "cuda":
+                if self.u_copied[k] is None:
+                    self.u_copied[k] = torch.cuda.Event()
+                self.u_copied[k].record()
         K.sample_prepare(logits, self.work, self.bias_off, self.bias_tok, self.bias_val, self.counts, self.penalty,
                          self.temperature)
         if self.filtered:
@@ -137,8 +153,7 @@ class SamplerState:
                             for p in st.params)
         st.work = self.work[:st.B]
         st.slow = self.slow[:st.B]
-        st.u = torch.zeros(st.B, dtype=torch.float32, device=self.device)
-        st.u_host = torch.zeros(st.B, dtype=torch.float32, pin_memory=self.device.type == "cuda")
+        st._make_u()
         return st
 
 

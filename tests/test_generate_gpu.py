@@ -94,6 +94,64 @@ def test_greedy_through_the_chain_equals_greedy_step_by_step(tiny_folders):
     assert free_run[0] == P.greedy_generate(cfg, w, prompts[0], 70)
 
 
+def test_sampled_through_the_chain_equals_sampled_step_by_step(tiny_folders):
+    """Sampled requests decode through a chain too: the recorded step, the resident sampler's
+    kernels and the move to the next step's arrays, one step launched ahead.  Every option of
+    the sampler, mixed in one batch with greedy rows, stop tokens and the context's end: the
+    tokens and reasons of single steps."""
+    from braidinfer_amd.engine import generate
+    from braidinfer_amd.sampling import SamplingParams
+    folder, cfg, w = tiny_folders["b"]
+    with_chain = B.Engine.from_folder(folder, dtype="float32", max_tokens=4096, max_seq_len=160)
+    without = B.Engine.from_folder(folder, dtype="float32", max_tokens=4096, max_seq_len=160, use_graphs=False)
+    prompts = prompts_of(cfg, [3, 60, 17, 120, 1, 63, 150, 9], 6)
+    V = cfg["vocab_size"]
+    params = [SamplingParams(temperature=0.8, top_k=0, seed=5),
+              SamplingParams(temperature=1.0, top_k=7, seed=5),
+              SamplingParams(temperature=0.9, top_k=0, top_p=0.8, seed=6),
+              SamplingParams(temperature=0.0, top_k=0, repetition_penalty=1.3),
+              SamplingParams.greedy(),
+              SamplingParams(temperature=1.1, top_k=0, min_p=0.05, repetition_penalty=1.2, seed=7),
+              SamplingParams(temperature=0.7, top_k=40, top_p=0.9, seed=8, logit_bias=[(3, 4.0), (V - 1, -2.0)]),
+              SamplingParams(temperature=1.0, top_k=V + 5, seed=9)]
+    free_run, _ = generate(without, prompts, params, max_new_tokens=50, stop_token_ids=[])
+    stop = free_run[2].tokens[7]
+    for kw in (dict(max_new_tokens=50, stop_token_ids=[]), dict(max_new_tokens=50, stop_token_ids=[stop]),
+               dict(max_new_tokens=6, stop_token_ids=[stop], include_stop=True), dict(max_new_tokens=2, stop_token_ids=[])):
+        a, sa = generate(without, prompts, params, **kw)
+        b, sb = generate(with_chain, prompts, params, **kw)
+        assert [(r.tokens, r.finish_reason) for r in a] == [(r.tokens, r.finish_reason) for r in b], kw
+        assert sb.decode_tokens >= sa.decode_tokens
+        for eng in (with_chain, without):
+            assert all(g.pool.held_count == 0 for g in eng.cache.groups) and eng.cache.slots.free_count == eng.cache.n_slots
+    assert free_run[6].finish_reason == "context" and len(free_run[6].tokens) == 43
+    assert len({tuple(r.tokens) for r in free_run}) == len(prompts)
+    # a chain of these rows by hand: two launches ahead of the first read, uniform numbers per launch
+    eng = with_chain
+    slots = [eng.alloc_slot() for _ in range(2)]
+    eng.step([B.StepEntry(s, p, []) for s, p in zip(slots, prompts[:2])])
+    from braidinfer_amd.sampling import Sampler
+    state = Sampler(eng.device, V).state(params[:2], [list(p) for p in prompts[:2]])
+    with pytest.raises(B.StepError, match="rows"):
+        eng.chain(slots[:1], [1], state)
+    chain = eng.chain(slots, [1, 2], state)
+    chain.launch([0.25, 0.5])
+    chain.launch([0.75, 0.125])
+    t1, t2 = chain.read(), chain.read()
+    chain.close()
+    for s in slots:
+        eng.free_slot(s)
+    # the same two steps one at a time through the step function and a fresh state
+    slots = [eng.alloc_slot() for _ in range(2)]
+    eng.step([B.StepEntry(s, p, []) for s, p in zip(slots, prompts[:2])])
+    state = Sampler(eng.device, V).state(params[:2], [list(p) for p in prompts[:2]])
+    s1 = state.sample(eng.step([B.StepEntry(s, [t], [0]) for s, t in zip(slots, [1, 2])]), [0.25, 0.5])
+    s2 = state.sample(eng.step([B.StepEntry(s, [t], [0]) for s, t in zip(slots, s1)]), [0.75, 0.125])
+    assert (t1, t2) == (s1, s2)
+    for s in slots:
+        eng.free_slot(s)
+
+
 def test_the_chain_by_hand(tiny_folders):
     folder, cfg, w = tiny_folders["a"]
     eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=1024)

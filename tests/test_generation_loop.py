@@ -166,15 +166,18 @@ def test_uniform_numbers_depend_only_on_seed_sequence_and_draw():
 
 # ---- greedy requests through a chain: the host reads a step behind -------------------------
 class FakeChain:
-    """What `Engine.greedy_chain` hands out, with the stand-in model: every launch feeds each
+    """What `Engine.chain` hands out, with the stand-in model: every launch feeds each
     row the token the launch before gave it, whether or not the host has read it yet."""
 
-    def __init__(self, engine, slots, tokens):
+    def __init__(self, engine, slots, tokens, state=None):
         self.e, self.slots, self.tokens, self.unread, self.closed = engine, list(slots), list(tokens), [], False
+        self.state, self.us = state, []
         engine.chains.append(self)
 
-    def launch(self):
+    def launch(self, us=None):
         assert not self.closed and len(self.unread) < 2
+        assert (us is None) == (self.state is None)
+        self.us.append(us)
         for s in self.slots:
             assert s in self.e.live, "a step for a slot that was given back"
             self.e.live[s] += 1
@@ -196,8 +199,8 @@ class ChainEngine(FakeEngine):
         super().__init__(*a, **k)
         self.chains, self.launched_ahead = [], 0
 
-    def greedy_chain(self, slots, tokens):
-        return FakeChain(self, slots, tokens)
+    def chain(self, slots, tokens, state=None):
+        return FakeChain(self, slots, tokens, state)
 
 
 def test_a_chain_gives_the_tokens_of_single_steps_for_every_way_of_ending():
@@ -227,7 +230,39 @@ def test_a_chain_runs_a_step_ahead_only_when_nobody_can_end_for_a_known_reason()
     res, _ = run(e, [[46], [10]], max_new_tokens=8)           # request 0 meets the stop token 0 on its fourth token
     assert res[0].tokens == [47, 48, 49] and res[0].finish_reason == "stop" and res[1].tokens == list(range(11, 19))
     assert len(e.chains) == 2 and e.chains[0].slots == [0, 1] and e.chains[1].slots == [1]
-    # sampled requests do not use the chain
+    # sampled requests do not use the chain when the sampler keeps no state on the device
     e = ChainEngine()
     run(e, [[5]], max_new_tokens=3, stop_token_ids=[], params=SamplingParams(temperature=0.5, seed=1))
     assert not e.chains
+
+
+class FakeState:
+    def __init__(self, rows):
+        self.rows = list(rows)
+
+    def sample(self, logits, us):
+        return [int(r.argmax()) for r in logits]
+
+    def keep(self, rows):
+        return FakeState([self.rows[r] for r in rows])
+
+
+class StateSampler:
+    def state(self, params, histories):
+        return FakeState(range(len(params)))
+
+
+def test_a_sampled_chain_brings_each_step_the_uniform_numbers_of_its_draws():
+    """Draw k of request i uses uniform(seed, i, k) whether it is launched ahead or not, and the
+    state handed to a chain is that of the rows that go on."""
+    p = SamplingParams(temperature=0.5, seed=11)
+    e = ChainEngine()
+    res, _ = generate(e, [[46], [10]], params=p, max_new_tokens=6, sampler=StateSampler())
+    assert res[0].tokens == [47, 48, 49] and res[0].finish_reason == "stop" and res[1].tokens == list(range(11, 17))
+    first, second = e.chains
+    assert first.state.rows == [0, 1] and second.state.rows == [1]
+    # the first token comes from the prompt step (draw 0); the chain's launches draw 1, 2, ...
+    assert first.us[:3] == [[uniform(11, 0, k), uniform(11, 1, k)] for k in (1, 2, 3)]
+    drawn_for_1 = [u[1] for u in first.us] + [u[0] for u in second.us]
+    assert drawn_for_1 == [uniform(11, 1, k) for k in range(1, 6)]
+    assert not e.live and all(c.closed for c in e.chains)
