@@ -755,13 +755,17 @@ __device__ __forceinline__ int kswz(int row, int cols) {      // the 16 key rows
 // rotated key and the value of the new token in that page (when `write_cache`), and waits
 // for the stores before the page is fetched.  For groups of up to 16 heads, so that one
 // workgroup alone reads that page.
+// `qruns` (FUSE only; null = none): the step's raw rows have not been put together yet; they are
+// the sums of `runs` float matrices [B, (nq + 2 nkv) HD], `run_stride` elements apart, as a
+// product cut along k leaves them.  Every value read from `q` is then the runs' sum in run
+// order, rounded to bf16: the bits the product's own sum kernel would have stored.
 template <int HD, int S, bool FUSE>
 __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
     const bf16* __restrict__ q, size_t q_stride, bf16* __restrict__ out, const int* __restrict__ slots,
     const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
     bf16* __restrict__ cache, int nq, int nkv, int window, float scale, int nsplit,
     float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ cs,
-    const float* __restrict__ sn, int write_cache) {
+    const float* __restrict__ sn, int write_cache, const float* __restrict__ qruns, int runs, size_t run_stride) {
     constexpr int NB = HD / 32;                      // 32-wide k-steps of the score product
     constexpr int KROWB = HD * 2, KCOLS = KROWB / 16; // a key row in bytes, in 16-byte columns
     constexpr int KB = PAGE * KROWB, STAGE = 2 * KB;  // keys, then values [HD][128 bytes]
@@ -796,8 +800,41 @@ __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
     const bool head_ok = c < nheads;
     const bf16* qrow = q + (size_t)b * q_stride + (size_t)(head0 + (head_ok ? c : 0)) * HD;
     bf16x8 qf[NB];
+    const size_t run_ld = (size_t)(nq + 2 * nkv) * HD;
+    if (FUSE && qruns) {
+        // four runs' loads at a time, so that they are in flight together; a run beyond the last adds +0
+        const float* pr = qruns + (size_t)b * run_ld + (size_t)(head0 + (head_ok ? c : 0)) * HD + 8 * g;
+        f32x4 lo[NB], hi[NB];
 #pragma unroll
-    for (int s = 0; s < NB; ++s) qf[s] = head_ok ? *(const bf16x8*)(qrow + s * 32 + 8 * g) : zero8();
+        for (int s = 0; s < NB; ++s) lo[s] = hi[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int p0 = 0; head_ok && p0 < runs; p0 += 4) {       // lanes without a head load nothing
+            f32x4 l[NB][4], h[NB][4];
+#pragma unroll
+            for (int s = 0; s < NB; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool on = p0 + j < runs;
+                    const float* a = pr + (size_t)(on ? p0 + j : 0) * run_stride + s * 32;
+                    l[s][j] = *(const f32x4*)a;
+                    h[s][j] = *(const f32x4*)(a + 4);
+                    if (!on) l[s][j] = h[s][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+            for (int s = 0; s < NB; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { lo[s] += l[s][j]; hi[s] += h[s][j]; }
+        }
+#pragma unroll
+        for (int s = 0; s < NB; ++s)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                qf[s][e] = head_ok ? (bf16)lo[s][e] : (bf16)0.f;
+                qf[s][4 + e] = head_ok ? (bf16)hi[s][e] : (bf16)0.f;
+            }
+    } else {
+#pragma unroll
+        for (int s = 0; s < NB; ++s) qf[s] = head_ok ? *(const bf16x8*)(qrow + s * 32 + 8 * g) : zero8();
+    }
     const size_t page_elems = (size_t)2 * nkv * PAGE * HD;
     const size_t k_off = (size_t)kvh * PAGE * HD, v_off = ((size_t)nkv + kvh) * PAGE * HD;
     if constexpr (FUSE) {
@@ -824,16 +861,32 @@ __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
         if (write_cache && hb == 0 && last_pg >= pg_begin && last_pg < pg_end) {
             const int off = (ctx - 1) % PAGE;
             bf16* pg = cache + (size_t)bt[last_pg] * page_elems;
-            const bf16* krow = q + (size_t)b * q_stride + (size_t)(nq + kvh) * HD;
-            const bf16* vrow = krow + (size_t)nkv * HD;
+            const size_t kcol = (size_t)(nq + kvh) * HD, vcol = kcol + (size_t)nkv * HD;
+            // element `col` of sequence b's raw row, from the row or from the runs
+            auto raw = [&](size_t col) -> bf16 {
+                if (!qruns) return q[(size_t)b * q_stride + col];
+                const float* a = qruns + (size_t)b * run_ld + col;
+                float v = 0.f;
+                for (int p0 = 0; p0 < runs; p0 += 4) {
+                    float t[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        t[j] = a[(size_t)(p0 + j < runs ? p0 + j : 0) * run_stride];
+                        if (p0 + j >= runs) t[j] = 0.f;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v += t[j];
+                }
+                return (bf16)v;
+            };
             if (tid < P) {
-                const float a = (float)krow[tid], bb = (float)krow[tid + P];
+                const float a = (float)raw(kcol + tid), bb = (float)raw(kcol + tid + P);
                 const float cc = cs ? cs[(size_t)b * P + tid] : 1.f, ss = cs ? sn[(size_t)b * P + tid] : 0.f;
                 pg[k_off + (size_t)off * HD + tid] = (bf16)(a * cc - bb * ss);
                 pg[k_off + (size_t)off * HD + tid + P] = (bf16)(a * ss + bb * cc);
             } else if (tid < P + HD) {
                 const int d = tid - P;
-                pg[v_off + (size_t)d * PAGE + off] = vrow[d];
+                pg[v_off + (size_t)d * PAGE + off] = raw(vcol + d);
             }
         }
         // __syncthreads below waits for these stores (they have reached the L2) before any page is fetched
@@ -1119,12 +1172,17 @@ extern "C" int br_attn_prefill_bf16(const void* q, size_t q_stride, void* out, c
 
 
 // part_o: float [B, nq, nsplit, hd]; part_ml: float [B, nq, nsplit, 2] (unused when nsplit == 1)
-extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, const int* slots,
-                                   const int* ctx_lens, const int* block_table, int table_stride,
-                                   void* cache, int B, int nq, int nkv, int hd, int page, int window,
-                                   float scale, int nsplit, float* part_o, float* part_ml, int variant,
-                                   int fuse, const float* cs, const float* sn, int write_cache, hipStream_t s) {
+// qruns, runs: with `fuse`, the step's raw rows as the float sums of `runs` runs of the product
+// that makes them ([runs][B][(nq + 2 nkv) hd], see the kernel); null = the rows stand in `q`.
+static int attn_decode_launch(const void* q, size_t q_stride, void* out, const int* slots,
+                              const int* ctx_lens, const int* block_table, int table_stride,
+                              void* cache, int B, int nq, int nkv, int hd, int page, int window,
+                              float scale, int nsplit, float* part_o, float* part_ml, int variant,
+                              int fuse, const float* cs, const float* sn, int write_cache, const float* qruns,
+                              int runs, hipStream_t s) {
     if (B <= 0) return BR_OK;
+    if (qruns && (!fuse || runs < 1 || runs > 64 || (uintptr_t)qruns % 16)) return BR_BAD_ARG;
+    const size_t run_stride = (size_t)B * (nq + 2 * nkv) * hd;
     if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd % 16 || hd > 256 || page != PAGE || window < 0 ||
         q_stride % 8 || ((uintptr_t)q % 16) || nsplit < 1 || nsplit > 1024 || B > 65535 ||
         (nsplit > 1 && (!part_o || !part_ml)))
@@ -1158,7 +1216,7 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
         }                                                                                                       \
         kern<<<grid, 256, lds2, s>>>((const bf16*)q, q_stride, (bf16*)out, slots, ctx_lens, block_table,        \
                                      table_stride, (bf16*)cache, nq, nkv, window, scale, nsplit, part_o,        \
-                                     part_ml, cs, sn, write_cache);                                             \
+                                     part_ml, cs, sn, write_cache, qruns, runs, run_stride);                    \
     } while (0)
         if (fuse) {
             if (hd == 128) { if (deep) BR_DECODE_LDS(128, 3, true); else BR_DECODE_LDS(128, 2, true); }
@@ -1203,6 +1261,28 @@ extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, co
     if (rc != BR_OK || nsplit == 1) return rc;
     attn_decode_combine_kernel<<<dim3(nq, B), 256, 0, s>>>(part_o, part_ml, (bf16*)out, nq, hd, nsplit);
     return br_check_launch();
+}
+
+extern "C" int br_attn_decode_bf16(const void* q, size_t q_stride, void* out, const int* slots,
+                                   const int* ctx_lens, const int* block_table, int table_stride,
+                                   void* cache, int B, int nq, int nkv, int hd, int page, int window,
+                                   float scale, int nsplit, float* part_o, float* part_ml, int variant,
+                                   int fuse, const float* cs, const float* sn, int write_cache, hipStream_t s) {
+    return attn_decode_launch(q, q_stride, out, slots, ctx_lens, block_table, table_stride, cache, B, nq, nkv, hd,
+                              page, window, scale, nsplit, part_o, part_ml, variant, fuse, cs, sn, write_cache,
+                              nullptr, 0, s);
+}
+
+// br_attn_decode_bf16 with rotation and cache write inside (`fuse` as there) from raw rows that
+// are still the float sums of the runs of their product.
+extern "C" int br_attn_decode_bf16_runs(const float* qruns, int runs, void* out, const int* slots,
+                                        const int* ctx_lens, const int* block_table, int table_stride,
+                                        void* cache, int B, int nq, int nkv, int hd, int page, int window,
+                                        float scale, int nsplit, float* part_o, float* part_ml,
+                                        const float* cs, const float* sn, int write_cache, hipStream_t s) {
+    if (!qruns) return BR_BAD_ARG;
+    return attn_decode_launch(qruns, 8, out, slots, ctx_lens, block_table, table_stride, cache, B, nq, nkv, hd,
+                              page, window, scale, nsplit, part_o, part_ml, 2, 1, cs, sn, write_cache, qruns, runs, s);
 }
 
 

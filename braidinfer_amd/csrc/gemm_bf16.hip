@@ -1355,15 +1355,20 @@ static void wide_shape(int M, int N, int K, int mode, int cus, size_t scratch_by
 // (needs a split product: the sum kernel does it; refused otherwise); 2 the activations were so
 // prepared and the sums are scaled (modes 0, 1, 3).  force_hb, force_parts: a tile height (in
 // blocks of 16 rows) and a number of runs other than wide_shape's (tests and measurements).
+// leave: the runs' sums stay in `scratch` ([runs][M][N] floats) for a consumer that adds them
+// in run order itself, and *leave says how many runs; refused (nothing launched) when the
+// product is not cut.
 template <int MB>
 static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                               int mode, float* scratch, size_t scratch_bytes, hipStream_t s, int norm = 0,
-                              StreamNorm nrm = StreamNorm{}, int force_hb = 0, int force_parts = 0, int wl = 0) {
+                              StreamNorm nrm = StreamNorm{}, int force_hb = 0, int force_parts = 0, int wl = 0,
+                              int* leave = nullptr) {
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
     const int nch = K / 128;
     int hb, parts;
     wide_shape(M, N, K, mode, cus, scratch ? scratch_bytes : 0, &hb, &parts);
+    if (leave && (parts < 2 || norm == 1 || force_hb || force_parts)) return BR_BAD_ARG;
     if (force_hb) {
         if (force_hb < 4 || force_hb > 8) return BR_BAD_ARG;
         hb = force_hb;
@@ -1410,6 +1415,10 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
 #undef BR_WIDE
     int rc = br_check_launch();
     if (rc != BR_OK || !partial) return rc;
+    if (leave) {
+        *leave = parts;
+        return rc;
+    }
     if (norm == 1) {
         gemm_split_sum_prep_kernel<<<(unsigned)(stride / 256), 256, 0, s>>>(scratch, parts, stride, (float*)C, N, ldc,
                                                                             nrm.gain, nrm.xg, nrm.ldx, nrm.ssq);
@@ -1604,6 +1613,25 @@ extern "C" int br_gemm_bf16_norm_scaled(const void* XG, const void* W, void* C, 
                                                scratch_bytes, s, 2, nrm, 0, 0, wl);
     }
     return BR_BAD_ARG;
+}
+
+// The float sums of the runs of A W^T (17 to 64 rows, bf16 result meant), left in `scratch` as
+// [*parts][M][N] for a consumer that adds them in run order and rounds, which gives the bits of
+// br_gemm_bf16 (or, with ssq, of br_gemm_bf16_norm_scaled) without the sum kernel's launch.
+// Refuses (BR_BAD_ARG, nothing launched) where those would not cut the product.
+extern "C" int br_gemm_bf16_wide_partial(const void* A, const void* W, int M, int N, int K, size_t lda,
+                                         const float* ssq, int ssq_tiles, int norm_width, float eps, void* scratch,
+                                         size_t scratch_bytes, int wl, int* parts, hipStream_t s) {
+    if (M <= 16 || M > 64 || N <= 0 || !parts || (wl != WL_ROWS && wl != WL_BLOCKED)) return BR_BAD_ARG;
+    if (!scratch || (uintptr_t)scratch % 16 || !wide_takes(A, W, M, K, lda)) return BR_BAD_ARG;
+    if (ssq && (ssq_tiles <= 0 || norm_width <= 0)) return BR_BAD_ARG;
+    StreamNorm nrm{};
+    if (ssq) nrm = StreamNorm{nullptr, nullptr, 0, (float*)ssq, ssq_tiles, 1.f / (float)norm_width, eps};
+    const int norm = ssq ? 2 : 0;
+    return M <= 32 ? launch_stream_wide<2>((const bf16*)A, (const bf16*)W, nullptr, M, N, K, lda, (size_t)N, OUT_BF16,
+                                           (float*)scratch, scratch_bytes, s, norm, nrm, 0, 0, wl, parts)
+                   : launch_stream_wide<4>((const bf16*)A, (const bf16*)W, nullptr, M, N, K, lda, (size_t)N, OUT_BF16,
+                                           (float*)scratch, scratch_bytes, s, norm, nrm, 0, 0, wl, parts);
 }
 
 // into how many runs along k br_gemm_bf16_ex and br_gemm_bf16_norm_prepare cut a product of 17 to 64 rows

@@ -360,6 +360,31 @@ def gemm_wide_parts(M: int, N: int, K: int, scratch_floats: int, accumulate: boo
     return int(f(M, N, K, 2 if accumulate else 1, scratch_floats * 4))
 
 
+def gemm_wide_partial(a: torch.Tensor, w: torch.Tensor, n_out: int, scratch: torch.Tensor,
+                      ssq: Optional[torch.Tensor] = None, tiles: int = 0, eps: float = 0.0) -> int:
+    """The runs of a @ w^T (17 to 64 bfloat16 rows, `n_out` columns) as float sums left in
+    `scratch`, [runs][M][n_out], for a consumer that adds them in run order and rounds to bfloat16
+    itself: the bits of `gemm` (with `ssq` and `tiles`: of `gemm_norm_scaled`) without the launch
+    that adds the runs.  Returns the number of runs, or 0 (nothing launched) where the product
+    would not be cut."""
+    _dev("gemm_wide_partial", a, w, scratch, ssq)
+    M, K = a.shape
+    N, wk, wl = _weight_dims("gemm_wide_partial", w, n_out)
+    _req(a.dtype == w.dtype == torch.bfloat16 and scratch.dtype == torch.float32 and wk == K and N == n_out,
+         "gemm_wide_partial: bfloat16 rows and matrix")
+    if not (16 < M <= 64 and gemm_stream_takes(M, K) and a.stride(1) == 1 and a.stride(0) % 8 == 0
+            and gemm_wide_parts(M, N, K, scratch.numel()) >= 2):
+        return 0
+    if ssq is not None:
+        _req(ssq.dtype == torch.float32 and tiles > 0 and ssq.numel() >= tiles * SSQ_LD, "gemm_wide_partial: sums of squares")
+    f = _fn("gemm_bf16", "br_gemm_bf16_wide_partial",
+            [_P, _P, c_int, c_int, c_int, c_size_t, _P, c_int, c_int, c_float, _P, c_size_t, c_int, _P, _P])
+    parts = c_int(0)
+    _check(f(_ptr(a), _ptr(w), M, N, K, a.stride(0), _ptr(ssq), int(tiles), K, float(eps), _ptr(scratch),
+             scratch.numel() * 4, wl, ctypes.byref(parts), _stream()), "gemm_wide_partial")
+    return parts.value
+
+
 SSQ_LD = 64        # row stride of the sums of squares that a product leaves for the next norm (SSQ_LD in csrc/gemm_bf16.hip)
 
 
@@ -471,7 +496,8 @@ def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slo
                           nq: int, nkv: int, hd: int, page: int, window: Optional[int], scale: float,
                           nsplit: int, part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
                           variant: int = 0, fuse_rope: bool = False, cos: Optional[torch.Tensor] = None,
-                          sin: Optional[torch.Tensor] = None, write_cache: bool = True) -> None:
+                          sin: Optional[torch.Tensor] = None, write_cache: bool = True,
+                          run_sums: Optional[torch.Tensor] = None, runs: int = 0) -> None:
     """Attention of one new token per sequence over its pages, cut into `nsplit` runs.
     `variant` forces a kernel: 1 reads operands straight from the cache, 2 brings pages
     through a ring in LDS (head sizes 64 and 128); 0 chooses.
@@ -479,8 +505,11 @@ def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slo
     `fuse_rope` (where `attention_decode_fuses_rope` says so): `q` is the step's raw
     [B, (nq + 2 nkv) * hd] rows; the kernel rotates queries and the new key by `cos` / `sin`
     ([B, hd / 2], pairs (p, p + hd / 2); None = no rotation) and stores key and value of the
-    new token in the cache itself (`write_cache`), so `rope_kv_write` is not called."""
-    _dev("attention_decode_bf16", out, slots, ctx_lens, block_table, cache, part_o, part_ml)
+    new token in the cache itself (`write_cache`), so `rope_kv_write` is not called.  With
+    `run_sums` (float32, `runs` matrices [B, (nq + 2 nkv) * hd] one after another, as
+    `gemm_wide_partial` leaves them) the raw rows are the runs' sums, which the kernel adds
+    itself; `q` is then not read."""
+    _dev("attention_decode_bf16", out, slots, ctx_lens, block_table, cache, part_o, part_ml, run_sums)
     _req(q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
          "attention_decode_bf16: bfloat16 only")
     _req(hd % 16 == 0 and hd <= 256, f"attention_decode_bf16: head_dim {hd} must be a multiple of 16, at most 256")
@@ -497,11 +526,23 @@ def attention_decode_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, slo
     if fuse_rope:
         _req(attention_decode_fuses_rope(hd, nq, nkv, page, block_table.shape[1], nsplit),
              "attention_decode_bf16: rotation and cache write are not fused for these sizes")
-        _req(q.shape[-1] == (nq + 2 * nkv) * hd, "attention_decode_bf16: fused rotation needs the raw q, k, v rows")
+        _req(run_sums is not None or q.shape[-1] == (nq + 2 * nkv) * hd,
+             "attention_decode_bf16: fused rotation needs the raw q, k, v rows")
         if cos is not None:
             _dev("attention_decode_bf16", cos, sin)
             _req(sin is not None and cos.dtype == sin.dtype == torch.float32 and cos.numel() >= B * (hd // 2)
                  and sin.numel() >= B * (hd // 2), "attention_decode_bf16: rotary tables must be float32 [B, hd / 2]")
+    if run_sums is not None:
+        _req(fuse_rope and variant in (0, 2) and run_sums.dtype == torch.float32 and 1 <= runs <= 64
+             and run_sums.numel() >= runs * B * (nq + 2 * nkv) * hd,
+             "attention_decode_bf16: run sums go with the fused rotation, float32 [runs, B, (nq + 2 nkv) * hd]")
+        g = _fn("attention_bf16", "br_attn_decode_bf16_runs",
+                [_P, c_int, _P, _P, _P, _P, c_int, _P] + [c_int] * 6 + [c_float, c_int, _P, _P, _P, _P, c_int, _P])
+        _check(g(_ptr(run_sums), int(runs), _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table),
+                 block_table.shape[1], _ptr(cache), B, nq, nkv, hd, page, int(window or 0), float(scale), nsplit,
+                 _ptr(part_o), _ptr(part_ml), _ptr(cos), _ptr(sin), int(write_cache), _stream()),
+               "attention_decode_bf16")
+        return
     _check(f(_ptr(q), q_stride, _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1],
              _ptr(cache), B, nq, nkv, hd, page, int(window or 0), float(scale), nsplit, _ptr(part_o),
              _ptr(part_ml), int(variant), int(fuse_rope), _ptr(cos) if fuse_rope else None,

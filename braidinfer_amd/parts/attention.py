@@ -21,7 +21,7 @@ from ..cache import CacheNeed
 from ..errors import ConfigError, StepError
 from ..weights import TensorSpec
 from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
-from .linear import fused_layout, linear, stream_layout
+from .linear import fused_layout, linear, linear_runs, stream_layout
 
 
 MAX_HEAD_DIM = 512      # attention_simple's limit; the matrix-core kernels take up to 256 in steps of 16
@@ -98,13 +98,18 @@ class GQAAttention(Mixer):
         nq, nkv, hd = self.nq, self.nkv, self.hd
         dt = self.rt.dtype
         qkv = step.ws.get("attn_qkv", (T, (nq + 2 * nkv) * hd), dt)
-        linear(h, self.w_qkv, qkv, step.ws)
         tables = step.position_data.get(self.position) if self.position else None
         if (tables is None and self._expects_tables) or (tables is not None and not isinstance(tables, RotaryTables)):
             raise StepError(f"attention: the position encoding {self.position!r} gave {type(tables).__name__}, "
                             "rotary tables were expected")
         if self._fused_decode(qkv, tables, step, ctx):
-            return self._finish(qkv, x, step, ctx, tables, True)
+            # the kernel that rotates and writes the cache itself reads only its own heads of the
+            # step's rows: where their product is cut into runs it adds the runs too
+            runs = linear_runs(h, self.w_qkv, qkv.shape[1], step.ws)
+            if runs is None:
+                linear(h, self.w_qkv, qkv, step.ws)
+            return self._finish(qkv, x, step, ctx, tables, True, runs)
+        linear(h, self.w_qkv, qkv, step.ws)
         K.rope_kv_write(qkv, tables.cos if tables else None, tables.sin if tables else None,
                         step.positions, step.seq_of_token, step.slots, ctx.block_table, ctx.storage,
                         nq, nkv, hd, tables.rotary_dim if tables else 0, tables.adjacent if tables else False,
@@ -121,12 +126,12 @@ class GQAAttention(Mixer):
         nsplit = decode_splits(step.n_seqs, self.nkv, step.max_ctx_bound, ctx.page_tokens, K.device_cus())
         return K.attention_decode_fuses_rope(self.hd, self.nq, self.nkv, ctx.page_tokens, ctx.block_table.shape[1], nsplit)
 
-    def _finish(self, qkv, x, step, ctx: MixerContext, fused_tables, fused: bool) -> None:
+    def _finish(self, qkv, x, step, ctx: MixerContext, fused_tables, fused: bool, runs=None) -> None:
         o = step.ws.get("attn_out", (step.n_tokens, self.nq * self.hd), self.rt.dtype)
-        self.attend(qkv, o, step, ctx, fused_tables, fused)
+        self.attend(qkv, o, step, ctx, fused_tables, fused, runs)
         linear(o, self.w_o, x, step.ws, accumulate=True)
 
-    def attend(self, qkv, o, step, ctx: MixerContext, fused_tables=None, fused: bool = False) -> None:
+    def attend(self, qkv, o, step, ctx: MixerContext, fused_tables=None, fused: bool = False, runs=None) -> None:
         """bf16 with a head size the matrix-core kernels take: split-context kernel when
         every sequence brings one token, flash kernel otherwise.  Else (32-bit path, head
         sizes beyond 256 or not in steps of 16) the one-wave-per-query kernel."""
@@ -144,7 +149,8 @@ class GQAAttention(Mixer):
                                         ctx.storage, B, nq, nkv, hd, ctx.page_tokens, self.window, self.scale,
                                         nsplit, part_o, part_ml, 0, fused,
                                         fused_tables.cos if fused_tables is not None else None,
-                                        fused_tables.sin if fused_tables is not None else None, ctx.writes_cache)
+                                        fused_tables.sin if fused_tables is not None else None, ctx.writes_cache,
+                                        runs.sums if runs is not None else None, runs.runs if runs is not None else 0)
             else:
                 K.attention_prefill_bf16(qkv, qkv.stride(0), o, step.cu_seqlens, step.slots, step.ctx_lens,
                                          ctx.block_table, ctx.storage, B, step.max_new, nq, nkv, hd,

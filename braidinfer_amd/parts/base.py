@@ -99,6 +99,25 @@ class Norm(Part):
         return False
 
 
+    def runs_of_prepared(self, prepared: Any, w: torch.Tensor, n_out: int, ws) -> Optional["ProductRuns"]:
+        """norm(x) @ w^T from what `prepare_in_product` left, as the float sums of its runs
+        along k (see `ProductRuns`); None with nothing done if the product is not cut so."""
+        return None
+
+
+@dataclass
+class ProductRuns:
+    """A product [rows, width] left as the float sums of `runs` runs along k, matrix after
+    matrix in `sums`; its bfloat16 value is the rounded sum of the runs in run order.  A kernel
+    that needs only a few of the product's elements adds them itself and saves the launch
+    that would."""
+
+    sums: torch.Tensor
+    runs: int
+    rows: int
+    width: int
+
+
 class ResidualSink:
     """The residual rows as a part that adds to them sees them, with the norm that reads them
     next.  `linear(a, w, sink, ws, accumulate=True)` adds the product and, where the norm

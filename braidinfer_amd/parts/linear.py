@@ -10,7 +10,7 @@ import os
 import torch
 
 from .. import kernels as K
-from .base import NormedInput, ResidualSink
+from .base import NormedInput, ProductRuns, ResidualSink
 
 
 def linear(a, w: torch.Tensor, out, ws, accumulate: bool = False) -> None:
@@ -57,6 +57,24 @@ def linear(a, w: torch.Tensor, out, ws, accumulate: bool = False) -> None:
         linear(a16, w, out, ws, accumulate)
         return
     raise TypeError(f"linear: activations {a.dtype}, weight {w.dtype}")
+
+
+def linear_runs(a, w: torch.Tensor, n_out: int, ws):
+    """a @ w^T (bfloat16, `n_out` columns) left as the float sums of its runs along k
+    (`ProductRuns`) where the product of these sizes is cut into runs anyway (17 to 64 rows over
+    few weight rows), for a caller whose next kernel adds the runs itself; None with nothing
+    done otherwise, and `linear` is then the way."""
+    if isinstance(a, NormedInput):
+        if a.prepared is not None:
+            return a.norm.runs_of_prepared(a.prepared, w, n_out, ws)
+        if not 16 < a.x.shape[0] <= 64 or w.dtype != torch.bfloat16 or a.dtype != torch.bfloat16:
+            return None
+        a = a.tensor()
+    if not (a.dtype == w.dtype == torch.bfloat16 and 16 < a.shape[0] <= 64):
+        return None
+    scratch = ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32)
+    runs = K.gemm_wide_partial(a, w, n_out, scratch)
+    return ProductRuns(scratch, runs, a.shape[0], n_out) if runs else None
 
 
 BLOCK_FROM_ROWS = 8192

@@ -8,7 +8,7 @@ import torch
 
 from .. import kernels as K
 from ..weights import TensorSpec
-from .base import Norm, Runtime, register_part
+from .base import Norm, ProductRuns, Runtime, register_part
 
 
 class RMSNorm(Norm):
@@ -50,6 +50,13 @@ class RMSNorm(Norm):
             return False
         K.gemm_norm_scaled(xg, ssq, tiles, self.eps, w, out, swiglu=swiglu, scratch=scratch)
         return True
+
+    def runs_of_prepared(self, prepared, w, n_out, ws):
+        xg, ssq, tiles, scratch = prepared
+        if w.dtype != torch.bfloat16 or scratch is None:
+            return None
+        runs = K.gemm_wide_partial(xg, w, n_out, scratch, ssq, tiles, self.eps)
+        return ProductRuns(scratch, runs, xg.shape[0], n_out) if runs else None
 
 
 register_part("norm", "rmsnorm", RMSNorm, replace=True)

@@ -423,6 +423,40 @@ def test_single_token_steps_launch_few_norm_kernels(serving, monkeypatch):
     eng.free_slot(s)
 
 
+@pytest.mark.parametrize("live", [17, 24, 48, 64])
+def test_single_token_steps_of_17_to_64_rows_add_the_runs_of_q_k_v_inside_attention(serving, live, monkeypatch):
+    """At 17 to 64 rows the product that makes queries, keys and values is cut along k; its
+    runs are added by the attention kernel for the heads it reads, not by a launch of their own.
+    The step must give the bits it gives with that launch, and the cache the same keys and values
+    (the next step reads them)."""
+    from braidinfer_amd.parts import attention as A
+    folder, cfg, w = serving
+    rng = np.random.default_rng(live)
+    lens = [int(x) for x in rng.integers(1, 150, live)]
+    seqs = [tokens(cfg, n + 2, 300 + i) for i, n in enumerate(lens)]
+    outs = []
+    for fold in (True, False):
+        eng = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=16384, use_graphs=False)
+        used = []
+        real = A.linear_runs
+        if fold:
+            monkeypatch.setattr(A, "linear_runs", lambda *a: (lambda r: (used.append(r is not None), r)[1])(real(*a)))
+        else:
+            monkeypatch.setattr(A, "linear_runs", lambda *a: None)
+        slots = [eng.alloc_slot() for _ in range(live)]
+        eng.step([StepEntry(sl, sq[:n], []) for sl, sq, n in zip(slots, seqs, lens)])
+        a = eng.step([StepEntry(sl, [sq[n]], [0]) for sl, sq, n in zip(slots, seqs, lens)])
+        b = eng.step([StepEntry(sl, [sq[n + 1]], [0]) for sl, sq, n in zip(slots, seqs, lens)])
+        outs.append((a.clone(), b.clone()))
+        if fold:
+            assert used and all(used), "the product of q, k and v was not left in runs"
+        monkeypatch.setattr(A, "linear_runs", real)
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    for i in (0, live // 2, live - 1):
+        close(np.stack([outs[0][0][i].cpu().numpy(), outs[0][1][i].cpu().numpy()]),
+              P.forward(cfg, w, seqs[i])[lens[i]:], "bfloat16", f"request {i} of {live}")
+
+
 @pytest.mark.parametrize("dtype,layout", [("float32", ""), ("bfloat16", ""), ("bfloat16", "blocks")])
 def test_serving_sizes_random_schedule(serving, dtype, layout, monkeypatch):
     """The random schedule at the sizes that take the serving kernels: up to 30 requests live,

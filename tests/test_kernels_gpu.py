@@ -648,6 +648,64 @@ def test_attention_decode_with_rotation_and_cache_write_fused(nq, nkv, hd, windo
                                 1 / math.sqrt(hd), nsplit, po, pml, 2, True, cs, sn, True)
 
 
+@pytest.mark.parametrize("normed", [False, True])
+@pytest.mark.parametrize("rows,nq,nkv,hd,width,window", [(24, 8, 2, 128, 1024, None), (64, 32, 8, 128, 4096, None),
+                                                          (40, 16, 1, 64, 512, 70), (17, 4, 4, 64, 1536, None)])
+def test_attention_decode_adds_the_runs_of_its_rows_itself(rows, nq, nkv, hd, width, window, normed):
+    """A product of 17 to 64 rows that is cut along k may leave its runs' sums, and the fused
+    decode attention adds them for the heads it reads: outputs and cache must have the bits
+    of the product summed by its own kernel followed by the same attention."""
+    B, page, nsplit = rows, 64, 2
+    lens = [int(x) for x in np.random.default_rng(rows).integers(1, 400, B)]
+    lens[0], lens[1], lens[2] = 64, 65, 1
+    _, _, cache, table = _multi_seq_cache(lens, nkv, hd, seed=rows + hd)
+    n_out = (nq + 2 * nkv) * hd
+    a = rnd(B, width, seed=3, dtype=torch.bfloat16)
+    w = rnd(n_out, width, seed=4, scale=0.05, dtype=torch.bfloat16)
+    scratch = torch.empty(K.GEMM_SCRATCH_FLOATS, device=DEV)
+    slots, ctx = i32(list(range(1, B + 1))), i32(lens)
+    pos = i32([l - 1 for l in lens])
+    inv = (1.0 / 1e4 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)).to(DEV)
+    cs, sn = torch.empty(B, hd // 2, device=DEV), torch.empty(B, hd // 2, device=DEV)
+    K.rope_table(pos, inv, cs, sn)
+    ssq, tiles, eps = None, 0, 1e-5
+    if normed:          # the rows as a product before left them for an RMS norm: sums of squares in tiles
+        tiles = width // 256
+        ssq = torch.zeros(tiles * K.SSQ_LD, device=DEV)
+        ssq.view(tiles, K.SSQ_LD)[:, :B] = (a.float() ** 2).view(B, tiles, 256).sum(-1).t()
+    part = lambda: (torch.empty(B * nq * nsplit * hd, device=DEV), torch.empty(B * nq * nsplit * 2, device=DEV))
+    # the product summed by its own kernel, then attention
+    qkv = torch.empty(B, n_out, device=DEV, dtype=torch.bfloat16)
+    if normed:
+        K.gemm_norm_scaled(a, ssq, tiles, eps, w, qkv, scratch=scratch)
+    else:
+        K.gemm(a, w, qkv, scratch=scratch)
+    cache_a, want = cache.clone(), torch.empty(B, nq * hd, device=DEV, dtype=torch.bfloat16)
+    po, pml = part()
+    K.attention_decode_bf16(qkv, n_out, want, slots, ctx, table, cache_a, B, nq, nkv, hd, page, window, 1 / math.sqrt(hd),
+                            nsplit, po, pml, 2, True, cs, sn, True)
+    # the runs left, attention adds them
+    scratch.fill_(float("nan"))
+    runs = K.gemm_wide_partial(a, w, n_out, scratch, ssq, tiles, eps)
+    if K.gemm_wide_parts(B, n_out, width, K.GEMM_SCRATCH_FLOATS) < 2:
+        assert runs == 0
+        return
+    assert runs >= 2
+    summed = scratch[:runs * B * n_out].view(runs, B, n_out)
+    total = summed[0].clone()
+    for r in range(1, runs):
+        total += summed[r]
+    assert torch.equal(total.to(torch.bfloat16), qkv)
+    cache_b, got = cache.clone(), torch.empty(B, nq * hd, device=DEV, dtype=torch.bfloat16)
+    po, pml = part()
+    K.attention_decode_bf16(torch.empty(0, device=DEV, dtype=torch.bfloat16), n_out, got, slots, ctx, table, cache_b, B,
+                            nq, nkv, hd, page, window, 1 / math.sqrt(hd), nsplit, po, pml, 0, True, cs, sn, True, scratch, runs)
+    assert torch.equal(cache_a, cache_b) and torch.equal(got, want)
+    with pytest.raises(KernelError):      # run sums without the fused rotation
+        K.attention_decode_bf16(qkv, n_out, got, slots, ctx, table, cache_b, B, nq, nkv, hd, page, window,
+                                1 / math.sqrt(hd), nsplit, po, pml, 0, False, None, None, True, scratch, runs)
+
+
 def test_attention_kernels_refuse_what_they_do_not_take():
     q = rnd(4, 2 * 24, dtype=torch.bfloat16)
     cache = torch.zeros(2, 2, 1, 64, 24, dtype=torch.bfloat16, device=DEV)
