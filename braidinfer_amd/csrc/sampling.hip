@@ -405,29 +405,136 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_sort_kernel(
     for (int i = keep + threadIdx.x; i < V; i += FBLOCK) w[~(uint32_t)(ks[i] & 0xffffffffu)] = -INFINITY;
 }
 
+// The general form for rows of up to LDS_SORT_MAX entries (padded to a power of two): only the
+// 32-bit value keys are sorted, in LDS.  The values in descending order are what the running
+// sum needs; which entries are kept follows from the last kept value T and from how many
+// entries equal to T are among the kept: those with the lowest indices, found by one scan in
+// index order.  The same masks as the sort of 64-bit keys in global memory, about twenty
+// times sooner at 32,768 entries.
+#define LDS_SORT_MAX 32768
+__global__ __launch_bounds__(FBLOCK) void sample_filter_sort_lds_kernel(
+    float* __restrict__ work, int V, int n2, const int* __restrict__ top_k, const float* __restrict__ min_p,
+    const float* __restrict__ top_p, const float* __restrict__ temperature, const int* __restrict__ slow) {
+    extern __shared__ uint32_t sk[];
+    __shared__ float red[16];
+    __shared__ float wsum[FBLOCK / 64];
+    __shared__ int wcnt[FBLOCK / 64];
+    __shared__ int keep_s, last_s;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    if (slow && !slow[b]) return;
+    const int k = top_k[b]; const float mp = min_p[b], tp = top_p[b];
+    const bool use_k = k > 0 && k < V, use_mp = mp > 0.f, use_tp = tp < 1.f;
+    if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
+    float* w = work + (size_t)b * V;
+    for (int i = tid; i < n2; i += FBLOCK) sk[i] = i < V ? f2key(w[i]) : 0u;
+    __syncthreads();
+    for (int size = 2; size <= n2; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int i = tid; i < n2 / 2; i += FBLOCK) {
+                const int lo = 2 * i - (i & (stride - 1)), hi = lo + stride;
+                const bool desc = (lo & size) == 0;
+                const uint32_t a = sk[lo], c = sk[hi];
+                if ((a < c) == desc) { sk[lo] = c; sk[hi] = a; }
+            }
+            __syncthreads();
+        }
+    }
+    int keep = use_k ? k : V;         // survivors are a prefix [0, keep) of the sorted order
+    const float vmax = key2f(sk[0]);
+    float cnt = 0.f, part = 0.f;
+    for (int i = tid; i < keep; i += FBLOCK) {
+        const float v = key2f(sk[i]);
+        if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { cnt += 1.f; part += expf(v - vmax); }
+    }
+    keep = (int)(block_sum(cnt, red) + 0.5f);
+    const float sum = block_sum(part, red);
+    if (use_tp) {
+        const int hit = block_first_reach(keep, tp, [&](int i) { return expf(key2f(sk[i]) - vmax) / sum; }, wsum, &keep_s);
+        if (hit < keep) keep = hit + 1;
+    }
+    if (keep <= 0) {                  // nothing survives (every entry was -inf): mask all, as the sort of whole keys does
+        for (int i = tid; i < V; i += FBLOCK) w[i] = -INFINITY;
+        return;
+    }
+    const uint32_t T = sk[keep - 1];
+    // entries above T come first in the order: their number by bisection, the same in every thread
+    int lo = 0, hi = keep - 1;        // sk[hi] == T; find the first index with sk[i] == T
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (sk[mid] > T) lo = mid + 1; else hi = mid;
+    }
+    const int need = keep - lo;       // kept entries equal to T: the `need` lowest indices among the equals
+    if (tid == 0) last_s = V;
+    __syncthreads();
+    const int lane = tid & 63, wv = tid >> 6;
+    int base = 0;
+    for (int i0 = 0; i0 < V && base < need; i0 += FBLOCK) {
+        const int i = i0 + tid;
+        const int flag = (i < V && f2key(w[i]) == T) ? 1 : 0;
+        int sc = flag;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+        __syncthreads();
+        if (lane == 63) wcnt[wv] = sc;
+        __syncthreads();
+        int before = base, tot = base;
+        for (int x = 0; x < FBLOCK / 64; ++x) { if (x < wv) before += wcnt[x]; tot += wcnt[x]; }
+        if (flag && before + sc == need) last_s = i;         // the last kept one among the equals
+        base = tot;
+        __syncthreads();
+    }
+    __syncthreads();
+    const int last = last_s;
+    for (int i = tid; i < V; i += FBLOCK) {
+        const uint32_t key = f2key(w[i]);
+        if (key < T || (key == T && i > last)) w[i] = -INFINITY;
+    }
+}
+
+static int launch_filter_sort(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
+                              const float* min_p, const float* top_p, const float* temperature, const int* slow,
+                              int in_lds, hipStream_t s) {
+    if (in_lds) {
+        const size_t lds = (size_t)n2 * sizeof(uint32_t);
+        static bool set = false;
+        if (!set) {
+            if (hipFuncSetAttribute((const void*)sample_filter_sort_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    LDS_SORT_MAX * (int)sizeof(uint32_t)) != hipSuccess)
+                return BR_LAUNCH_FAILED;
+            set = true;
+        }
+        sample_filter_sort_lds_kernel<<<B, FBLOCK, lds, s>>>(work, V, n2, top_k, min_p, top_p, temperature, slow);
+    } else {
+        sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, slow);
+    }
+    return br_check_launch();
+}
+
 // slow: int [B] scratch.  keys: [B, n2] scratch, needed only when `with_sort` (some row may
-// take the general form: top_k above 1024, or top-p without top-k).
+// take the general form: top_k above 1024, or top-p without top-k) and n2 is beyond
+// LDS_SORT_MAX (shorter rows are sorted in LDS).
 extern "C" int br_sample_filter(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
                                 const float* min_p, const float* top_p, const float* temperature, int* slow,
                                 int with_sort, hipStream_t s) {
     if (B <= 0) return BR_OK;
-    if (V <= 0 || !slow || (with_sort && (!keys || n2 < V || (n2 & (n2 - 1))))) return BR_BAD_ARG;
+    if (V <= 0 || !slow || (with_sort && (n2 < V || (n2 & (n2 - 1)) || (n2 > LDS_SORT_MAX && !keys)))) return BR_BAD_ARG;
     sample_filter_select_kernel<<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
     int rc = br_check_launch();
     if (rc != BR_OK || !with_sort) return rc;
-    sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, slow);
-    return br_check_launch();
+    return launch_filter_sort(work, keys, B, V, n2, top_k, min_p, top_p, temperature, slow, n2 <= LDS_SORT_MAX, s);
 }
 
-// the general form alone, for every row (tests compare the two)
+// the general form alone, for every row (tests compare the forms): in_lds 0 sorts whole keys in
+// `keys`, 1 the value keys in LDS (n2 up to LDS_SORT_MAX; `keys` is not used)
 extern "C" int br_sample_filter_sort(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
-                                     const float* min_p, const float* top_p, const float* temperature,
+                                     const float* min_p, const float* top_p, const float* temperature, int in_lds,
                                      hipStream_t s) {
     if (B <= 0) return BR_OK;
-    if (V <= 0 || !keys || n2 < V || (n2 & (n2 - 1))) return BR_BAD_ARG;
-    sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, nullptr);
-    return br_check_launch();
+    if (V <= 0 || n2 < V || (n2 & (n2 - 1)) || (in_lds ? n2 > LDS_SORT_MAX : !keys)) return BR_BAD_ARG;
+    return launch_filter_sort(work, keys, B, V, n2, top_k, min_p, top_p, temperature, nullptr, in_lds, s);
 }
+
+extern "C" int br_sample_lds_sort_max() { return LDS_SORT_MAX; }
 
 // ----------------------------------------------------------- softmax + draw --------
 // out[b] = first index i with u <= sum_{j<=i} softmax(work[b])_j  (sampling.rs:153-170);

@@ -89,7 +89,7 @@ def _filter_gpu(rows, top_k, min_p, top_p, general):
     keys = torch.empty((B, 1 << (V - 1).bit_length()), dtype=torch.int64, device=DEV)
     temp = f32([1.0] * B)
     if general:
-        K.sample_filter_sort(work, keys, i32(top_k), f32(min_p), f32(top_p), temp)
+        K.sample_filter_sort(work, keys, i32(top_k), f32(min_p), f32(top_p), temp, in_lds=general == "lds")
         return work.cpu().numpy(), None
     slow = torch.full((B,), -1, dtype=torch.int32, device=DEV)
     K.sample_filter(work, i32(top_k), f32(min_p), f32(top_p), temp, slow, keys)
@@ -114,7 +114,7 @@ def _check_row(row, got, k, mp, tp, label):
     assert min(counts) <= len(kept) <= max(counts), f"{label}: kept {len(kept)}, plain {sorted(counts)}"
 
 
-@pytest.mark.parametrize("V", [257, 3000, 32768 + 5])
+@pytest.mark.parametrize("V", [257, 3000, 20000, 32768, 32768 + 5])
 def test_filter_short_list_and_whole_row_sort_agree_with_the_plain_filter(V):
     rng = np.random.default_rng(V)
     smooth = (rng.normal(size=V) * 3).astype(np.float32)
@@ -131,7 +131,15 @@ def test_filter_short_list_and_whole_row_sort_agree_with_the_plain_filter(V):
     rows = np.stack([c[1] for c in cases])
     ks, mps, tps = [c[2] for c in cases], [c[3] for c in cases], [c[4] for c in cases]
     fast, slow = _filter_gpu(rows, ks, mps, tps, general=False)
-    whole, _ = _filter_gpu(rows, ks, mps, tps, general=True)
+    whole, _ = _filter_gpu(rows, ks, mps, tps, general="global")
+    if V <= 32768:
+        # rows this short are sorted in LDS by their values alone: the masks of the sort of whole keys, bit for bit
+        in_lds, _ = _filter_gpu(rows, ks, mps, tps, general="lds")
+        assert np.array_equal(in_lds, whole)
+    else:
+        from braidinfer_amd.errors import KernelError
+        with pytest.raises(KernelError):
+            _filter_gpu(rows[:2], ks[:2], mps[:2], tps[:2], general="lds")
     assert set(np.unique(slow)) <= {0, 1}
     for b, (label, row, k, mp, tp) in enumerate(cases):
         if V > 1100:
