@@ -210,7 +210,7 @@ def main() -> int:
         toks = sampler.argmax(torch.cat(last)).tolist()
 
         # the generation loop's way for greedy requests: a chain, one step launched ahead of the read
-        chain = eng.greedy_chain(slots, toks)
+        chain = eng.chain(slots, toks)
 
         def one():
             nonlocal toks

@@ -229,9 +229,6 @@ class Engine:
         from .graph import DecodeChain
         return DecodeChain(self._graphs, self.cache, slots, tokens, sampler_state)
 
-    def greedy_chain(self, slots: Sequence[int], tokens: Sequence[int]):
-        return self.chain(slots, tokens)
-
     # ---- generation (the Python entry point) -----------------------------------------------
     def generate(self, prompts, max_new_tokens: int = 64, temperature: float = 0.0, seed=None,
                  stop_token_ids=None, top_k: int = 0, top_p: float = 1.0, min_p: float = 0.0,

@@ -227,5 +227,3 @@ class DecodeChain:
         if self.g.owner is self:
             self.g.owner = None
 
-
-GreedyChain = DecodeChain

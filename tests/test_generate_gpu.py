@@ -76,7 +76,7 @@ def test_greedy_through_the_chain_equals_greedy_step_by_step(tiny_folders):
     folder, cfg, w = tiny_folders["b"]
     with_chain = B.Engine.from_folder(folder, dtype="float32", max_tokens=4096, max_seq_len=160)
     without = B.Engine.from_folder(folder, dtype="float32", max_tokens=4096, max_seq_len=160, use_graphs=False)
-    assert with_chain.greedy_chain is not None and without.greedy_chain([0], [1]) is None
+    assert without.chain([0], [1]) is None
     prompts = prompts_of(cfg, [3, 60, 17, 120, 1, 63, 150], 5)
     free_run = without.generate(prompts, max_new_tokens=70, stop_token_ids=[])
     stop = free_run[2][9]
@@ -160,7 +160,7 @@ def test_the_chain_by_hand(tiny_folders):
     slots = [eng.alloc_slot() for _ in prompts]
     logits = eng.step([B.StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
     first = logits.argmax(-1).tolist()
-    chain = eng.greedy_chain(slots, first)
+    chain = eng.chain(slots, first)
     chain.launch()
     chain.launch()
     with pytest.raises(B.StepError, match="unread"):
@@ -179,8 +179,8 @@ def test_the_chain_by_hand(tiny_folders):
         chain.launch()
     chain.close()
     with pytest.raises(B.StepError, match="vocabulary"):
-        eng.greedy_chain(slots, [0, cfg["vocab_size"]])
-    again = eng.greedy_chain(slots, got[-1])       # a new chain goes on where the old one stopped
+        eng.chain(slots, [0, cfg["vocab_size"]])
+    again = eng.chain(slots, got[-1])       # a new chain goes on where the old one stopped
     again.launch()
     more = again.read()
     again.close()
