@@ -12,8 +12,8 @@ Workloads (the benchmark description's shapes): `headline` Mistral-7B-v0.3, cont
 batch 8, prompts in [128, 2048]; `v0.1` Mistral-7B-v0.1 with its window of 4,096, context
 8,192, batch 8, prompts in [4096, 7168]; `24b` Mistral-Small-24B, context 32,768, batch 16,
 prompts in [1024, 16384].  Beside the headline value the line carries: the decode step's
-share of the published memory rate (`roofline`), further batch sizes and prompt lengths
-(`points`), what this GPU delivers to plain streaming and matrix-core kernels of this library
+share of the published memory rate (`roofline`), further batch sizes and prompt lengths and the
+headline batch with the reference's default sampling instead of greedy (`points`), what this GPU delivers to plain streaming and matrix-core kernels of this library
 (`measured_peaks`), and where an eager decode step's kernel time goes (`kernel_share`).
 """
 import argparse
@@ -143,7 +143,7 @@ def main() -> int:
     import braidinfer_amd as B
     from braidinfer_amd import StepEntry
     from braidinfer_amd import kernels as K
-    from braidinfer_amd.sampling import Sampler
+    from braidinfer_amd.sampling import Sampler, SamplingParams, uniform
 
     full = B.preset(args.preset)
     layers = args.layers or full.num_hidden_layers
@@ -191,7 +191,9 @@ def main() -> int:
         print(json.dumps({"metric": "prefill tok/s", "layers": layers, "prefill": prefill(eng, args.prefill_tokens)}), flush=True)
         return 0
 
-    def decode(batch, steps, warmup, seed, share=False):
+    def decode(batch, steps, warmup, seed, share=False, sampling=None):
+        """`sampling`: a SamplingParams for every request (the generation loop's sampled chain);
+        None is greedy."""
         rng = np.random.default_rng(seed)
         lens = [int(n) for n in rng.integers(args.prompt_min, args.prompt_max + 1, batch)]
         prompts = [[int(t) for t in rng.integers(0, V, n)] for n in lens]
@@ -207,21 +209,30 @@ def main() -> int:
             for r, b in enumerate(range(i, j)):
                 last[b] = out[r:r + 1].clone()
             i = j
-        toks = sampler.argmax(torch.cat(last)).tolist()
+        state, draws = None, 0
+        if sampling is not None:
+            state = sampler.state([sampling] * batch, prompts)
 
-        # the generation loop's way for greedy requests: a chain, one step launched ahead of the read
-        chain = eng.chain(slots, toks)
+        def us():
+            nonlocal draws
+            draws += 1
+            return [uniform(seed, b, draws) for b in range(batch)]
+        toks = sampler.argmax(torch.cat(last)).tolist() if state is None else state.sample(torch.cat(last), us())
+
+        # the generation loop's way: a chain, one step launched ahead of the read
+        chain = eng.chain(slots, toks, state)
+        launch = (lambda: chain.launch()) if state is None else (lambda: chain.launch(us()))
 
         def one():
             nonlocal toks
             if chain is None:
                 lg = eng.step([StepEntry(slots[b], [toks[b]], [0]) for b in range(batch)])
-                toks = sampler.argmax(lg).tolist()
+                toks = sampler.argmax(lg).tolist() if state is None else state.sample(lg, us())
             else:
-                chain.launch()
+                launch()
                 toks = chain.read()
         if chain is not None:
-            chain.launch()
+            launch()
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()
@@ -244,6 +255,8 @@ def main() -> int:
                         (H, I): "down_product", (V, H): "head_product"}
 
             def classes(name, a, k):
+                if name == "gemm_wide_partial":
+                    return products.get((a[2], a[1].shape[1] * 128 if a[1].dim() == 4 else a[1].shape[1]), "other_product")
                 if name in ("gemm", "gemm_swiglu", "gemm_norm_prepare"):
                     w, out, glu = a[1], a[2], name == "gemm_swiglu"
                 elif name == "gemm_norm_scaled":
@@ -288,6 +301,10 @@ def main() -> int:
                 d, _, _, _ = decode(b, k, max(2, args.warmup // 2), seed=10 + b)
                 points[f"decode_b{b}"] = round(b / d, 2)
                 print(f"[bench] batch {b}: {d * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+            # the reference's default sampling (temperature 1, top-k 50: sampling.rs:21-33) at the headline batch
+            d, _, _, _ = decode(args.batch, max(8, args.steps // 2), max(2, args.warmup // 2), seed=3,
+                                sampling=SamplingParams(seed=3))
+            points[f"decode_b{args.batch}_sampled"] = round(args.batch / d, 2)
         line["prefill"] = prefill(eng, min(args.prefill_tokens, args.context))
         if headline:
             for T in (128, 512):
