@@ -143,7 +143,7 @@ def main() -> int:
     import braidinfer_amd as B
     from braidinfer_amd import StepEntry
     from braidinfer_amd import kernels as K
-    from braidinfer_amd.sampling import Sampler, SamplingParams, uniform
+    from braidinfer_amd.sampling import Sampler, SamplingParams
 
     full = B.preset(args.preset)
     layers = args.layers or full.num_hidden_layers
@@ -209,30 +209,24 @@ def main() -> int:
             for r, b in enumerate(range(i, j)):
                 last[b] = out[r:r + 1].clone()
             i = j
-        state, draws = None, 0
-        if sampling is not None:
-            state = sampler.state([sampling] * batch, prompts)
-
-        def us():
-            nonlocal draws
-            draws += 1
-            return [uniform(seed, b, draws) for b in range(batch)]
-        toks = sampler.argmax(torch.cat(last)).tolist() if state is None else state.sample(torch.cat(last), us())
+        state = None
+        if sampling is not None:      # as the generation loop makes it: the state draws its own uniform numbers
+            state = sampler.state([sampling] * batch, prompts, random=[(seed, b, 0) for b in range(batch)])
+        toks = sampler.argmax(torch.cat(last)).tolist() if state is None else state.sample(torch.cat(last))
 
         # the generation loop's way: a chain, one step launched ahead of the read
         chain = eng.chain(slots, toks, state)
-        launch = (lambda: chain.launch()) if state is None else (lambda: chain.launch(us()))
 
         def one():
             nonlocal toks
             if chain is None:
                 lg = eng.step([StepEntry(slots[b], [toks[b]], [0]) for b in range(batch)])
-                toks = sampler.argmax(lg).tolist() if state is None else state.sample(lg, us())
+                toks = sampler.argmax(lg).tolist() if state is None else state.sample(lg)
             else:
-                launch()
+                chain.launch()
                 toks = chain.read()
         if chain is not None:
-            launch()
+            chain.launch()
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()

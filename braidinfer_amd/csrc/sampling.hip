@@ -101,48 +101,49 @@ extern "C" int br_step_advance(const int* drawn, int* tokens, int* positions, co
 // the temperature when it is not 0.  The bias lists are ragged: entries of row b are
 // [off[b], off[b+1]).  The history is a table counts[B, V] of occurrences per token (null: none),
 // which br_sample_draw_count keeps up to date on the device.
+#define PSEG 2048      // entries of a row that one workgroup prepares
 __global__ __launch_bounds__(SBLOCK) void sample_prepare_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int V,
     const int* __restrict__ bias_off, const int* __restrict__ bias_tok, const float* __restrict__ bias_val,
     const float* __restrict__ penalty, const float* __restrict__ temperature, const int* __restrict__ counts) {
-    const int b = blockIdx.x;
-    const float* r = logits + (size_t)b * V;
-    float* w = work + (size_t)b * V;
-    for (int i = threadIdx.x; i < V; i += SBLOCK) w[i] = r[i];
-    __syncthreads();
+    __shared__ float seg[PSEG];
+    const int b = blockIdx.y, lo = blockIdx.x * PSEG;
+    const int n = V - lo < PSEG ? V - lo : PSEG;
+    const float* r = logits + (size_t)b * V + lo;
+    float* w = work + (size_t)b * V + lo;
+    for (int i = threadIdx.x; i < n; i += SBLOCK) seg[i] = r[i];
     if (bias_off) {
-        // entries of one row may repeat a token: one thread applies them in order
+        __syncthreads();
+        // entries of one row may repeat a token: one thread applies those of this segment in order
         if (threadIdx.x == 0)
             for (int e = bias_off[b]; e < bias_off[b + 1]; ++e) {
-                int tk = bias_tok[e];
-                if (tk >= 0 && tk < V) w[tk] += bias_val[e];
+                const int tk = bias_tok[e] - lo;
+                if (tk >= 0 && tk < n) seg[tk] += bias_val[e];
             }
         __syncthreads();
     }
     const float pen = penalty ? penalty[b] : 1.f;
-    if (counts && pen != 1.f) {
-        const int* cn = counts + (size_t)b * V;
-        for (int i = threadIdx.x; i < V; i += SBLOCK) {
-            const int n = cn[i];
-            if (n > 0) {
-                float v = w[i];
-                for (int c = 0; c < n; ++c) v = (v > 0.f) ? v / pen : v * pen;
-                w[i] = v;
-            }
-        }
-        __syncthreads();
-    }
+    const bool penalised = counts && pen != 1.f;
+    const int* cn = penalised ? counts + (size_t)b * V + lo : nullptr;
     const float temp = temperature[b];
-    if (temp != 0.f)
-        for (int i = threadIdx.x; i < V; i += SBLOCK) w[i] = w[i] / temp;
+    for (int i = threadIdx.x; i < n; i += SBLOCK) {
+        float v = seg[i];
+        if (penalised) {
+            const int c_ = cn[i];
+            for (int c = 0; c < c_; ++c) v = (v > 0.f) ? v / pen : v * pen;
+        }
+        if (temp != 0.f) v = v / temp;
+        w[i] = v;
+    }
 }
 
 extern "C" int br_sample_prepare(const float* logits, float* work, int B, int V, const int* bias_off,
                                  const int* bias_tok, const float* bias_val, const int* counts,
                                  const float* penalty, const float* temperature, hipStream_t s) {
     if (B <= 0) return BR_OK;
-    if (V <= 0) return BR_BAD_ARG;
-    sample_prepare_kernel<<<B, SBLOCK, 0, s>>>(logits, work, V, bias_off, bias_tok, bias_val, penalty, temperature, counts);
+    if (V <= 0 || B > 65535) return BR_BAD_ARG;
+    sample_prepare_kernel<<<dim3((V + PSEG - 1) / PSEG, B), SBLOCK, 0, s>>>(logits, work, V, bias_off, bias_tok, bias_val,
+                                                                          penalty, temperature, counts);
     return br_check_launch();
 }
 
@@ -162,32 +163,45 @@ extern "C" int br_sample_count_add(int* counts, int B, int V, const int* row, co
 }
 
 // The first index i in [0, n) at which the running sum of f(0..i) reaches `target` (as
-// `target <= sum`), or n.  Sums run in index order, blockDim.x at a time: a scan inside
-// each wave, then the waves' totals in wave order.  Every thread of the block calls it;
-// `wsum` holds one float per wave, `found` one int.
+// `target <= sum`), or n.  The sums run in index order: every wave takes a run of consecutive
+// indices, 64 at a time with a scan inside the wave and the run's sum carried on; the runs'
+// totals, added in wave order, give each run its start.  Two passes over the run (its total,
+// then the search) with one barrier between them: no barrier per 64 indices, which is what a
+// row of a whole vocabulary would cost otherwise.  Every thread of the block calls it; `wsum`
+// holds one float per wave, `found` one int.
 template <typename F>
 __device__ __forceinline__ int block_first_reach(int n, float target, F f, float* wsum, int* found) {
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int nblk = (n + 63) >> 6, bpw = (nblk + nw - 1) / nw;
+    const int lo = wv * bpw * 64;
+    int hi = lo + bpw * 64;
+    if (hi > n) hi = n;
+    __syncthreads();                  // the caller may still be reading what `wsum` or `found` held
     if (threadIdx.x == 0) *found = 0x7fffffff;
-    float base = 0.f;
-    for (int i0 = 0; i0 < n; i0 += blockDim.x) {
-        const int i = i0 + threadIdx.x;
-        const float p = i < n ? f(i) : 0.f;
-        float sc = p;
+    float run = 0.f;
+    for (int i0 = lo; i0 < hi; i0 += 64) {
+        const int i = i0 + lane;
+        float sc = i < n ? f(i) : 0.f;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
-        __syncthreads();
-        if (lane == 63) wsum[wv] = sc;
-        __syncthreads();
-        float before = base;
-        for (int x = 0; x < wv; ++x) before += wsum[x];
-        if (i < n && target <= before + sc) atomicMin(found, i);
-        float tot = base;
-        for (int x = 0; x < nw; ++x) tot += wsum[x];
-        base = tot;
-        __syncthreads();
-        if (*found != 0x7fffffff) break;
+        run += __shfl(sc, 63, 64);
     }
+    if (lane == 0) wsum[wv] = run;
+    __syncthreads();
+    float acc = 0.f;
+    for (int x = 0; x < wv; ++x) acc += wsum[x];
+    int first = 0x7fffffff;
+    for (int i0 = lo; i0 < hi; i0 += 64) {
+        const int i = i0 + lane;
+        float sc = i < n ? f(i) : 0.f;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+        if (i < n && first == 0x7fffffff && target <= acc + sc) first = i;
+        acc += __shfl(sc, 63, 64);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { const int t = __shfl_xor(first, o, 64); first = t < first ? t : first; }
+    if (lane == 0 && first != 0x7fffffff) atomicMin(found, first);
     __syncthreads();
     const int r = *found;
     __syncthreads();
@@ -226,6 +240,8 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return t;
 }
 
+#define SEL_K 32       // a row of up to SEL_K * FBLOCK entries is read once and its keys kept in registers
+template <bool REG>
 __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
     float* __restrict__ work, int V, const int* __restrict__ top_k, const float* __restrict__ min_p,
     const float* __restrict__ top_p, const float* __restrict__ temperature, int* __restrict__ slow) {
@@ -234,6 +250,7 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
     __shared__ float red[16];
     __shared__ float wsum[FBLOCK / 64];
     __shared__ int sh_bin, sh_need, sh_ties, sh_cnt, keep_s;
+    __shared__ int wtot[4];
     const int b = blockIdx.x, tid = threadIdx.x;
     const int k = top_k[b];
     const float mp = min_p[b], tp = top_p[b];
@@ -242,12 +259,26 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
     if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
     if (use_k && k > CAND) { if (tid == 0) slow[b] = 1; return; }
     float* w = work + (size_t)b * V;
-    float mx = -INFINITY;
-    for (int i = tid; i < V; i += FBLOCK) mx = fmaxf(mx, w[i]);
-    const float vmax = block_max(mx, red);
+    // entry j of this thread is i = j * FBLOCK + tid; its value key stands in kx[j] (REG) or is read again
+    const int per = (V + FBLOCK - 1) / FBLOCK;
+    uint32_t kx[SEL_K];
+    if (REG) {
+#pragma unroll
+        for (int j = 0; j < SEL_K; ++j) {
+            const int i = j * FBLOCK + tid;
+            kx[j] = i < V ? f2key(w[i]) : 0u;
+        }
+    }
+#define SEL_ROW(j, i) _Pragma("unroll") for (int j = 0; j < (REG ? SEL_K : per); ++j) if (const int i = j * FBLOCK + tid; i < V)
+#define SEL_KEY(j, i) (REG ? kx[j] : f2key(w[i]))
+    uint32_t kmax = 0;
+    SEL_ROW(j, i) { const uint32_t key = SEL_KEY(j, i); kmax = key > kmax ? key : kmax; }
+    const float vmax = block_max(key2f(kmax), red);
     if (!use_k && !use_tp) {          // min-p alone is a threshold on the value
-        for (int i = tid; i < V; i += FBLOCK)
-            if (w[i] > -INFINITY && expf(w[i] - vmax) < mp) w[i] = -INFINITY;
+        SEL_ROW(j, i) {
+            const float v = key2f(SEL_KEY(j, i));
+            if (v > -INFINITY && expf(v - vmax) < mp) w[i] = -INFINITY;
+        }
         return;
     }
     const int cand = use_k ? k : (V < CAND ? V : CAND);
@@ -257,21 +288,34 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
     for (int shift = 24; shift >= 0; shift -= 8) {
         if (tid < 256) hist[tid] = 0;
         __syncthreads();
-        for (int i = tid; i < V; i += FBLOCK) {
-            const uint32_t key = f2key(w[i]);
+        SEL_ROW(j, i) {
+            const uint32_t key = SEL_KEY(j, i);
             if ((key & bits) == prefix) atomicAdd(&hist[(key >> shift) & 255], 1);
         }
         __syncthreads();
-        if (tid == 0) {
-            int cum = 0, bin = 255;
-            for (; bin > 0; --bin) {
-                if (cum + hist[bin] >= need) break;
-                cum += hist[bin];
-            }
-            sh_bin = bin; sh_need = need - cum; sh_ties = hist[bin];
+        // the highest bin at which the count from the top reaches `need` (bin 0 if none does): thread t
+        // of the first four waves stands for bin 255 - t and scans the counts from the top
+        const int lane = tid & 63, wv = tid >> 6;
+        int h = 0, sc = 0;
+        if (tid < 256) {
+            h = hist[255 - tid];
+            sc = h;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+            if (lane == 63) wtot[wv] = sc;
+        }
+        if (tid == 0) sh_bin = 255;
+        __syncthreads();
+        if (tid < 256) {
+            for (int x = 0; x < wv; ++x) sc += wtot[x];
+            const unsigned long long m = __ballot(sc >= need);
+            if (m && lane == __ffsll((long long)m) - 1) atomicMin(&sh_bin, tid);
         }
         __syncthreads();
-        prefix |= (uint32_t)sh_bin << shift;
+        if (tid == sh_bin) { sh_need = need - (sc - h); sh_ties = h; }
+        __syncthreads();
+        const int bin = 255 - sh_bin;
+        prefix |= (uint32_t)bin << shift;
         bits |= 255u << shift;
         need = sh_need;
         ties = sh_ties;
@@ -280,25 +324,24 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
     const uint32_t T = prefix;        // take every key above T and `need` of the `ties` keys equal to it
     if (tid == 0) sh_cnt = 0;
     __syncthreads();
-    for (int i = tid; i < V; i += FBLOCK) {
-        const float v = w[i];
-        if (f2key(v) > T) ck[atomicAdd(&sh_cnt, 1)] = comp_key(v, i);
+    SEL_ROW(j, i) {
+        const uint32_t key = SEL_KEY(j, i);
+        if (key > T) ck[atomicAdd(&sh_cnt, 1)] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
     }
     __syncthreads();
     const int ngt = sh_cnt;
     if (ties == need) {
-        for (int i = tid; i < V; i += FBLOCK) {
-            const float v = w[i];
-            if (f2key(v) == T) ck[atomicAdd(&sh_cnt, 1)] = comp_key(v, i);
+        SEL_ROW(j, i) {
+            const uint32_t key = SEL_KEY(j, i);
+            if (key == T) ck[atomicAdd(&sh_cnt, 1)] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
         }
     } else {
         // more equal values than places: the lowest indices win, found by an ordered scan
         const int lane = tid & 63, wv = tid >> 6;
         int base = 0;
-        for (int i0 = 0; i0 < V && base < need; i0 += FBLOCK) {
-            const int i = i0 + tid;
-            const float v = i < V ? w[i] : 0.f;
-            const int flag = (i < V && f2key(v) == T) ? 1 : 0;
+        for (int j = 0; j < per && base < need; ++j) {
+            const int i = j * FBLOCK + tid;
+            const int flag = (i < V && f2key(w[i]) == T) ? 1 : 0;
             int sc = flag;
 #pragma unroll
             for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
@@ -308,17 +351,19 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
             int before = base, tot = base;
             for (int x = 0; x < FBLOCK / 64; ++x) { if (x < wv) before += hist[x]; tot += hist[x]; }
             const int rank = before + sc - flag;
-            if (flag && rank < need) ck[ngt + rank] = comp_key(v, i);
+            if (flag && rank < need) ck[ngt + rank] = ((unsigned long long)T << 32) | (uint32_t)(~(uint32_t)i);
             base = tot;
             __syncthreads();
         }
     }
-    for (int t = cand + tid; t < CAND; t += FBLOCK) ck[t] = 0ull;
+    // bitonic sort of the candidates in LDS, descending, over the least power of two that holds them
+    int sortn = 64;
+    while (sortn < cand) sortn <<= 1;
+    for (int t = cand + tid; t < sortn; t += FBLOCK) ck[t] = 0ull;
     __syncthreads();
-    // bitonic sort of the candidates in LDS, descending
-    for (int size = 2; size <= CAND; size <<= 1) {
+    for (int size = 2; size <= sortn; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            if (tid < CAND / 2) {
+            if (tid < sortn / 2) {
                 const int lo = 2 * tid - (tid & (stride - 1)), hi = lo + stride;
                 const bool desc = (lo & size) == 0;
                 const unsigned long long a = ck[lo], c = ck[hi];
@@ -340,8 +385,8 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
     if (!use_k) {
         // without top-k the survivors are all entries that pass min-p: count and add them all
         float call = 0.f, pall = 0.f;
-        for (int i = tid; i < V; i += FBLOCK) {
-            const float v = w[i];
+        SEL_ROW(j, i) {
+            const float v = key2f(SEL_KEY(j, i));
             if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { call += 1.f; pall += expf(v - vmax); }
         }
         covered = (int)(block_sum(call, red) + 0.5f) <= keep;
@@ -354,8 +399,20 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
         else if (!covered) { if (tid == 0) slow[b] = 1; return; }
     }
     const unsigned long long last = ck[keep - 1];
-    for (int i = tid; i < V; i += FBLOCK)
-        if (comp_key(w[i], i) < last) w[i] = -INFINITY;
+    SEL_ROW(j, i) {
+        if ((((unsigned long long)SEL_KEY(j, i) << 32) | (uint32_t)(~(uint32_t)i)) < last) w[i] = -INFINITY;
+    }
+#undef SEL_ROW
+#undef SEL_KEY
+}
+
+static int launch_filter_select(float* work, int B, int V, const int* top_k, const float* min_p, const float* top_p,
+                                const float* temperature, int* slow, hipStream_t s) {
+    if (V <= SEL_K * FBLOCK)
+        sample_filter_select_kernel<true><<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
+    else
+        sample_filter_select_kernel<false><<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
+    return br_check_launch();
 }
 
 // The general form: the whole row is sorted once as 64-bit keys by a bitonic network in
@@ -518,8 +575,7 @@ extern "C" int br_sample_filter(float* work, unsigned long long* keys, int B, in
                                 int with_sort, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0 || !slow || (with_sort && (n2 < V || (n2 & (n2 - 1)) || (n2 > LDS_SORT_MAX && !keys)))) return BR_BAD_ARG;
-    sample_filter_select_kernel<<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
-    int rc = br_check_launch();
+    int rc = launch_filter_select(work, B, V, top_k, min_p, top_p, temperature, slow, s);
     if (rc != BR_OK || !with_sort) return rc;
     return launch_filter_sort(work, keys, B, V, n2, top_k, min_p, top_p, temperature, slow, n2 <= LDS_SORT_MAX, s);
 }
@@ -539,51 +595,145 @@ extern "C" int br_sample_lds_sort_max() { return LDS_SORT_MAX; }
 // ----------------------------------------------------------- softmax + draw --------
 // out[b] = first index i with u <= sum_{j<=i} softmax(work[b])_j  (sampling.rs:153-170);
 // argmax of the row when temperature is 0 (:81-84) or when rounding leaves u above the
-// last partial sum (:170).  Sums run over indices in ascending order, SBLOCK at a time.
-__global__ __launch_bounds__(SBLOCK) void sample_draw_kernel(const float* __restrict__ work, int* __restrict__ out,
+// last partial sum (:170).  Sums run over indices in ascending order (see block_first_reach).
+#define DBLOCK 1024
+//
+// The row's uniform number comes from u[b], or, with `rng_key`, is made here: 24 bits of
+// splitmix64(rng_key[b] ^ draw * 0xCA5A826395121157), draw = rng_draw[b], which then goes up by
+// one (every call, whatever the temperature): the numbers of sampling/params.py::uniform for
+// draws 0, 1, 2, ... of a request, without a copy from the host per step.
+__device__ __forceinline__ unsigned long long splitmix64(unsigned long long x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+#define DRAW_K 32      // a row of up to DRAW_K * DBLOCK entries is read once and kept in registers
+template <bool REG>
+__global__ __launch_bounds__(DBLOCK) void sample_draw_kernel(const float* __restrict__ work, int* __restrict__ out,
                                                              int V, const float* __restrict__ temperature,
-                                                             const float* __restrict__ u, int* __restrict__ counts) {
+                                                             const float* __restrict__ u, int* __restrict__ counts,
+                                                             const unsigned long long* __restrict__ rng_key,
+                                                             int* __restrict__ rng_draw) {
     __shared__ float red[16];
-    __shared__ float wsum[SBLOCK / 64];
+    __shared__ float wsum[DBLOCK / 64];
     __shared__ int found;
-    __shared__ float sv[SBLOCK / 64];
-    __shared__ int si[SBLOCK / 64];
+    __shared__ float sv[DBLOCK / 64];
+    __shared__ int si[DBLOCK / 64];
     const int b = blockIdx.x;
     const float* w = work + (size_t)b * V;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    // read before the first barrier; thread 0 moves the count on behind it
+    const int draw = rng_key ? rng_draw[b] : 0;
+    const float ub = rng_key ? (float)(splitmix64(rng_key[b] ^ ((unsigned long long)draw * 0xCA5A826395121157ull)) >> 40) *
+                                   (1.f / 16777216.f)
+                             : u[b];
+    // REG: wave wv holds the run of bpw * 64 consecutive entries from lo on, 64 at a time (the runs of block_first_reach)
+    const int nblk = (V + 63) >> 6, bpw = (nblk + DBLOCK / 64 - 1) / (DBLOCK / 64);
+    const int lo = wv * bpw * 64;
+    float x[DRAW_K];
     // argmax (lowest index wins)
     float bv = -INFINITY; int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += SBLOCK) argmax_combine(bv, bi, w[i], i);
+    if (REG) {
+#pragma unroll
+        for (int k = 0; k < DRAW_K; ++k) {
+            const int i = lo + k * 64 + lane;
+            const bool in = k < bpw && i < V;
+            x[k] = in ? w[i] : -INFINITY;
+            if (in) argmax_combine(bv, bi, x[k], i);
+        }
+    } else {
+        for (int i = threadIdx.x; i < V; i += DBLOCK) argmax_combine(bv, bi, w[i], i);
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         float ov = __shfl_xor(bv, o, 64); int oi = __shfl_xor(bi, o, 64);
         argmax_combine(bv, bi, ov, oi);
     }
-    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    if (lane == 0) { sv[wv] = bv; si[wv] = bi; }
     __syncthreads();
-    for (int ww = 0; ww < SBLOCK / 64; ++ww) argmax_combine(bv, bi, sv[ww], si[ww]);
+    for (int ww = 0; ww < DBLOCK / 64; ++ww) argmax_combine(bv, bi, sv[ww], si[ww]);
     if (bi == 0x7fffffff) bi = 0;
     if (temperature[b] == 0.f) {
-        if (threadIdx.x == 0) { out[b] = bi; if (counts) counts[(size_t)b * V + bi] += 1; }
+        if (threadIdx.x == 0) {
+            out[b] = bi;
+            if (counts) counts[(size_t)b * V + bi] += 1;
+            if (rng_key) rng_draw[b] = draw + 1;
+        }
         return;
     }
     const float vmax = bv;
     float part = 0.f;
-    for (int i = threadIdx.x; i < V; i += SBLOCK) part += expf(w[i] - vmax);
-    const float sum = block_sum(part, red);
-    const int hit = block_first_reach(V, u[b], [&](int i) { return expf(w[i] - vmax) / sum; }, wsum, &found);
+    int hit;
+    if (REG) {
+#pragma unroll
+        for (int k = 0; k < DRAW_K; ++k) {
+            const bool in = k < bpw && lo + k * 64 + lane < V;
+            x[k] = in ? expf(x[k] - vmax) : 0.f;
+            part += x[k];
+        }
+        const float sum = block_sum(part, red);
+        // the running sums as in block_first_reach, from the registers
+        if (threadIdx.x == 0) found = 0x7fffffff;
+        float run = 0.f;
+#pragma unroll
+        for (int k = 0; k < DRAW_K; ++k)
+            if (k < bpw) {
+                x[k] = x[k] / sum;
+                float sc = x[k];
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+                run += __shfl(sc, 63, 64);
+            }
+        if (lane == 0) wsum[wv] = run;
+        __syncthreads();
+        float acc = 0.f;
+        for (int ww = 0; ww < wv; ++ww) acc += wsum[ww];
+        int first = 0x7fffffff;
+#pragma unroll
+        for (int k = 0; k < DRAW_K; ++k)
+            if (k < bpw) {
+                float sc = x[k];
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) { float t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
+                const int i = lo + k * 64 + lane;
+                if (i < V && first == 0x7fffffff && ub <= acc + sc) first = i;
+                acc += __shfl(sc, 63, 64);
+            }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) { const int t = __shfl_xor(first, o, 64); first = t < first ? t : first; }
+        if (lane == 0 && first != 0x7fffffff) atomicMin(&found, first);
+        __syncthreads();
+        hit = found == 0x7fffffff ? V : found;
+    } else {
+        for (int i = threadIdx.x; i < V; i += DBLOCK) part += expf(w[i] - vmax);
+        const float sum = block_sum(part, red);
+        hit = block_first_reach(V, ub, [&](int i) { return expf(w[i] - vmax) / sum; }, wsum, &found);
+    }
     if (threadIdx.x == 0) {
         const int tok = hit < V ? hit : bi;
         out[b] = tok;
         if (counts) counts[(size_t)b * V + tok] += 1;       // the row's history grows by its new token
+        if (rng_key) rng_draw[b] = draw + 1;
     }
+}
+
+static int launch_draw(const float* work, int* out, int B, int V, const float* temperature, const float* u, int* counts,
+                       const unsigned long long* rng_key, int* rng_draw, hipStream_t s) {
+    if (V <= DRAW_K * DBLOCK)
+        sample_draw_kernel<true><<<B, DBLOCK, 0, s>>>(work, out, V, temperature, u, counts, rng_key, rng_draw);
+    else
+        sample_draw_kernel<false><<<B, DBLOCK, 0, s>>>(work, out, V, temperature, u, counts, rng_key, rng_draw);
+    return br_check_launch();
 }
 
 extern "C" int br_sample_draw(const float* work, int* out, int B, int V, const float* temperature,
                               const float* u, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0) return BR_BAD_ARG;
-    sample_draw_kernel<<<B, SBLOCK, 0, s>>>(work, out, V, temperature, u, nullptr);
-    return br_check_launch();
+    if (!u) return BR_BAD_ARG;
+    return launch_draw(work, out, B, V, temperature, u, nullptr, nullptr, nullptr, s);
 }
 
 // The same, and counts[b, token drawn] += 1 (the dense history of br_sample_prepare_dense; null: none).
@@ -591,6 +741,15 @@ extern "C" int br_sample_draw_count(const float* work, int* out, int B, int V, c
                                     const float* u, int* counts, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (V <= 0) return BR_BAD_ARG;
-    sample_draw_kernel<<<B, SBLOCK, 0, s>>>(work, out, V, temperature, u, counts);
-    return br_check_launch();
+    if (!u) return BR_BAD_ARG;
+    return launch_draw(work, out, B, V, temperature, u, counts, nullptr, nullptr, s);
+}
+
+// The same with the uniform numbers made on the device: rng_key[b] (the request's key, see the
+// kernel) and rng_draw[b] (its next draw, moved on by the call); counts may be null.
+extern "C" int br_sample_draw_random(const float* work, int* out, int B, int V, const float* temperature,
+                                     const unsigned long long* rng_key, int* rng_draw, int* counts, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0 || !rng_key || !rng_draw) return BR_BAD_ARG;
+    return launch_draw(work, out, B, V, temperature, nullptr, counts, rng_key, rng_draw, s);
 }

@@ -208,16 +208,21 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
                 old = resident["rows"]
                 if old is not None and set(live) <= set(old):
                     resident["state"] = resident["state"].keep([old.index(i) for i in live])
+                elif getattr(sampler, "takes_random", False):
+                    # the state draws its own numbers: uniform(seed, request, draw) from each request's next draw on
+                    resident["state"] = make_state([plist[i] for i in live], [hist[i] for i in live],
+                                                   random=[(seeds[i], i, len(out[i])) for i in live])
                 else:
                     resident["state"] = make_state([plist[i] for i in live], [hist[i] for i in live])
                 resident["rows"] = list(live)
             return resident["state"]
 
         def draw(logits, live):
-            us = [uniform(seeds[i], i, len(out[i])) for i in live]
+            us = lambda: [uniform(seeds[i], i, len(out[i])) for i in live]
             if make_state is None:
-                return sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live], us)
-            return state_of(live).sample(logits, us)
+                return sampler.sample(logits, [plist[i] for i in live], [hist[i] for i in live], us())
+            state = state_of(live)
+            return state.sample(logits) if getattr(state, "device_random", False) else state.sample(logits, us())
 
         def sample_and_book(logits, live, prefill):
             toks = draw(logits, live)
@@ -253,8 +258,10 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
                     if all(plist[i].is_plain_greedy for i in rows):
                         chain = open_chain([slot[i] for i in rows], [out[i][-1] for i in rows])
                     elif make_state is not None:
-                        chain = open_chain([slot[i] for i in rows], [out[i][-1] for i in rows], state_of(rows))
-                        us_of = lambda ahead: [uniform(seeds[i], i, len(out[i]) + ahead) for i in rows]
+                        state = state_of(rows)
+                        chain = open_chain([slot[i] for i in rows], [out[i][-1] for i in rows], state)
+                        if not getattr(state, "device_random", False):
+                            us_of = lambda ahead: [uniform(seeds[i], i, len(out[i]) + ahead) for i in rows]
                 if chain is not None:
                     live = _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cache, stats, t0, us_of)
                 else:

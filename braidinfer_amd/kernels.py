@@ -653,16 +653,28 @@ def sample_filter_sort(work, keys, top_k, min_p, top_p, temperature, in_lds: boo
              _stream()), "sample_filter_sort")
 
 
-def sample_draw(work, out, temperature, u, counts=None):
+def sample_draw(work, out, temperature, u, counts=None, rng_key=None, rng_draw=None):
     """`counts` (int32 [B, V], optional): the table of `sample_prepare`; the token drawn
-    for a row is added to the row's history there."""
-    _dev("sample_draw", work, out, temperature, u, counts)
+    for a row is added to the row's history there.  The rows' uniform numbers stand in `u`
+    (float32 [B]), or with `rng_key` (int64 [B]: `sampling.uniform_key` of each request) and
+    `rng_draw` (int32 [B]: each request's next draw, moved on by the call) are made by the
+    kernel: `sampling.uniform(seed, sequence, draw)` bit for bit."""
+    _dev("sample_draw", work, out, temperature, u, counts, rng_key, rng_draw)
     B, V = work.shape
-    _req(out.dtype == torch.int32 and u.dtype == torch.float32 and temperature.dtype == torch.float32, "sample_draw: dtypes")
+    _req(out.dtype == torch.int32 and temperature.dtype == torch.float32, "sample_draw: dtypes")
+    if counts is not None:
+        _req(counts.dtype == torch.int32 and counts.shape[0] >= B and counts.shape[1] == V, "sample_draw: counts must be int32 [B, V]")
+    if rng_key is not None:
+        _req(rng_draw is not None and rng_key.dtype == torch.int64 and rng_draw.dtype == torch.int32
+             and rng_key.numel() >= B and rng_draw.numel() >= B, "sample_draw: rng_key int64 [B] and rng_draw int32 [B]")
+        f = _fn("sampling", "br_sample_draw_random", [_P, _P, c_int, c_int, _P, _P, _P, _P, _P])
+        _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(rng_key), _ptr(rng_draw), _ptr(counts), _stream()),
+               "sample_draw")
+        return
+    _req(u is not None and u.dtype == torch.float32 and u.numel() >= B, "sample_draw: u must be float32 [B]")
     if counts is None:
         f = _fn("sampling", "br_sample_draw", [_P, _P, c_int, c_int, _P, _P, _P])
         _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(u), _stream()), "sample_draw")
         return
-    _req(counts.dtype == torch.int32 and counts.shape[0] >= B and counts.shape[1] == V, "sample_draw: counts must be int32 [B, V]")
     f = _fn("sampling", "br_sample_draw_count", [_P, _P, c_int, c_int, _P, _P, _P, _P])
     _check(f(_ptr(work), _ptr(out), B, V, _ptr(temperature), _ptr(u), _ptr(counts), _stream()), "sample_draw")

@@ -1,4 +1,4 @@
-from .params import SamplingParams, uniform, resolve_seed
-from .sampler import Sampler
+from .params import SamplingParams, uniform, uniform_key, resolve_seed
+from .sampler import Sampler, SamplerState
 
-__all__ = ["SamplingParams", "uniform", "resolve_seed", "Sampler"]
+__all__ = ["SamplingParams", "uniform", "uniform_key", "resolve_seed", "Sampler", "SamplerState"]

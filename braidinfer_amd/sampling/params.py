@@ -52,11 +52,16 @@ def _splitmix64(x: int) -> int:
     return x ^ (x >> 31)
 
 
-def uniform(seed: int, sequence: int, draw: int) -> float:
-    """A float in [0, 1) with 24 random bits, a pure function of its arguments."""
+def uniform_key(seed: int, sequence: int) -> int:
+    """What a request's uniform numbers are made from: 64 bits of its seed and its number."""
     h = _splitmix64(seed & _MASK)
-    h = _splitmix64(h ^ ((sequence * 0xD6E8FEB86659FD93) & _MASK))
-    h = _splitmix64(h ^ ((draw * 0xCA5A826395121157) & _MASK))
+    return _splitmix64(h ^ ((sequence * 0xD6E8FEB86659FD93) & _MASK))
+
+
+def uniform(seed: int, sequence: int, draw: int) -> float:
+    """A float in [0, 1) with 24 random bits, a pure function of its arguments (the draw
+    kernel of csrc/sampling.hip makes the same from `uniform_key` and the draw's number)."""
+    h = _splitmix64(uniform_key(seed, sequence) ^ ((draw * 0xCA5A826395121157) & _MASK))
     return (h >> 40) / float(1 << 24)
 
 

@@ -5,7 +5,9 @@ the HIP kernels in csrc/sampling.hip.  Order of operations as the reference's `s
 `SamplerState` is the sampler of one fixed set of rows over many steps: the rows' options,
 their bias lists and their histories (a table of occurrences per token, for the repetition
 penalty) live on the device; a step brings only its uniform numbers, and the kernel that draws
-a token also adds it to the row's history.  `Sampler.sample` is the same for a single call.
+a token also adds it to the row's history.  With `random` (each row's seed, request number and
+next draw) the uniform numbers are made by that kernel too (`sampling.uniform`, bit for bit), and a
+step brings nothing.  `Sampler.sample` is the same for a single call.
 """
 from __future__ import annotations
 
@@ -16,20 +18,30 @@ import numpy as np
 import torch
 
 from .. import kernels as K
-from .params import SamplingParams
+from .params import SamplingParams, uniform_key
 
 
 class SamplerState:
     def __init__(self, device, vocab_size: int, params: Sequence[SamplingParams],
-                 histories: Optional[Sequence[Sequence[int]]] = None, keys_cache: Optional[dict] = None):
+                 histories: Optional[Sequence[Sequence[int]]] = None, keys_cache: Optional[dict] = None,
+                 random: Optional[Sequence[tuple]] = None):
+        """`random[b]` = (seed, request number, next draw) of row b: `launch` without numbers then
+        draws with `uniform(seed, request number, draw)` for draw = next draw, next draw + 1, ..."""
         self.device, self.V, self.params = torch.device(device), int(vocab_size), list(params)
         B, V = len(self.params), self.V
         self.B = B
         self.greedy = all(p.is_plain_greedy for p in self.params)
         self._keys_cache = keys_cache if keys_cache is not None else {}
         self.out = torch.empty(B, dtype=torch.int32, device=self.device)
+        self.rng_key = self.rng_draw = None
         if self.greedy:
             return
+        if random is not None:
+            if len(random) != B:
+                raise ValueError(f"{len(random)} random states for {B} rows")
+            keys = np.array([uniform_key(int(s), int(q)) for s, q, _ in random], dtype=np.uint64)
+            self.rng_key = torch.from_numpy(keys.view(np.int64)).to(self.device)
+            self.rng_draw = self._i32([int(d) for _, _, d in random])
         # the per-row numbers go over in one copy: four float rows and one int row
         host = np.empty((5, B), dtype=np.float32)
         host[0] = [p.temperature for p in self.params]
@@ -84,6 +96,11 @@ class SamplerState:
     def _i32(self, v):
         return torch.tensor(v, dtype=torch.int32).to(self.device)
 
+    @property
+    def device_random(self) -> bool:
+        """Whether `launch` needs no uniform numbers from its caller."""
+        return self.greedy or self.rng_key is not None
+
     def _keys(self):
         n2 = 1 << (self.V - 1).bit_length()
         k = self._keys_cache.get("keys")
@@ -93,7 +110,8 @@ class SamplerState:
 
     def launch(self, logits: torch.Tensor, us: Optional[Sequence[float]] = None) -> torch.Tensor:
         """Enqueue the sampling of one step; returns the device tensor the tokens will stand in
-        (int32 [B], overwritten by the next launch).  `us[b]` is row b's uniform number in [0, 1)."""
+        (int32 [B], overwritten by the next launch).  `us[b]` is row b's uniform number in [0, 1);
+        without `us` a state made with `random` draws its own (one draw per row and call)."""
         B, V = logits.shape
         assert V == self.V and B == self.B
         if self.greedy:
@@ -115,7 +133,10 @@ class SamplerState:
         if self.filtered:
             K.sample_filter(self.work, self.top_k, self.min_p, self.top_p, self.temperature, self.slow,
                             self._keys() if self.needs_keys else None)
-        K.sample_draw(self.work, self.out, self.temperature, self.u, self.counts)
+        if us is None and self.rng_key is not None:
+            K.sample_draw(self.work, self.out, self.temperature, None, self.counts, self.rng_key, self.rng_draw)
+        else:
+            K.sample_draw(self.work, self.out, self.temperature, self.u, self.counts)
         return self.out
 
     def sample(self, logits: torch.Tensor, us: Optional[Sequence[float]] = None) -> List[int]:
@@ -128,10 +149,13 @@ class SamplerState:
         st.device, st.V, st.params = self.device, self.V, [self.params[r] for r in rows]
         st.B, st.greedy, st._keys_cache = len(rows), self.greedy, self._keys_cache
         st.out = torch.empty(st.B, dtype=torch.int32, device=self.device)
+        st.rng_key = st.rng_draw = None
         if self.greedy:
             return st
         idx = torch.tensor(list(rows), dtype=torch.long, device=self.device)
         pick = lambda t: t.index_select(0, idx)
+        if self.rng_key is not None:
+            st.rng_key, st.rng_draw = pick(self.rng_key), pick(self.rng_draw)
         st.temperature, st.penalty, st.min_p, st.top_p, st.top_k = (pick(t) for t in (
             self.temperature, self.penalty, self.min_p, self.top_p, self.top_k))
         st.bias_off = st.bias_tok = st.bias_val = None
@@ -158,6 +182,8 @@ class SamplerState:
 
 
 class Sampler:
+    takes_random = True        # `state` accepts `random`: the generation loop then sends no numbers per step
+
     def __init__(self, device, vocab_size: int):
         self.device = torch.device(device)
         self.V = int(vocab_size)
@@ -168,9 +194,11 @@ class Sampler:
         K.argmax(logits, out)
         return out
 
-    def state(self, params: Sequence[SamplingParams], histories: Optional[Sequence[Sequence[int]]] = None) -> SamplerState:
-        """The resident sampler of these rows: `state.sample(logits, us)` step after step."""
-        return SamplerState(self.device, self.V, params, histories, self._scratch)
+    def state(self, params: Sequence[SamplingParams], histories: Optional[Sequence[Sequence[int]]] = None,
+              random: Optional[Sequence[tuple]] = None) -> SamplerState:
+        """The resident sampler of these rows: `state.sample(logits, us)` step after step, or with
+        `random` (see `SamplerState`) `state.sample(logits)`."""
+        return SamplerState(self.device, self.V, params, histories, self._scratch, random)
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                histories: Optional[Sequence[Sequence[int]]] = None,

@@ -188,3 +188,36 @@ def test_a_resident_state_keeps_its_rows_histories_on_the_device():
         if step == 5:
             rows = [5, 0]                                    # another order, too
             state = state.keep([3, 0])
+
+
+def test_a_state_that_draws_its_own_numbers_draws_the_hosts():
+    """With `random` the draw kernel makes each row's uniform number itself from the request's
+    seed, number and draw count: the tokens of a state that is handed `uniform(seed, request, draw)`
+    step by step, through `keep` and for rows of temperature 0, whose count goes on too."""
+    from braidinfer_amd.sampling import uniform
+    V, B = 700, 5
+    rng = np.random.default_rng(4)
+    params = [SamplingParams(temperature=[1.0, 0.7, 0.0][b % 3], top_k=[0, 30][b % 2], repetition_penalty=[1.0, 1.3][b % 2])
+              for b in range(B)]
+    hists = [[int(t) for t in rng.integers(0, V, 5)] for _ in range(B)]
+    random = [(2 ** 63 + 11 * b, 3 * b + 1, 4 + b) for b in range(B)]        # seeds beyond 63 bits too
+    own = Sampler(DEV, V).state(params, hists, random=random)
+    told = Sampler(DEV, V).state(params, hists)
+    assert own.device_random and not told.device_random
+    rows, draws = list(range(B)), [d for _, _, d in random]
+    seen = set()
+    for step in range(9):
+        logits = torch.tensor(rng.normal(size=(len(rows), V)).astype(np.float32)).to(DEV)
+        a = own.sample(logits)
+        b = told.sample(logits, [uniform(random[r][0], random[r][1], draws[r]) for r in rows])
+        assert a == b, step
+        seen.update(a)
+        for r in rows:
+            draws[r] += 1
+        if step == 3:
+            rows = [4, 1, 2]
+            own, told = own.keep([4, 1, 2]), told.keep([4, 1, 2])
+    assert len(seen) > 10
+    assert own.rng_draw.tolist() == [draws[r] for r in rows]
+    with pytest.raises(ValueError):
+        Sampler(DEV, V).state(params, hists, random=random[:2])
