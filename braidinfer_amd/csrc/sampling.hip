@@ -38,7 +38,15 @@ __global__ __launch_bounds__(ABLOCK) void argmax_kernel(const float* __restrict_
     __shared__ int si[ABLOCK / 64];
     const float* r = logits + (size_t)blockIdx.x * V;
     float bv = -INFINITY; int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += ABLOCK) argmax_combine(bv, bi, r[i], i);
+    // eight loads in flight per thread: one load per trip would wait a memory latency each time
+    for (int i0 = threadIdx.x; i0 < V; i0 += 8 * ABLOCK) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = i0 + k * ABLOCK < V ? r[i0 + k * ABLOCK] : -INFINITY;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (i0 + k * ABLOCK < V) argmax_combine(bv, bi, v[k], i0 + k * ABLOCK);
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         float ov = __shfl_xor(bv, o, 64); int oi = __shfl_xor(bi, o, 64);
