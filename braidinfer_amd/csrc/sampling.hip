@@ -7,9 +7,12 @@
 
 #define SBLOCK 256
 
-// order-preserving map float -> uint32 (larger float = larger key; -0 < +0 is harmless)
+// order-preserving map float -> uint32 (larger float = larger key).  -0 takes the key of +0: the
+// two are equal in the reference's order (a sort by value, the lower index first among equals),
+// so which of a row's zeros a cut keeps is decided by their indices alone.
 __device__ __forceinline__ uint32_t f2key(float f) {
     uint32_t u = __float_as_uint(f);
+    if (u == 0x80000000u) u = 0u;
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 __device__ __forceinline__ float key2f(uint32_t k) {

@@ -157,6 +157,29 @@ def test_filter_short_list_and_whole_row_sort_agree_with_the_plain_filter(V):
         assert slow[peaked_top_p[0]] == 0
 
 
+def test_zeros_of_either_sign_are_equal_in_the_filters_order():
+    """-0.0 and +0.0 are one value to the reference's sort, so a cut inside a row's zeros keeps
+    those with the lowest indices whatever their signs, in every form of the filter."""
+    rng = np.random.default_rng(9)
+    for V in (300, 5000):
+        row = np.where(rng.random(V) < 0.5, np.float32(0.0), np.float32(-0.0)).astype(np.float32)
+        big = rng.choice(V, 20, replace=False)
+        row[big] = 3.0
+        row[rng.choice(np.setdiff1d(np.arange(V), big), V // 3, replace=False)] = -2.0
+        cases = [(60, 0.0, 1.0), (0, 0.0, 0.9), (1025, 0.0, 0.97), (100, 0.0, 0.95)]
+        rows = np.stack([row] * len(cases))
+        ks, mps, tps = [c[0] for c in cases], [c[1] for c in cases], [c[2] for c in cases]
+        forms = [_filter_gpu(rows, ks, mps, tps, general=False)[0], _filter_gpu(rows, ks, mps, tps, general="global")[0],
+                 _filter_gpu(rows, ks, mps, tps, general="lds")[0]]
+        for b, (k, mp, tp) in enumerate(cases):
+            for name, got in zip(("short list", "whole keys", "value keys in LDS"), forms):
+                _check_row(row, got[b], k, mp, tp, f"{name}, V={V} k={k} top_p={tp}")
+                kept = np.nonzero(got[b] > -np.inf)[0]
+                zeros = [i for i in kept if row[i] == 0.0]
+                assert zeros and len(zeros) < int((row == 0.0).sum()), "the cut was meant to fall among the zeros"
+                assert zeros == [i for i in range(V) if row[i] == 0.0][:len(zeros)]
+
+
 def test_a_resident_state_keeps_its_rows_histories_on_the_device():
     """Step after step with only the uniform numbers coming from the host: every drawn token
     joins its row's history (what the repetition penalty sees), rows that end are dropped with
