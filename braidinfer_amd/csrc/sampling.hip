@@ -223,18 +223,18 @@ __device__ __forceinline__ int block_first_reach(int n, float target, F f, float
 // Masks entries of work[b, :] to -inf as sampling.rs:89-151 does: top-k keeps the k
 // largest; min-p keeps values with exp(v - max) >= min_p; top-p keeps the shortest prefix,
 // in descending order, of the survivors whose probabilities (softmax over the survivors)
-// sum to >= top_p.  Order is by value, the lower index first among equals: every entry
-// has a 64-bit key (value key << 32 | ~index), all distinct, and "kept" is "key >= some
-// key", so the mask is one pass once that key is known.
+// sum to >= top_p.  Order is by value, the lower index first among equals.
 //
-// sample_filter_select_kernel finds it without sorting the row: a radix select over the
-// value keys picks the (at most 1024) largest entries, which are sorted in LDS; top-k,
-// min-p and top-p are then decided on that short list.  A row it cannot decide there
-// (top_k above 1024, or no top-k and a top-p that the 1024 largest do not reach) is
-// flagged in `slow` and left untouched for sample_filter_sort_kernel, which sorts the
-// whole row in global memory.
+// Nothing is sorted.  Both cuts are "the largest value T such that the entries from T upwards
+// weigh at least so much": for top-k an entry weighs 1 and so much is k; for top-p a survivor
+// weighs exp(v - max) as a whole number of 2^-40ths and so much is top_p times the survivors'
+// total (whole numbers: the sums are exact, whatever the order the atomics add them in).  T
+// comes from a radix descent over the value keys, 8 bits a pass, each pass a 256-bin table of
+// weights in LDS whose bins four waves scan from the top.  Of the entries equal to T the
+// lowest indices are kept, as many as are still needed: found by one count in index order,
+// and only when not all of them are.
 #define FBLOCK 1024
-#define CAND 1024
+#define FIL_RESIDENT 32768      // a row of up to so many entries is read once and its value keys kept in LDS
 
 __device__ __forceinline__ unsigned long long comp_key(float v, int i) {
     return ((unsigned long long)f2key(v) << 32) | (uint32_t)(~(uint32_t)i);
@@ -251,184 +251,206 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return t;
 }
 
-#define SEL_K 32       // a row of up to SEL_K * FBLOCK entries is read once and its keys kept in registers
-template <bool REG>
-__global__ __launch_bounds__(FBLOCK) void sample_filter_select_kernel(
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// weight of a survivor of value v in the top-p cut: exp(v - vmax) in 2^-40ths, at most 2^40
+__device__ __forceinline__ unsigned long long mass_of(float v, float vmax) {
+    return __float2ull_rn(expf(v - vmax) * 1099511627776.f);
+}
+
+template <bool RES>
+__global__ __launch_bounds__(FBLOCK) void sample_filter_kernel(
     float* __restrict__ work, int V, const int* __restrict__ top_k, const float* __restrict__ min_p,
-    const float* __restrict__ top_p, const float* __restrict__ temperature, int* __restrict__ slow) {
-    __shared__ unsigned long long ck[CAND];
-    __shared__ int hist[256];
+    const float* __restrict__ top_p, const float* __restrict__ temperature) {
+    __shared__ unsigned long long hist[3 * 256];
+    __shared__ unsigned long long wtot[FBLOCK / 64];
     __shared__ float red[16];
-    __shared__ float wsum[FBLOCK / 64];
-    __shared__ int sh_bin, sh_need, sh_ties, sh_cnt, keep_s;
-    __shared__ int wtot[4];
-    const int b = blockIdx.x, tid = threadIdx.x;
+    __shared__ int wcnt[FBLOCK / 64];
+    __shared__ int sh_idx;
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int k = top_k[b];
     const float mp = min_p[b], tp = top_p[b];
     const bool use_k = k > 0 && k < V, use_mp = mp > 0.f, use_tp = tp < 1.f;
-    if (tid == 0) slow[b] = 0;
     if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
-    if (use_k && k > CAND) { if (tid == 0) slow[b] = 1; return; }
     float* w = work + (size_t)b * V;
-    // entry j of this thread is i = j * FBLOCK + tid; its value key stands in kx[j] (REG) or is read again
-    const int per = (V + FBLOCK - 1) / FBLOCK;
-    uint32_t kx[SEL_K];
-    if (REG) {
-#pragma unroll
-        for (int j = 0; j < SEL_K; ++j) {
-            const int i = j * FBLOCK + tid;
-            kx[j] = i < V ? f2key(w[i]) : 0u;
+    // wave wv takes the run of bpw * 64 consecutive entries from lo on, 64 at a time: entry j of a lane is
+    // i = lo + 64 j + lane; its value key stands in sk[i] (RES) or is made from the row again
+    extern __shared__ uint32_t sk[];
+    const int nblk = (V + 63) >> 6, bpw = (nblk + FBLOCK / 64 - 1) / (FBLOCK / 64);
+    const int lo = wv * bpw * 64;
+    if (RES)
+        for (int j = 0; j < bpw; ++j) {
+            const int i = lo + 64 * j + lane;
+            if (i < V) sk[i] = f2key(w[i]);          // read back by the same lane only
         }
-    }
-#define SEL_ROW(j, i) _Pragma("unroll") for (int j = 0; j < (REG ? SEL_K : per); ++j) if (const int i = j * FBLOCK + tid; i < V)
-#define SEL_KEY(j, i) (REG ? kx[j] : f2key(w[i]))
+#define FIL_ROW(j, i) _Pragma("unroll 4") for (int j = 0; j < bpw; ++j) if (const int i = lo + 64 * j + lane; i < V)
+#define FIL_KEY(j, i) (RES ? sk[i] : f2key(w[i]))
+    for (int t = tid; t < 3 * 256; t += FBLOCK) hist[t] = 0ull;
     uint32_t kmax = 0;
-    SEL_ROW(j, i) { const uint32_t key = SEL_KEY(j, i); kmax = key > kmax ? key : kmax; }
-    const float vmax = block_max(key2f(kmax), red);
-    if (!use_k && !use_tp) {          // min-p alone is a threshold on the value
-        SEL_ROW(j, i) {
-            const float v = key2f(SEL_KEY(j, i));
-            if (v > -INFINITY && expf(v - vmax) < mp) w[i] = -INFINITY;
-        }
+    FIL_ROW(j, i) { const uint32_t key = FIL_KEY(j, i); kmax = key > kmax ? key : kmax; }
+    const float vmax = block_max(key2f(kmax), red);          // its barriers also stand behind the clearing
+
+    // The largest key T such that the entries with pred and a key >= T weigh at least `need` (need >= 1, and
+    // all of them together do): T in `pick_T`, what the entries equal to T still have to bring in `pick_rest`
+    // (>= 1) and what they weigh together in `pick_at`.  A pass: every thread adds its entries' weights into
+    // the pass's table, one barrier, then every wave reads the table for itself (four bins a lane, from the
+    // top) and finds the bin.  Three tables in turn, each cleared two passes before it is used, so that the
+    // barrier of the pass between stands between the clearing and both its neighbours.
+    uint32_t pick_T;
+    unsigned long long pick_rest, pick_at;
+    int table = 0;                    // the table of the next pass; tables table + 1 and + 2 (mod 3) are clear
+#define FIL_PICK(TYPE, PRED, MASS, NEED)                                                                      \
+    do {                                                                                                      \
+        uint32_t prefix_ = 0, bits_ = 0;                                                                      \
+        TYPE need_ = (TYPE)(NEED), at_ = 0;                                                                   \
+        for (int shift_ = 24; shift_ >= 0; shift_ -= 8) {                                                     \
+            TYPE* h_ = (TYPE*)(hist + 256 * table);                                                           \
+            FIL_ROW(j, i) {                                                                                   \
+                const uint32_t key = FIL_KEY(j, i);                                                           \
+                if ((key & bits_) == prefix_ && (PRED)) atomicAdd(&h_[(key >> shift_) & 255], (TYPE)(MASS));  \
+            }                                                                                                 \
+            __syncthreads();                                                                                  \
+            if (tid < 256) hist[256 * ((table + 2) % 3) + tid] = 0ull;      /* for the pass after the next */ \
+            /* lane l reads bins 255 - 4 l down to 252 - 4 l */                                               \
+            TYPE b_[4], run_ = 0;                                                                             \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q) { b_[q] = h_[255 - 4 * lane - q]; run_ += b_[q]; } \
+            TYPE sc_ = run_;                                                                                  \
+            _Pragma("unroll") for (int o = 1; o < 64; o <<= 1) {                                              \
+                const TYPE t_ = __shfl_up(sc_, o, 64);                                                        \
+                if (lane >= o) sc_ += t_;                                                                     \
+            }                                                                                                 \
+            const unsigned long long m_ = __ballot(sc_ >= need_);                                             \
+            const int first_ = m_ ? __ffsll((long long)m_) - 1 : 63;      /* none: the lowest bin */          \
+            TYPE above_ = sc_ - run_;                                       /* weight of the bins above this lane's */ \
+            int bin_ = 252 - 4 * lane;                                                                        \
+            TYPE here_ = b_[3];                                                                               \
+            {                                                                                                 \
+                TYPE c_ = above_;                                                                             \
+                bool done_ = false;                                                                           \
+                _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                 \
+                    if (!done_ && (c_ + b_[q] >= need_ || q == 3)) {                                          \
+                        bin_ = 255 - 4 * lane - q; here_ = b_[q]; above_ = c_; done_ = true;                  \
+                    } else if (!done_) c_ += b_[q];                                                           \
+            }                                                                                                 \
+            bin_ = __shfl(bin_, first_, 64);                                                                  \
+            above_ = __shfl(above_, first_, 64);                                                              \
+            here_ = __shfl(here_, first_, 64);                                                                \
+            prefix_ |= (uint32_t)bin_ << shift_;                                                              \
+            bits_ |= 255u << shift_;                                                                          \
+            need_ -= above_;                                                                                  \
+            at_ = here_;                                                                                      \
+            table = (table + 1) % 3;                                                                          \
+        }                                                                                                     \
+        pick_T = prefix_; pick_rest = need_; pick_at = at_;                                                   \
+    } while (0)
+
+    // The index of the n-th entry (n >= 1), in index order, with key T and pred; V if there are fewer.
+    int nth_idx;
+#define FIL_NTH(PRED, T_, N_)                                                                                 \
+    do {                                                                                                      \
+        int cnt_ = 0;                                                                                         \
+        FIL_ROW(j, i) { const uint32_t key = FIL_KEY(j, i); if (key == (T_) && (PRED)) ++cnt_; }              \
+        _Pragma("unroll") for (int o = 32; o > 0; o >>= 1) cnt_ += __shfl_xor(cnt_, o, 64);                   \
+        if (lane == 0) wcnt[wv] = cnt_;                                                                       \
+        if (tid == 0) sh_idx = V;                                                                             \
+        __syncthreads();                                                                                      \
+        int before_ = 0;                                                                                      \
+        for (int x = 0; x < wv; ++x) before_ += wcnt[x];                                                      \
+        if (before_ < (N_) && before_ + cnt_ >= (N_)) {          /* the wave whose run holds it */            \
+            for (int j = 0; j < bpw; ++j) {                                                                   \
+                {                                                                                             \
+                    const int i = lo + 64 * j + lane;                                                         \
+                    const uint32_t key = i < V ? FIL_KEY(j, i) : 0u;                                          \
+                    const bool f_ = i < V && key == (T_) && (PRED);                                           \
+                    const unsigned long long m_ = __ballot(f_);                                               \
+                    const int rank_ = before_ + __popcll(m_ & ((1ull << lane) - 1ull));                       \
+                    if (f_ && rank_ == (N_) - 1) sh_idx = i;                                                  \
+                    before_ += __popcll(m_);                                                                  \
+                }                                                                                             \
+            }                                                                                                 \
+        }                                                                                                     \
+        __syncthreads();                                                                                      \
+        nth_idx = sh_idx;                                                                                     \
+        __syncthreads();                                                                                      \
+    } while (0)
+
+    // top-k: the entries above Tk and, of those equal to it, the ones up to index idx_k
+    uint32_t Tk = 0;
+    int idx_k = V;
+    if (use_k) {
+        FIL_PICK(unsigned int, true, 1u, k);
+        Tk = pick_T;
+        if (pick_rest < pick_at) { FIL_NTH(true, Tk, (int)pick_rest); idx_k = nth_idx; }
+    }
+#define FIL_SURVIVES(key, i)                                                                                 \
+    ((!use_k || (key) > Tk || ((key) == Tk && (i) <= idx_k)) && key2f(key) > -INFINITY &&                   \
+     !(use_mp && expf(key2f(key) - vmax) < mp))
+    if (!use_tp) {
+        FIL_ROW(j, i) { const uint32_t key = FIL_KEY(j, i); if (!FIL_SURVIVES(key, i)) w[i] = -INFINITY; }
         return;
     }
-    const int cand = use_k ? k : (V < CAND ? V : CAND);
-    // radix select: the value key T of the cand-th largest entry, 8 bits a pass
-    uint32_t prefix = 0, bits = 0;
-    int need = cand, ties = 0;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        if (tid < 256) hist[tid] = 0;
-        __syncthreads();
-        SEL_ROW(j, i) {
-            const uint32_t key = SEL_KEY(j, i);
-            if ((key & bits) == prefix) atomicAdd(&hist[(key >> shift) & 255], 1);
-        }
-        __syncthreads();
-        // the highest bin at which the count from the top reaches `need` (bin 0 if none does): thread t
-        // of the first four waves stands for bin 255 - t and scans the counts from the top
-        const int lane = tid & 63, wv = tid >> 6;
-        int h = 0, sc = 0;
-        if (tid < 256) {
-            h = hist[255 - tid];
-            sc = h;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
-            if (lane == 63) wtot[wv] = sc;
-        }
-        if (tid == 0) sh_bin = 255;
-        __syncthreads();
-        if (tid < 256) {
-            for (int x = 0; x < wv; ++x) sc += wtot[x];
-            const unsigned long long m = __ballot(sc >= need);
-            if (m && lane == __ffsll((long long)m) - 1) atomicMin(&sh_bin, tid);
-        }
-        __syncthreads();
-        if (tid == sh_bin) { sh_need = need - (sc - h); sh_ties = h; }
-        __syncthreads();
-        const int bin = 255 - sh_bin;
-        prefix |= (uint32_t)bin << shift;
-        bits |= 255u << shift;
-        need = sh_need;
-        ties = sh_ties;
-        __syncthreads();
-    }
-    const uint32_t T = prefix;        // take every key above T and `need` of the `ties` keys equal to it
-    if (tid == 0) sh_cnt = 0;
+    // top-p over the survivors
+    unsigned long long part = 0;
+    FIL_ROW(j, i) { const uint32_t key = FIL_KEY(j, i); if (FIL_SURVIVES(key, i)) part += mass_of(key2f(key), vmax); }
+    part = wave_sum_u64(part);
     __syncthreads();
-    SEL_ROW(j, i) {
-        const uint32_t key = SEL_KEY(j, i);
-        if (key > T) ck[atomicAdd(&sh_cnt, 1)] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
-    }
+    if (lane == 0) wtot[wv] = part;
     __syncthreads();
-    const int ngt = sh_cnt;
-    if (ties == need) {
-        SEL_ROW(j, i) {
-            const uint32_t key = SEL_KEY(j, i);
-            if (key == T) ck[atomicAdd(&sh_cnt, 1)] = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
-        }
-    } else {
-        // more equal values than places: the lowest indices win, found by an ordered scan
-        const int lane = tid & 63, wv = tid >> 6;
-        int base = 0;
-        for (int j = 0; j < per && base < need; ++j) {
-            const int i = j * FBLOCK + tid;
-            const int flag = (i < V && f2key(w[i]) == T) ? 1 : 0;
-            int sc = flag;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
-            __syncthreads();
-            if (lane == 63) hist[wv] = sc;
-            __syncthreads();
-            int before = base, tot = base;
-            for (int x = 0; x < FBLOCK / 64; ++x) { if (x < wv) before += hist[x]; tot += hist[x]; }
-            const int rank = before + sc - flag;
-            if (flag && rank < need) ck[ngt + rank] = ((unsigned long long)T << 32) | (uint32_t)(~(uint32_t)i);
-            base = tot;
-            __syncthreads();
-        }
-    }
-    // bitonic sort of the candidates in LDS, descending, over the least power of two that holds them
-    int sortn = 64;
-    while (sortn < cand) sortn <<= 1;
-    for (int t = cand + tid; t < sortn; t += FBLOCK) ck[t] = 0ull;
+    unsigned long long total = 0;
+    for (int x = 0; x < FBLOCK / 64; ++x) total += wtot[x];
     __syncthreads();
-    for (int size = 2; size <= sortn; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            if (tid < sortn / 2) {
-                const int lo = 2 * tid - (tid & (stride - 1)), hi = lo + stride;
-                const bool desc = (lo & size) == 0;
-                const unsigned long long a = ck[lo], c = ck[hi];
-                if ((a < c) == desc) { ck[lo] = c; ck[hi] = a; }
-            }
-            __syncthreads();
-        }
+    if (total == 0) {                 // nothing survives with any weight (every entry was -inf): mask all
+        FIL_ROW(j, i) w[i] = -INFINITY;
+        return;
     }
-    // survivors are a prefix [0, keep) of the candidates
-    int keep = cand;
-    float cnt = 0.f, part = 0.f;
-    for (int i = tid; i < cand; i += FBLOCK) {
-        const float v = key2f((uint32_t)(ck[i] >> 32));
-        if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { cnt += 1.f; part += expf(v - vmax); }
+    unsigned long long target = (unsigned long long)ceil((double)tp * (double)total);
+    target = target < 1 ? 1 : (target > total ? total : target);
+    FIL_PICK(unsigned long long, FIL_SURVIVES(key, i), mass_of(key2f(key), vmax), target);
+    const uint32_t Tp = pick_T;
+    int idx_p = V;
+    {
+        const unsigned long long each = mass_of(key2f(Tp), vmax);
+        const unsigned long long n = each ? (pick_rest + each - 1) / each : 1ull;
+        if (each == 0 || n * each < pick_at) { FIL_NTH(FIL_SURVIVES(key, i), Tp, (int)n); idx_p = nth_idx; }
     }
-    keep = (int)(block_sum(cnt, red) + 0.5f);
-    float sum = block_sum(part, red);
-    bool covered = true;              // do the candidates hold every survivor?
-    if (!use_k) {
-        // without top-k the survivors are all entries that pass min-p: count and add them all
-        float call = 0.f, pall = 0.f;
-        SEL_ROW(j, i) {
-            const float v = key2f(SEL_KEY(j, i));
-            if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { call += 1.f; pall += expf(v - vmax); }
-        }
-        covered = (int)(block_sum(call, red) + 0.5f) <= keep;
-        sum = block_sum(pall, red);
+    FIL_ROW(j, i) {
+        const uint32_t key = FIL_KEY(j, i);
+        if (!(FIL_SURVIVES(key, i) && (key > Tp || (key == Tp && i <= idx_p)))) w[i] = -INFINITY;
     }
-    if (use_tp) {
-        const int hit = block_first_reach(keep, tp, [&](int i) {
-            return expf(key2f((uint32_t)(ck[i] >> 32)) - vmax) / sum; }, wsum, &keep_s);
-        if (hit < keep) keep = hit + 1;
-        else if (!covered) { if (tid == 0) slow[b] = 1; return; }
-    }
-    const unsigned long long last = ck[keep - 1];
-    SEL_ROW(j, i) {
-        if ((((unsigned long long)SEL_KEY(j, i) << 32) | (uint32_t)(~(uint32_t)i)) < last) w[i] = -INFINITY;
-    }
-#undef SEL_ROW
-#undef SEL_KEY
+#undef FIL_ROW
+#undef FIL_KEY
+#undef FIL_PICK
+#undef FIL_NTH
+#undef FIL_SURVIVES
 }
 
-static int launch_filter_select(float* work, int B, int V, const int* top_k, const float* min_p, const float* top_p,
-                                const float* temperature, int* slow, hipStream_t s) {
-    if (V <= SEL_K * FBLOCK)
-        sample_filter_select_kernel<true><<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
-    else
-        sample_filter_select_kernel<false><<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature, slow);
+extern "C" int br_sample_filter(float* work, int B, int V, const int* top_k, const float* min_p, const float* top_p,
+                                const float* temperature, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (V <= 0) return BR_BAD_ARG;
+    if (V <= FIL_RESIDENT) {
+        static bool set = false;
+        if (!set) {
+            if (hipFuncSetAttribute((const void*)sample_filter_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    FIL_RESIDENT * (int)sizeof(uint32_t)) != hipSuccess)
+                return BR_LAUNCH_FAILED;
+            set = true;
+        }
+        sample_filter_kernel<true><<<B, FBLOCK, (size_t)V * sizeof(uint32_t), s>>>(work, V, top_k, min_p, top_p, temperature);
+    } else {
+        sample_filter_kernel<false><<<B, FBLOCK, 0, s>>>(work, V, top_k, min_p, top_p, temperature);
+    }
     return br_check_launch();
 }
 
-// The general form: the whole row is sorted once as 64-bit keys by a bitonic network in
-// `keys` ([B, n2], n2 = V rounded up to a power of two).  With `slow` given, only the rows
-// it flags are treated.
+// The same masks the plain way, for tests to hold against the kernel above: the whole row is
+// sorted once as 64-bit keys (value key << 32 | ~index) by a bitonic network in `keys`
+// ([B, n2], n2 = V rounded up to a power of two), and the probabilities are added in that
+// order in float.  With `slow` given, only the rows it flags are treated.
 __global__ __launch_bounds__(FBLOCK) void sample_filter_sort_kernel(
     float* __restrict__ work, unsigned long long* __restrict__ keys, int V, int n2,
     const int* __restrict__ top_k, const float* __restrict__ min_p, const float* __restrict__ top_p,
@@ -473,135 +495,15 @@ __global__ __launch_bounds__(FBLOCK) void sample_filter_sort_kernel(
     for (int i = keep + threadIdx.x; i < V; i += FBLOCK) w[~(uint32_t)(ks[i] & 0xffffffffu)] = -INFINITY;
 }
 
-// The general form for rows of up to LDS_SORT_MAX entries (padded to a power of two): only the
-// 32-bit value keys are sorted, in LDS.  The values in descending order are what the running
-// sum needs; which entries are kept follows from the last kept value T and from how many
-// entries equal to T are among the kept: those with the lowest indices, found by one scan in
-// index order.  The same masks as the sort of 64-bit keys in global memory, about twenty
-// times sooner at 32,768 entries.
-#define LDS_SORT_MAX 32768
-__global__ __launch_bounds__(FBLOCK) void sample_filter_sort_lds_kernel(
-    float* __restrict__ work, int V, int n2, const int* __restrict__ top_k, const float* __restrict__ min_p,
-    const float* __restrict__ top_p, const float* __restrict__ temperature, const int* __restrict__ slow) {
-    extern __shared__ uint32_t sk[];
-    __shared__ float red[16];
-    __shared__ float wsum[FBLOCK / 64];
-    __shared__ int wcnt[FBLOCK / 64];
-    __shared__ int keep_s, last_s;
-    const int b = blockIdx.x, tid = threadIdx.x;
-    if (slow && !slow[b]) return;
-    const int k = top_k[b]; const float mp = min_p[b], tp = top_p[b];
-    const bool use_k = k > 0 && k < V, use_mp = mp > 0.f, use_tp = tp < 1.f;
-    if (temperature[b] == 0.f || !(use_k || use_mp || use_tp)) return;
-    float* w = work + (size_t)b * V;
-    for (int i = tid; i < n2; i += FBLOCK) sk[i] = i < V ? f2key(w[i]) : 0u;
-    __syncthreads();
-    for (int size = 2; size <= n2; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            for (int i = tid; i < n2 / 2; i += FBLOCK) {
-                const int lo = 2 * i - (i & (stride - 1)), hi = lo + stride;
-                const bool desc = (lo & size) == 0;
-                const uint32_t a = sk[lo], c = sk[hi];
-                if ((a < c) == desc) { sk[lo] = c; sk[hi] = a; }
-            }
-            __syncthreads();
-        }
-    }
-    int keep = use_k ? k : V;         // survivors are a prefix [0, keep) of the sorted order
-    const float vmax = key2f(sk[0]);
-    float cnt = 0.f, part = 0.f;
-    for (int i = tid; i < keep; i += FBLOCK) {
-        const float v = key2f(sk[i]);
-        if (v > -INFINITY && !(use_mp && expf(v - vmax) < mp)) { cnt += 1.f; part += expf(v - vmax); }
-    }
-    keep = (int)(block_sum(cnt, red) + 0.5f);
-    const float sum = block_sum(part, red);
-    if (use_tp) {
-        const int hit = block_first_reach(keep, tp, [&](int i) { return expf(key2f(sk[i]) - vmax) / sum; }, wsum, &keep_s);
-        if (hit < keep) keep = hit + 1;
-    }
-    if (keep <= 0) {                  // nothing survives (every entry was -inf): mask all, as the sort of whole keys does
-        for (int i = tid; i < V; i += FBLOCK) w[i] = -INFINITY;
-        return;
-    }
-    const uint32_t T = sk[keep - 1];
-    // entries above T come first in the order: their number by bisection, the same in every thread
-    int lo = 0, hi = keep - 1;        // sk[hi] == T; find the first index with sk[i] == T
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (sk[mid] > T) lo = mid + 1; else hi = mid;
-    }
-    const int need = keep - lo;       // kept entries equal to T: the `need` lowest indices among the equals
-    if (tid == 0) last_s = V;
-    __syncthreads();
-    const int lane = tid & 63, wv = tid >> 6;
-    int base = 0;
-    for (int i0 = 0; i0 < V && base < need; i0 += FBLOCK) {
-        const int i = i0 + tid;
-        const int flag = (i < V && f2key(w[i]) == T) ? 1 : 0;
-        int sc = flag;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) { int t = __shfl_up(sc, o, 64); if (lane >= o) sc += t; }
-        __syncthreads();
-        if (lane == 63) wcnt[wv] = sc;
-        __syncthreads();
-        int before = base, tot = base;
-        for (int x = 0; x < FBLOCK / 64; ++x) { if (x < wv) before += wcnt[x]; tot += wcnt[x]; }
-        if (flag && before + sc == need) last_s = i;         // the last kept one among the equals
-        base = tot;
-        __syncthreads();
-    }
-    __syncthreads();
-    const int last = last_s;
-    for (int i = tid; i < V; i += FBLOCK) {
-        const uint32_t key = f2key(w[i]);
-        if (key < T || (key == T && i > last)) w[i] = -INFINITY;
-    }
-}
-
-static int launch_filter_sort(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
-                              const float* min_p, const float* top_p, const float* temperature, const int* slow,
-                              int in_lds, hipStream_t s) {
-    if (in_lds) {
-        const size_t lds = (size_t)n2 * sizeof(uint32_t);
-        static bool set = false;
-        if (!set) {
-            if (hipFuncSetAttribute((const void*)sample_filter_sort_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    LDS_SORT_MAX * (int)sizeof(uint32_t)) != hipSuccess)
-                return BR_LAUNCH_FAILED;
-            set = true;
-        }
-        sample_filter_sort_lds_kernel<<<B, FBLOCK, lds, s>>>(work, V, n2, top_k, min_p, top_p, temperature, slow);
-    } else {
-        sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, slow);
-    }
-    return br_check_launch();
-}
-
-// slow: int [B] scratch.  keys: [B, n2] scratch, needed only when `with_sort` (some row may
-// take the general form: top_k above 1024, or top-p without top-k) and n2 is beyond
-// LDS_SORT_MAX (shorter rows are sorted in LDS).
-extern "C" int br_sample_filter(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
-                                const float* min_p, const float* top_p, const float* temperature, int* slow,
-                                int with_sort, hipStream_t s) {
-    if (B <= 0) return BR_OK;
-    if (V <= 0 || !slow || (with_sort && (n2 < V || (n2 & (n2 - 1)) || (n2 > LDS_SORT_MAX && !keys)))) return BR_BAD_ARG;
-    int rc = launch_filter_select(work, B, V, top_k, min_p, top_p, temperature, slow, s);
-    if (rc != BR_OK || !with_sort) return rc;
-    return launch_filter_sort(work, keys, B, V, n2, top_k, min_p, top_p, temperature, slow, n2 <= LDS_SORT_MAX, s);
-}
-
-// the general form alone, for every row (tests compare the forms): in_lds 0 sorts whole keys in
-// `keys`, 1 the value keys in LDS (n2 up to LDS_SORT_MAX; `keys` is not used)
+// every row through the sort (tests)
 extern "C" int br_sample_filter_sort(float* work, unsigned long long* keys, int B, int V, int n2, const int* top_k,
-                                     const float* min_p, const float* top_p, const float* temperature, int in_lds,
+                                     const float* min_p, const float* top_p, const float* temperature,
                                      hipStream_t s) {
     if (B <= 0) return BR_OK;
-    if (V <= 0 || n2 < V || (n2 & (n2 - 1)) || (in_lds ? n2 > LDS_SORT_MAX : !keys)) return BR_BAD_ARG;
-    return launch_filter_sort(work, keys, B, V, n2, top_k, min_p, top_p, temperature, nullptr, in_lds, s);
+    if (V <= 0 || !keys || n2 < V || (n2 & (n2 - 1))) return BR_BAD_ARG;
+    sample_filter_sort_kernel<<<B, FBLOCK, 0, s>>>(work, keys, V, n2, top_k, min_p, top_p, temperature, nullptr);
+    return br_check_launch();
 }
-
-extern "C" int br_sample_lds_sort_max() { return LDS_SORT_MAX; }
 
 // ----------------------------------------------------------- softmax + draw --------
 // out[b] = first index i with u <= sum_{j<=i} softmax(work[b])_j  (sampling.rs:153-170);

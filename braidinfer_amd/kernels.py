@@ -614,43 +614,31 @@ def sample_count_add(counts, rows, toks, cnts):
     _check(f(_ptr(counts), counts.shape[0], counts.shape[1], _ptr(rows), _ptr(toks), _ptr(cnts), n, _stream()), "sample_count_add")
 
 
-FILTER_CANDIDATES = 1024    # CAND in csrc/sampling.hip
-
-
-SORT_IN_LDS_MAX = 32768      # LDS_SORT_MAX in csrc/sampling.hip
-
-
-def sample_filter(work, top_k, min_p, top_p, temperature, slow, keys=None):
-    """Top-k, min-p and top-p masks on `work` [B, V].  `slow` is int32 [B] scratch.  `keys`
-    (int64 [B, power of two >= V] scratch) is given when some row may need the whole row
-    sorted: a top_k above 1024, or top-p without top-k.  Rows of up to 32,768 entries are then
-    sorted in LDS and `keys` only says so (it may be any int64 tensor of that shape)."""
-    _dev("sample_filter", work, top_k, min_p, top_p, temperature, slow)
+def sample_filter(work, top_k, min_p, top_p, temperature):
+    """Top-k, min-p and top-p masks on `work` [B, V] (entries cut become -inf), the reference's
+    order and rules (sampling.rs:89-151), the lower index first among equal values; rows of
+    temperature 0 are left alone.  Any vocabulary size, any top_k."""
+    _dev("sample_filter", work, top_k, min_p, top_p, temperature)
     B, V = work.shape
-    _req(slow.dtype == torch.int32 and slow.numel() >= B, "sample_filter: slow must be int32 [B]")
-    n2 = 0
-    if keys is not None:
-        _dev("sample_filter", keys)
-        n2 = keys.shape[1]
-        _req(keys.dtype == torch.int64 and keys.shape[0] >= B and n2 >= V and n2 & (n2 - 1) == 0
-             and keys.is_contiguous(), "sample_filter: keys must be int64 [B, power of two >= V]")
-    f = _fn("sampling", "br_sample_filter", [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int, _P])
-    _check(f(_ptr(work), _ptr(keys), B, V, n2, _ptr(top_k), _ptr(min_p), _ptr(top_p),
-             _ptr(temperature), _ptr(slow), 1 if keys is not None else 0, _stream()), "sample_filter")
+    _req(work.dtype == torch.float32 and work.is_contiguous() and top_k.dtype == torch.int32
+         and min_p.dtype == top_p.dtype == temperature.dtype == torch.float32
+         and min(top_k.numel(), min_p.numel(), top_p.numel(), temperature.numel()) >= B,
+         "sample_filter: float32 rows, int32 top_k [B], float32 min_p, top_p, temperature [B]")
+    f = _fn("sampling", "br_sample_filter", [_P, c_int, c_int, _P, _P, _P, _P, _P])
+    _check(f(_ptr(work), B, V, _ptr(top_k), _ptr(min_p), _ptr(top_p), _ptr(temperature), _stream()), "sample_filter")
 
 
-def sample_filter_sort(work, keys, top_k, min_p, top_p, temperature, in_lds: bool = False):
-    """The same masks by sorting every row whole (the general form of `sample_filter`): whole
-    keys in `keys`, or with `in_lds` the value keys in LDS (rows of up to 32,768 entries)."""
+def sample_filter_sort(work, keys, top_k, min_p, top_p, temperature):
+    """The same masks by sorting every row whole and adding the probabilities in that order
+    (what tests hold `sample_filter` against).  `keys`: int64 [B, power of two >= V] scratch."""
     _dev("sample_filter_sort", work, keys, top_k, min_p, top_p, temperature)
     B, V = work.shape
     n2 = keys.shape[1]
     _req(keys.dtype == torch.int64 and keys.shape[0] >= B and n2 >= V and n2 & (n2 - 1) == 0 and keys.is_contiguous(),
          "sample_filter_sort: keys must be int64 [B, power of two >= V]")
-    _req(not in_lds or n2 <= SORT_IN_LDS_MAX, f"sample_filter_sort: rows of up to {SORT_IN_LDS_MAX} entries are sorted in LDS")
-    f = _fn("sampling", "br_sample_filter_sort", [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, c_int, _P])
-    _check(f(_ptr(work), _ptr(keys), B, V, n2, _ptr(top_k), _ptr(min_p), _ptr(top_p), _ptr(temperature), int(in_lds),
-             _stream()), "sample_filter_sort")
+    f = _fn("sampling", "br_sample_filter_sort", [_P, _P, c_int, c_int, c_int, _P, _P, _P, _P, _P])
+    _check(f(_ptr(work), _ptr(keys), B, V, n2, _ptr(top_k), _ptr(min_p), _ptr(top_p), _ptr(temperature), _stream()),
+           "sample_filter_sort")
 
 
 def sample_draw(work, out, temperature, u, counts=None, rng_key=None, rng_draw=None):

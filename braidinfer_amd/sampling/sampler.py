@@ -23,15 +23,13 @@ from .params import SamplingParams, uniform_key
 
 class SamplerState:
     def __init__(self, device, vocab_size: int, params: Sequence[SamplingParams],
-                 histories: Optional[Sequence[Sequence[int]]] = None, keys_cache: Optional[dict] = None,
-                 random: Optional[Sequence[tuple]] = None):
+                 histories: Optional[Sequence[Sequence[int]]] = None, random: Optional[Sequence[tuple]] = None):
         """`random[b]` = (seed, request number, next draw) of row b: `launch` without numbers then
         draws with `uniform(seed, request number, draw)` for draw = next draw, next draw + 1, ..."""
         self.device, self.V, self.params = torch.device(device), int(vocab_size), list(params)
         B, V = len(self.params), self.V
         self.B = B
         self.greedy = all(p.is_plain_greedy for p in self.params)
-        self._keys_cache = keys_cache if keys_cache is not None else {}
         self.out = torch.empty(B, dtype=torch.int32, device=self.device)
         self.rng_key = self.rng_draw = None
         if self.greedy:
@@ -76,12 +74,7 @@ class SamplerState:
                 K.sample_count_add(self.counts, self._i32(rows), self._i32(toks), self._i32(cnts))
         self.filtered = any(p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)
                             for p in self.params)
-        # rows that the short-list kernel may hand on need room for a sort of the whole row
-        self.needs_keys = any(p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)
-                              and (p.top_k > K.FILTER_CANDIDATES or (not 0 < p.top_k < V and p.top_p < 1.0))
-                              for p in self.params)
         self.work = torch.empty((B, V), dtype=torch.float32, device=self.device)
-        self.slow = torch.empty(B, dtype=torch.int32, device=self.device)
         self._make_u()
 
     def _make_u(self):
@@ -100,13 +93,6 @@ class SamplerState:
     def device_random(self) -> bool:
         """Whether `launch` needs no uniform numbers from its caller."""
         return self.greedy or self.rng_key is not None
-
-    def _keys(self):
-        n2 = 1 << (self.V - 1).bit_length()
-        k = self._keys_cache.get("keys")
-        if k is None or k.shape[0] < self.B or k.shape[1] != n2:
-            k = self._keys_cache["keys"] = torch.empty((self.B, n2), dtype=torch.int64, device=self.device)
-        return k
 
     def launch(self, logits: torch.Tensor, us: Optional[Sequence[float]] = None) -> torch.Tensor:
         """Enqueue the sampling of one step; returns the device tensor the tokens will stand in
@@ -131,8 +117,7 @@ class SamplerState:
         K.sample_prepare(logits, self.work, self.bias_off, self.bias_tok, self.bias_val, self.counts, self.penalty,
                          self.temperature)
         if self.filtered:
-            K.sample_filter(self.work, self.top_k, self.min_p, self.top_p, self.temperature, self.slow,
-                            self._keys() if self.needs_keys else None)
+            K.sample_filter(self.work, self.top_k, self.min_p, self.top_p, self.temperature)
         if us is None and self.rng_key is not None:
             K.sample_draw(self.work, self.out, self.temperature, None, self.counts, self.rng_key, self.rng_draw)
         else:
@@ -147,7 +132,7 @@ class SamplerState:
         stay on the device."""
         st = SamplerState.__new__(SamplerState)
         st.device, st.V, st.params = self.device, self.V, [self.params[r] for r in rows]
-        st.B, st.greedy, st._keys_cache = len(rows), self.greedy, self._keys_cache
+        st.B, st.greedy = len(rows), self.greedy
         st.out = torch.empty(st.B, dtype=torch.int32, device=self.device)
         st.rng_key = st.rng_draw = None
         if self.greedy:
@@ -173,10 +158,7 @@ class SamplerState:
         V = self.V
         flt = lambda p: p.temperature != 0.0 and ((0 < p.top_k < V) or p.min_p > 0.0 or p.top_p < 1.0)
         st.filtered = any(flt(p) for p in st.params)
-        st.needs_keys = any(flt(p) and (p.top_k > K.FILTER_CANDIDATES or (not 0 < p.top_k < V and p.top_p < 1.0))
-                            for p in st.params)
         st.work = self.work[:st.B]
-        st.slow = self.slow[:st.B]
         st._make_u()
         return st
 
@@ -187,7 +169,6 @@ class Sampler:
     def __init__(self, device, vocab_size: int):
         self.device = torch.device(device)
         self.V = int(vocab_size)
-        self._scratch: dict = {}       # scratch for whole-row sorts, made when first needed and shared by the states
 
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
@@ -198,7 +179,7 @@ class Sampler:
               random: Optional[Sequence[tuple]] = None) -> SamplerState:
         """The resident sampler of these rows: `state.sample(logits, us)` step after step, or with
         `random` (see `SamplerState`) `state.sample(logits)`."""
-        return SamplerState(self.device, self.V, params, histories, self._scratch, random)
+        return SamplerState(self.device, self.V, params, histories, random)
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                histories: Optional[Sequence[Sequence[int]]] = None,
