@@ -430,6 +430,8 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path, dtype):
         assert not eng.use_graphs                          # the toys decide on the host: no graph capture
         _, w = P.read_folder(folder)
 
+        gaps = []
+
         def plain(toks):
             T = len(toks)
             x = P.embedding(w["r.embed.weight"], toks) + w["position.learned.weight"][:T]
@@ -443,6 +445,7 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path, dtype):
                     x = x + P.swiglu(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
                 else:
                     logits = n @ w[p + "mlp.router.weight"].T
+                    gaps.append(np.abs(logits[:, 0] - logits[:, 1]).min())
                     gate = np.exp(logits - logits.max(-1, keepdims=True)); gate /= gate.sum(-1, keepdims=True)
                     for t in range(T):
                         e = int(logits[t].argmax())
@@ -450,8 +453,12 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path, dtype):
                         x[t] = x[t] + y * gate[t, e]
             return P.linear(P.rms_norm(x, w["r.norm.weight"], 1e-5), w["r.head.weight"])
 
-        toks = [int(t) for t in np.random.default_rng(2).integers(0, 60, 50)]
+        # tokens for which every routing decision is clear: the least difference of the two router logits is
+        # 0.12 (of logits up to 2.3), ten times what bfloat16 rounding moves them by, so both precisions send
+        # every token to the same expert and every position can be held to the usual bounds
+        toks = [int(t) for t in np.random.default_rng(7).integers(0, 60, 50)]
         ref = plain(toks)
+        assert min(gaps) > 0.1
         s = eng.alloc_slot()
         got = [eng.step([StepEntry(s, toks[:30], list(range(30)))]).cpu().numpy()]
         for t in toks[30:]:
@@ -461,10 +468,8 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path, dtype):
         if dtype == "float32":
             assert np.abs(got - ref).max() < 1e-4 * np.abs(ref).max()
         else:
-            # bf16 may send a token whose two router logits are within rounding to the other
-            # expert, which changes that position and those after it: most positions agree
             cos = (got * ref).sum(-1) / (np.linalg.norm(got, axis=-1) * np.linalg.norm(ref, axis=-1))
-            assert np.median(cos) > 0.999
+            assert np.abs(got - ref).max() < 3e-2 * np.abs(ref).max() and cos.min() > 0.999
     finally:
         unregister_architecture("ToyRoutedForCausalLM")
         unregister_part("feed_forward", "top1_experts")
