@@ -110,6 +110,9 @@ def kernel_share(torch, eng, entries_of, classes):
     return share
 
 
+SETTLE_STEPS = 40
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -227,7 +230,9 @@ def main() -> int:
                 toks = chain.read()
         if chain is not None:
             chain.launch()
-        for _ in range(warmup):
+        # before the warm-up steps asked for, some more untimed ones: the first steps after the prompts run
+        # while the GPU's clocks still settle (measured: up to 3 % on the step when a heavy job ran just before)
+        for _ in range(warmup + SETTLE_STEPS):
             one()
         torch.cuda.synchronize()
         # keys a step has to read: the whole context, or the window where the model has one
