@@ -56,6 +56,36 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
+class _PinnedStaging:
+    """Pinned host memory for the changed pieces of a block table on their way to the device: two
+    halves used in turn; a half is written again only when every copy made from it has finished
+    (an event recorded when the half was left).  Copies from it need not wait for the device, so a
+    step that takes a new page does not hold the host up."""
+
+    def __init__(self, half: int):
+        self.half = half
+        self.buf = torch.empty(2 * half, dtype=torch.int32, pin_memory=True)
+        self.turn = 0
+        self.used = 0
+        self.left = [None, None]        # per half: the event behind the last copy made from it
+
+    def take(self, n: int) -> Optional[torch.Tensor]:
+        """`n` integers of staging memory, or None when a piece is larger than a half."""
+        if n > self.half:
+            return None
+        if self.used + n > self.half:
+            ev = self.left[self.turn] or torch.cuda.Event()
+            ev.record()
+            self.left[self.turn] = ev
+            self.turn ^= 1
+            self.used = 0
+            if self.left[self.turn] is not None:
+                self.left[self.turn].synchronize()
+        o = self.turn * self.half + self.used
+        self.used += n
+        return self.buf[o:o + n]
+
+
 class CacheGroup:
     def __init__(self, need: CacheNeed, unit_ids: Sequence[int], n_pages: int, n_slots: int,
                  max_pages_per_seq: int, page_tokens: int, dtype: torch.dtype, device):
@@ -70,6 +100,7 @@ class CacheGroup:
         self.table_cpu = torch.full((n_slots, max_pages_per_seq), -1, dtype=torch.int32)
         self.table_dev = self.table_cpu.to(self.device) if self.device.type != "cpu" else self.table_cpu
         self._dirty: Dict[int, Tuple[int, int]] = {}
+        self._staging = _PinnedStaging(max(4096, 2 * max_pages_per_seq)) if self.device.type == "cuda" else None
         if need.kv_heads <= 0 or need.key_dim <= 0 or need.val_dim < 0:
             raise CacheError(f"a cache unit needs kv heads and a key width above zero, got {need}")
         self.key_elems = need.kv_heads * page_tokens * need.key_dim        # of one page
@@ -147,7 +178,14 @@ class CacheGroup:
         """Bring the device block table up to date (changed row segments only)."""
         if self.table_dev is not self.table_cpu:
             for slot, (lo, hi) in self._dirty.items():
-                self.table_dev[slot, lo:hi].copy_(self.table_cpu[slot, lo:hi])
+                piece = self._staging.take(hi - lo) if self._staging is not None else None
+                if piece is None:
+                    self.table_dev[slot, lo:hi].copy_(self.table_cpu[slot, lo:hi])
+                else:
+                    # through pinned memory, in stream order, without waiting: the host's table may
+                    # change again (a trim, a freed slot) before the device has taken this piece
+                    piece.copy_(self.table_cpu[slot, lo:hi])
+                    self.table_dev[slot, lo:hi].copy_(piece, non_blocking=True)
         self._dirty.clear()
 
 
@@ -236,22 +274,26 @@ class SequenceCache:
                 g.grow(s, self.lengths[s] + n)
             g.sync()
 
-    def pages_held(self) -> List[List[int]]:
-        """Per group and slot the number of page entries a sequence has now (what
-        `release_reserved` rolls back to)."""
-        return [[len(p) for p in g.pages] for g in self.groups]
+    def pages_held(self, slots: Sequence[int]) -> List[List[int]]:
+        """Per group the number of page entries each of `slots` has now, in their order (what
+        `release_reserved` rolls back to).  Slots that are not live count as holding none:
+        `reserve` refuses them before it takes anything."""
+        n = self.n_slots
+        return [[len(g.pages[s]) if isinstance(s, int) and 0 <= s < n else 0 for s in slots] for g in self.groups]
 
     def release_reserved(self, slots: Sequence[int], held: List[List[int]]) -> None:
         """Undo a `reserve` that no `commit` follows: pages the slots took since `held` was
-        read go back to their pools."""
+        read (`pages_held` of the same slots) go back to their pools."""
         for g, before in zip(self.groups, held):
-            for s in slots:
-                extra = g.pages[s][before[s]:]
+            for s, had in zip(slots, before):
+                if not (isinstance(s, int) and 0 <= s < self.n_slots):
+                    continue
+                extra = g.pages[s][had:]
                 if extra:
                     g.pool.free([p for p in extra if p >= 0])
-                    g.table_cpu[s, before[s]:len(g.pages[s])] = -1
-                    g._mark(s, before[s], len(g.pages[s]))
-                    del g.pages[s][before[s]:]
+                    g.table_cpu[s, had:len(g.pages[s])] = -1
+                    g._mark(s, had, len(g.pages[s]))
+                    del g.pages[s][had:]
             g.sync()
 
     def commit(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:

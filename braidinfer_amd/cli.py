@@ -63,7 +63,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--min-p", type=float, default=0.0)
     ap.add_argument("--repetition-penalty", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=None)
-    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32", "bf16", "fp32"], default="bfloat16",
+                    help="bfloat16 (bf16) or float32 (fp32)")
     ap.add_argument("--random-weights", type=int, metavar="SEED", default=None,
                     help="make a model folder of random weights for --preset instead of reading MODEL")
     ap.add_argument("--preset", default="tiny-a")

@@ -15,6 +15,7 @@ from typing import Dict, List, Optional, Sequence, Union
 import numpy as np
 import torch
 
+from .. import kernels as K
 from ..cache import SequenceCache
 from ..config import config_from_folder, generation_stop_tokens, spec_of
 from ..errors import BraidError, CacheError, ConfigError, KernelError, StepError
@@ -183,7 +184,7 @@ class Engine:
                 if len(e.position_ids) != len(tl):
                     raise StepError(f"slot {e.slot}: {len(e.position_ids)} position numbers for {len(tl)} tokens")
         new = [len(tl) for tl in token_lists]
-        held = self.cache.pages_held()
+        held = self.cache.pages_held(slots)
         self.cache.reserve(slots, new)          # all or nothing
         try:
             starts = [self.cache.lengths[s] for s in slots]
@@ -193,11 +194,15 @@ class Engine:
                 if self._graphs is None:
                     from .graph import DecodeGraphs
                     self._graphs = DecodeGraphs(self.model, self.cache, self.device)
-                all_logits = self._graphs.run(slots, [tl[0] for tl in token_lists], starts)
-                if rows == list(range(len(slots))):
-                    logits = all_logits.clone()          # the graph's buffer is overwritten by the next step
-                else:
-                    logits = all_logits[torch.tensor(rows, dtype=torch.long, device=self.device)]
+                g = self._graphs.of(len(slots))
+                all_logits = g.run(slots, [tl[0] for tl in token_lists], starts)
+                # the graph's buffer is overwritten by the next step: the wanted rows go into a tensor
+                # of the caller's own (one copy kernel; nothing wanted: nothing copied)
+                logits = torch.empty((n_want, V), dtype=torch.float32, device=self.device)
+                if n_want:
+                    which = (g.want_rows[:n_want] if rows == list(range(n_want))
+                             else torch.tensor(rows, dtype=torch.int32).to(self.device))
+                    K.gather_rows(all_logits, which, logits)
             else:
                 try:
                     step = pack_step(slots, token_lists, starts, self.device, self.ws, position_ids=position_ids)

@@ -119,7 +119,10 @@ def _run_chain(chain, live, out, slot, take, finish, max_new_tokens, engine, cac
             while launched > read:
                 toks = chain.read()
                 read += 1
+                now = time.perf_counter()
                 stats.decode_tokens += len(going)
+                stats.decode_seconds += now - t0
+                t0 = now
                 for i, t in zip(live, toks):
                     if i in going:
                         reason = take(i, t, launched - read)

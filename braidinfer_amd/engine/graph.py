@@ -115,6 +115,12 @@ class DecodeGraph:
         if self.greedy_graph is None:
             torch.cuda.synchronize(self.device)
             saved = self.ints.clone()
+            # once eagerly, so that the kernel is loaded before the capture begins (nothing may be
+            # loaded under capture); the arrays it moves on are put back below
+            K.argmax_advance(self.logits, self.next_tokens, self.step.tokens, self.step.positions,
+                             self.step.slots, self.step.ctx_lens)
+            torch.cuda.synchronize(self.device)
+            self.ints.copy_(saved)
             g = torch.cuda.CUDAGraph()
             gc_was_on = gc.isenabled()
             gc.disable()
@@ -198,7 +204,7 @@ class DecodeChain:
             raise StepError("this chain's recorded step has been used by another step since; open a new chain")
         if len(self.pending) >= 2:
             raise StepError("two launched steps are unread; read one first")
-        held = self.cache.pages_held()
+        held = self.cache.pages_held(self.slots)
         self.cache.reserve(self.slots, self.ones)
         try:
             drawn = self._run(us)

@@ -95,7 +95,8 @@ class Replayer:
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description="replay token traces through the engine and write logits")
     ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
-    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32", "bf16", "fp32"],
+                    help="bfloat16 (bf16): the kernels and precisions of serving; float32 (fp32): everything in true 32-bit")
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")

@@ -110,6 +110,11 @@ class SafetensorsFolder:
             if not isinstance(weight_map, dict) or not weight_map or \
                     not all(isinstance(k, str) and isinstance(v, str) for k, v in weight_map.items()):
                 raise WeightError(f"{index}: 'weight_map' must map tensor names to file names")
+            # a file of the index lies in the folder itself: no path that leads elsewhere is followed
+            outside = sorted({v for v in weight_map.values()
+                              if os.path.basename(v) != v or v in ("", ".", "..") or os.path.isabs(v)})
+            if outside:
+                raise WeightError(f"{index}: the index names files outside the model folder: {', '.join(outside)}")
             paths = [os.path.join(folder, v) for v in sorted(set(weight_map.values()))]
             absent = [os.path.basename(p) for p in paths if not os.path.isfile(p)]
             if absent:

@@ -147,6 +147,30 @@ def sizes(cfg):
 
 
 # ------------------------------------------------------------------------ the parts ----
+def bf16_round(a):
+    """float32 -> the nearest bfloat16 (ties to even), kept as float32 (quant.rs:203-207)."""
+    bits = np.ascontiguousarray(a, dtype=F).view(np.uint32)
+    r = ((bits + (((bits >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF))) >> np.uint32(16)) << np.uint32(16)
+    return r.astype(np.uint32).view(F).reshape(np.shape(a))
+
+
+def _same(a):
+    return a
+
+
+def rounding(act_dtype):
+    """What the forward functions apply to every activation that a bfloat16 engine keeps in
+    bfloat16: the normed rows, q, k and v as the projection leaves them, q and k after rotation
+    (keys are cached so), the probabilities that multiply the values, the attention's output
+    and the SwiGLU output.  The residual rows, scores, sums and logits stay float.
+    None or "float32": nothing is rounded."""
+    if act_dtype in (None, "float32"):
+        return _same
+    if act_dtype == "bfloat16":
+        return bf16_round
+    raise ValueError(f"act_dtype {act_dtype!r}")
+
+
 def embedding(table, tokens):
     """x[t] = table[token[t]], no scaling (kernels/megakernel_ops.hip:1757-1768)."""
     return table[np.asarray(tokens, dtype=np.int64)].astype(F)
@@ -194,12 +218,14 @@ def rope(x, positions, inv_freq, pairing):
     return out.astype(F)
 
 
-def attention(q, k, v, nq, nkv, window=None, scale=None):
+def attention(q, k, v, nq, nkv, window=None, scale=None, rnd=_same):
     """softmax over the keys a query may see of (q . k_j) * rsqrt(hd), times v
     (kernels/megakernel_ops.hip:2192-2194 kv head = q head / (nq/nkv) and the scale,
     :2310-2342 the softmax; causality is the loop bound j <= i, compile_attention.rs:285).
     Window W (ours; the reference has none): query i sees keys j with i - W < j <= i.
-    q: [T, nq, hd], k, v: [T, nkv, hd] -> [T, nq, hd]."""
+    q: [T, nq, hd], k, v: [T, nkv, hd] -> [T, nq, hd].
+    `rnd` rounds the unnormalised probabilities exp(s - max) that multiply the values (the
+    divisor stays the float sum of the unrounded ones)."""
     T, _, hd = q.shape
     scale = F(1.0 / math.sqrt(hd)) if scale is None else F(scale)
     out = np.zeros((T, nq, hd), dtype=F)
@@ -215,8 +241,11 @@ def attention(q, k, v, nq, nkv, window=None, scale=None):
         s = np.where(allowed, s, F(-np.inf))
         m = s.max(axis=-1, keepdims=True)
         e = np.exp(s - m, dtype=F)
-        p = e / e.sum(axis=-1, keepdims=True, dtype=F)
-        out[:, h, :] = p.astype(F) @ v[:, kh, :].astype(F)
+        if rnd is _same:
+            p = e / e.sum(axis=-1, keepdims=True, dtype=F)
+            out[:, h, :] = p.astype(F) @ v[:, kh, :].astype(F)
+        else:
+            out[:, h, :] = (rnd(e) @ v[:, kh, :].astype(F)) / e.sum(axis=-1, keepdims=True, dtype=F)
     return out
 
 
@@ -226,30 +255,30 @@ def silu(x):
     return (x / (F(1.0) + np.exp(-x, dtype=F))).astype(F)
 
 
-def swiglu(n, Wg, Wu, Wd):
+def swiglu(n, Wg, Wu, Wd, rnd=_same):
     """W_d (silu(W_g n) * (W_u n)) (kernels/megakernel_ops.hip:1538-1544, :1559-1602)."""
-    return linear(silu(linear(n, Wg)) * linear(n, Wu), Wd)
+    return linear(rnd(silu(linear(n, Wg)) * linear(n, Wu)), Wd)
 
 
-def attention_block(x, positions, w, prefix, sz, window):
+def attention_block(x, positions, w, prefix, sz, window, rnd=_same):
     """x + W_o attn(rope(W_q n), rope(W_k n), W_v n), n = norm(x)
     (megakernel/compile_attention.rs:78-376)."""
     T = x.shape[0]
-    n = rms_norm(x, w[prefix + "input_layernorm.weight"], sz["eps"])
-    q = linear(n, w[prefix + "self_attn.q_proj.weight"]).reshape(T, sz["nq"], sz["hd"])
-    k = linear(n, w[prefix + "self_attn.k_proj.weight"]).reshape(T, sz["nkv"], sz["hd"])
-    v = linear(n, w[prefix + "self_attn.v_proj.weight"]).reshape(T, sz["nkv"], sz["hd"])
+    n = rnd(rms_norm(x, w[prefix + "input_layernorm.weight"], sz["eps"]))
+    q = rnd(linear(n, w[prefix + "self_attn.q_proj.weight"])).reshape(T, sz["nq"], sz["hd"])
+    k = rnd(linear(n, w[prefix + "self_attn.k_proj.weight"])).reshape(T, sz["nkv"], sz["hd"])
+    v = rnd(linear(n, w[prefix + "self_attn.v_proj.weight"])).reshape(T, sz["nkv"], sz["hd"])
     inv = rope_inv_freq(sz["hd"], sz["theta"])
-    q, k = rope(q, positions, inv, sz["pairing"]), rope(k, positions, inv, sz["pairing"])
-    o = attention(q, k, v, sz["nq"], sz["nkv"], window).reshape(T, sz["nq"] * sz["hd"])
+    q, k = rnd(rope(q, positions, inv, sz["pairing"])), rnd(rope(k, positions, inv, sz["pairing"]))
+    o = rnd(attention(q, k, v, sz["nq"], sz["nkv"], window, rnd=rnd)).reshape(T, sz["nq"] * sz["hd"])
     return (x + linear(o, w[prefix + "self_attn.o_proj.weight"])).astype(F)
 
 
-def ffn_block(x, w, prefix, sz):
+def ffn_block(x, w, prefix, sz, rnd=_same):
     """x + swiglu(norm(x)) (megakernel/compile_layers.rs:373-386)."""
-    n = rms_norm(x, w[prefix + "post_attention_layernorm.weight"], sz["eps"])
+    n = rnd(rms_norm(x, w[prefix + "post_attention_layernorm.weight"], sz["eps"]))
     return (x + swiglu(n, w[prefix + "mlp.gate_proj.weight"], w[prefix + "mlp.up_proj.weight"],
-                       w[prefix + "mlp.down_proj.weight"])).astype(F)
+                       w[prefix + "mlp.down_proj.weight"], rnd)).astype(F)
 
 
 def layer_window(sz, i):
@@ -260,18 +289,21 @@ def layer_window(sz, i):
     return sz["window"] if sz["layer_types"][i] == "sliding_attention" else None
 
 
-def forward(cfg, w, tokens, positions=None):
+def forward(cfg, w, tokens, positions=None, act_dtype=None):
     """Logits [T, V] of one whole sequence (layer loop megakernel/megakernel_compile.rs:115-236;
-    final norm and lm_head :238-262)."""
+    final norm and lm_head :238-262).  `act_dtype="bfloat16"` rounds the activations a bfloat16
+    engine keeps in bfloat16 (see `rounding`): what such an engine may differ by from the float
+    result through rounding alone."""
+    rnd = rounding(act_dtype)
     sz = sizes(cfg)
     T = len(tokens)
     positions = np.arange(T) if positions is None else np.asarray(positions)
     x = embedding(w["model.embed_tokens.weight"], tokens)
     for i in range(sz["L"]):
         p = f"model.layers.{i}."
-        x = attention_block(x, positions, w, p, sz, layer_window(sz, i))
-        x = ffn_block(x, w, p, sz)
-    n = rms_norm(x, w["model.norm.weight"], sz["eps"])
+        x = attention_block(x, positions, w, p, sz, layer_window(sz, i), rnd)
+        x = ffn_block(x, w, p, sz, rnd)
+    n = rnd(rms_norm(x, w["model.norm.weight"], sz["eps"]))
     head = w["model.embed_tokens.weight"] if sz["tied"] else w["lm_head.weight"]
     return linear(n, head)
 
@@ -348,6 +380,33 @@ def greedy_generate(cfg, w, prompt, max_new_tokens, stop_ids=()):
     out = []
     for _ in range(max_new_tokens):
         nxt = argmax_lowest(forward(cfg, w, toks)[-1])
+        if nxt in stop_ids:
+            break
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+def uniform(seed, sequence, draw):
+    """The uniform number of draw `draw` of request `sequence` under `seed` (ours; the reference
+    seeds a StdRng, sampling.rs:188-191, whose stream exists in Rust only): with
+    mix'(x) = mix64(x + G) (splitmix64's step), key = mix'(mix'(seed) ^ (sequence * 0xD6E8FEB86659FD93)),
+    u = (mix'(key ^ (draw * 0xCA5A826395121157)) >> 40) * 2^-24: 24 bits in [0, 1)."""
+    def step(x):
+        return _mix64((x + _GOLDEN) & _M64)
+    key = step(step(seed & _M64) ^ ((sequence * 0xD6E8FEB86659FD93) & _M64))
+    return (step(key ^ ((draw * 0xCA5A826395121157) & _M64)) >> 40) / float(1 << 24)
+
+
+def sampled_generate(cfg, w, prompt, max_new_tokens, seed, sequence=0, stop_ids=(), **options):
+    """The reference's sampled loop (sampling.rs:181-220): every new token is sampled from the
+    logits of the last position with the history = prompt + everything generated so far, one
+    uniform number a token; as in `greedy_generate` the first token comes from the prompt's last
+    logits and a stop token ends the sequence without being emitted."""
+    toks = list(prompt)
+    out = []
+    for k in range(max_new_tokens):
+        nxt = sample(forward(cfg, w, toks)[-1], uniform(seed, sequence, k), history=toks, **options)
         if nxt in stop_ids:
             break
         out.append(nxt)

@@ -189,6 +189,50 @@ def test_the_chain_by_hand(tiny_folders):
         eng.free_slot(s)
 
 
+def test_a_chain_keeps_two_steps_unread_while_sequences_take_new_pages(tiny_folders):
+    """64 sequences whose lengths straddle a page edge: in each of the next steps some of them take a
+    new page (a changed piece of the block table goes to the device).  Launching must not wait for the
+    device: with torch's check for synchronizing calls set to raise, two steps are launched and left
+    unread across such steps; the tokens are those of single steps on an engine without graphs."""
+    import torch
+    folder, cfg, w = tiny_folders["b"]
+    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=64 * 192)
+    plain = B.Engine.from_folder(folder, dtype="float32", max_tokens=64 * 192, use_graphs=False)
+    lens = [58 + i % 8 for i in range(64)]                      # 58..65: pages are taken at steps 0 to 6
+    prompts = prompts_of(cfg, lens, 12)
+    outs = []
+    for e in (eng, plain):
+        slots = [e.alloc_slot() for _ in prompts]
+        first = e.step([B.StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)]).argmax(-1).tolist()
+        got = [first]
+        if e is plain:
+            for _ in range(9):
+                got.append(e.step([B.StepEntry(s, [t], [0]) for s, t in zip(slots, got[-1])]).argmax(-1).tolist())
+        else:
+            chain = e.chain(slots, first)
+            chain.launch()                                      # records the chain's graph: that may wait
+            got.append(chain.read())
+            pages = [g.pool.held_count for g in e.cache.groups]
+            torch.cuda.set_sync_debug_mode("error")
+            try:
+                with pytest.raises(RuntimeError):               # the check itself: a blocking copy raises
+                    torch.zeros(4, device=e.device).copy_(torch.ones(4))
+                for _ in range(4):
+                    chain.launch()
+                    chain.launch()
+                    torch.cuda.set_sync_debug_mode("default")
+                    got += [chain.read(), chain.read()]          # reading waits, by design
+                    torch.cuda.set_sync_debug_mode("error")
+            finally:
+                torch.cuda.set_sync_debug_mode("default")
+            chain.close()
+            assert [g.pool.held_count for g in e.cache.groups] != pages     # pages were taken on the way
+        outs.append(got)
+        for s in slots:
+            e.free_slot(s)
+    assert outs[0] == outs[1]
+
+
 def test_command_line(tiny_folders):
     folder, cfg, w = tiny_folders["a"]
     p = [7, 3, 200, 5]
@@ -199,7 +243,7 @@ def test_command_line(tiny_folders):
     assert r.returncode == 0, r.stderr
     assert [int(t) for t in r.stdout.split()] == want
     assert "PPTG pp=" in r.stderr and "tokens in" in r.stderr and "stop tokens:" in r.stderr
-    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), folder, "--dtype", "float32",
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "generate"), folder, "--dtype", "fp32",
                         "--prompt-ids", "1,2", "--prompt-ids", "3,4,5"],
                        env={k: v for k, v in env.items() if k != "MODEL"}, capture_output=True, text=True)
     assert r.returncode == 0 and len(r.stdout.strip().splitlines()) == 2

@@ -193,3 +193,33 @@ def test_sampler_filters():
     assert P.sample(logits, u=float(cum[0]) - 1e-3) == 0 and P.sample(logits, u=float(cum[0]) + 1e-3) == 1
     # a repeated token is penalised once per occurrence
     assert P.sample([4.0, 3.9], u=0.0, temperature=0.0, repetition_penalty=1.01, history=[0, 0, 0]) == 1
+
+
+def test_uniform_numbers_and_the_sampled_loop():
+    us = [P.uniform(7, s, d) for s in range(3) for d in range(200)]
+    assert all(0.0 <= u < 1.0 for u in us) and len(set(us)) > 590           # 24 bits: hardly a repeat in 600
+    assert abs(np.mean(us) - 0.5) < 0.05
+    assert P.uniform(7, 1, 5) == P.uniform(7, 1, 5) != P.uniform(8, 1, 5)
+    cfg = dict(num_hidden_layers=1, hidden_size=16, num_attention_heads=2, num_key_value_heads=1, head_dim=8,
+               intermediate_size=24, vocab_size=20)
+    w = P.random_weights(cfg, 3, std=0.5)
+    # temperature 0 through the sampled loop is the greedy loop; a request's tokens depend on its number
+    assert P.sampled_generate(cfg, w, [1, 2, 3], 5, seed=1, temperature=0.0) == P.greedy_generate(cfg, w, [1, 2, 3], 5)
+    a = P.sampled_generate(cfg, w, [1, 2, 3], 12, seed=1, sequence=0, temperature=1.5)
+    assert a == P.sampled_generate(cfg, w, [1, 2, 3], 12, seed=1, sequence=0, temperature=1.5)
+    assert a != P.sampled_generate(cfg, w, [1, 2, 3], 12, seed=1, sequence=1, temperature=1.5)
+
+
+def test_rounding_to_bfloat16():
+    import torch
+    x = np.random.default_rng(0).standard_normal(5000).astype(np.float32) * np.float32(3.0)
+    x[:4] = [1.0, 1.00390625, 1.01171875, -0.0]          # a tie that goes down to even, one that goes up
+    assert np.array_equal(P.bf16_round(x), torch.from_numpy(x).bfloat16().float().numpy())
+    cfg = dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+               intermediate_size=96, vocab_size=50)
+    w = P.random_weights(cfg, 1, std=0.1)
+    toks = list(range(1, 30))
+    a, b = P.forward(cfg, w, toks), P.forward(cfg, w, toks, act_dtype="bfloat16")
+    assert np.array_equal(a, P.forward(cfg, w, toks, act_dtype="float32"))
+    d = np.abs(a - b).max() / np.abs(a).max()
+    assert 1e-5 < d < 2e-2                                 # rounding moves the logits, by about 2^-8 of them

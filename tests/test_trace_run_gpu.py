@@ -84,7 +84,7 @@ def test_replay_under_every_cut(tiny_folders, tmp_path, name, dtype):
 
 def test_bad_input_is_an_error_not_a_crash(tiny_folders, tmp_path):
     folder, cfg, _ = tiny_folders["a"]
-    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "fp32",
                         "--out", str(tmp_path / "o"), "--max-tokens", "64"],
                        input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [99999], "want": [0]}], "end": []}) + "\n",
                        capture_output=True, text=True)

@@ -146,6 +146,11 @@ def test_shard_errors(tmp_path):
     json.dump({"weight_map": []}, open(index_path, "w"))
     with pytest.raises(B.WeightError, match="weight_map"):
         SafetensorsFolder(folder)
+    # a file name that leads out of the folder is refused before anything is opened
+    for elsewhere in ("../m2/" + files[0], os.path.join(str(tmp_path), "m", files[0]), "sub/" + files[0]):
+        json.dump({"weight_map": dict(index["weight_map"], **{dup: elsewhere})}, open(index_path, "w"))
+        with pytest.raises(B.WeightError, match="outside the model folder"):
+            SafetensorsFolder(folder)
 
 
 def test_dtypes_kept(tmp_path):
