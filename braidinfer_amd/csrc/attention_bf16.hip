@@ -488,32 +488,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             const int krow = kl + key_of_row32(c);
             const int kswz_ = KCOLS == 16 ? (krow & 15) : ((krow >> 1) & 7);
             const unsigned char* kp = st + krow * KROWB;
-            f32x16 s_acc;
+            f32x16 sv;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+            for (int r = 0; r < 16; ++r) sv[r] = 0.f;
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int s = 0; s < 2 * NB; ++s) {
                 const bf16x8 kf = *(const bf16x8*)(kp + (((2 * s + g) ^ kswz_) * 16));
-                s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+                sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sv, 0, 0, 0);
             }
             __builtin_amdgcn_s_setprio(0);
-            float sv[16];
-            float mx = -INFINITY;
             const bool whole = row0 + 31 < rows_total && kb + 31 <= pq_min_w &&
                                (window <= 0 || kb > pq_max_w - window);
-            if (whole) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { sv[r] = s_acc[r]; mx = fmaxf(mx, sv[r]); }
-            } else {
+            if (!whole) {                                  // masked in place: only blocks at the diagonal and the window's edge
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
                     const bool ok = row_ok && key <= pq && (window <= 0 || key > pq - window);
-                    sv[r] = ok ? s_acc[r] : -INFINITY;
-                    mx = fmaxf(mx, sv[r]);
+                    sv[r] = ok ? sv[r] : -INFINITY;
                 }
             }
+            float mx = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+#pragma unroll
+            for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, sv[r]), sv[r + 1]);
+            mx = fmaxf(mx, sv[15]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;      // the scale is positive
             const float m_new = fmaxf(m, mx);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -526,15 +524,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                     for (int r = 0; r < 16; ++r) acc_o[i2][r] *= corr;
             }
-            float psum = 0.f;
+            float ps0 = 0.f, ps1 = 0.f;
             bf16x8 p1, p2;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float p = fast_exp2(fmaf(sv[r], scale2, -m_use));
-                psum += p;
-                if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
+            for (int r = 0; r < 16; r += 2) {
+                const float pa = fast_exp2(fmaf(sv[r], scale2, -m_use));
+                const float pb = fast_exp2(fmaf(sv[r + 1], scale2, -m_use));
+                ps0 += pa;
+                ps1 += pb;
+                if (r < 8) { p1[r] = (bf16)pa; p1[r + 1] = (bf16)pb; }
+                else { p2[r - 8] = (bf16)pa; p2[r - 7] = (bf16)pb; }
             }
-            lsum += psum;
+            lsum += ps0 + ps1;
             m = m_new;
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
@@ -545,10 +546,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 bf16x8 v1 = *(const bf16x8*)(vp + (((kl / 8 + g) ^ vswz) * 16));
                 bf16x8 v2 = *(const bf16x8*)(vp + (((kl / 8 + g + 2) ^ vswz) * 16));
                 if (tail_page) {
+                    // keys of this lane's two value fragments that lie inside the context; the count is made
+                    // opaque here so that its compares stay inside the branch (they were computed for every page)
+                    int live = ctx - (kb + 8 * g);
+                    asm volatile("" : "+v"(live));
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        if (kb + 8 * g + e >= ctx) v1[e] = (bf16)0.f;
-                        if (kb + 16 + 8 * g + e >= ctx) v2[e] = (bf16)0.f;
+                        if (e >= live) v1[e] = (bf16)0.f;
+                        if (e + 16 >= live) v2[e] = (bf16)0.f;
                     }
                 }
                 acc_o[i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i2], 0, 0, 0);
