@@ -18,7 +18,7 @@ that lie wholly before the window to its pool after every step.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -38,10 +38,21 @@ class CacheNeed:
     head_dim: int
     window: Optional[int] = None      # None: all keys; W: the last W positions
     value_dim: Optional[int] = None
+    # Which rows later tokens can still see, for mixers with another rule than "all" or "the last W": a
+    # function from a sequence's length to the first position that stays visible (rows before it are never
+    # read again, pages wholly before it go back to the pool).  None: the window's rule.  Units whose needs
+    # are to share a group name the same function object.
+    live_from: Optional[Callable[[int], int]] = None
 
     @property
     def key_dim(self) -> int:
         return self.head_dim
+
+    def first_live(self, length: int) -> int:
+        """The first position of a sequence of `length` tokens that a later token may still read."""
+        if self.live_from is not None:
+            return max(0, min(int(length), int(self.live_from(int(length)))))
+        return 0 if self.window is None else max(0, length - self.window + 1)
 
     @property
     def val_dim(self) -> int:
@@ -144,11 +155,10 @@ class CacheGroup:
             self._mark(slot, have, want)
 
     def trim(self, slot: int, length: int) -> None:
-        """Return pages that no later query can see (windowed groups only)."""
-        w = self.need.window
-        if w is None:
+        """Return pages that no later query can see (by the window, or by the need's own rule)."""
+        if self.need.window is None and self.need.live_from is None:
             return
-        first_live = max(0, length - w + 1) // self.page_tokens
+        first_live = self.need.first_live(length) // self.page_tokens
         lo = self.first_page[slot]
         if first_live > lo:
             dead = [p for p in self.pages[slot][lo:first_live] if p >= 0]

@@ -189,13 +189,21 @@ class Engine:
         try:
             starts = [self.cache.lengths[s] for s in slots]
             n_want = len(rows)
-            if (self.use_graphs and probe is None and position_ids is None and all(n == 1 for n in new)
-                    and len(slots) <= 256):
+            if self.use_graphs and probe is None and all(n == 1 for n in new) and len(slots) <= 256:
                 if self._graphs is None:
                     from .graph import DecodeGraphs
                     self._graphs = DecodeGraphs(self.model, self.cache, self.device)
-                g = self._graphs.of(len(slots))
-                all_logits = g.run(slots, [tl[0] for tl in token_lists], starts)
+                pid = None
+                if position_ids is not None:
+                    # the caller's position numbers, k per token: a recorded step of their own per k
+                    try:
+                        pid = np.asarray([p[0] for p in position_ids], dtype=np.int64).reshape(len(slots), -1)
+                    except (ValueError, TypeError):
+                        pid = np.zeros((len(slots), 0), dtype=np.int64)
+                    if pid.shape[1] == 0 or np.abs(pid).max() >= 2 ** 31:
+                        raise StepError("position_ids: every token needs the same number of position numbers, each a 32-bit integer")
+                g = self._graphs.of(len(slots), 0 if pid is None else pid.shape[1])
+                all_logits = g.run(slots, [tl[0] for tl in token_lists], starts, pid)
                 # the graph's buffer is overwritten by the next step: the wanted rows go into a tensor
                 # of the caller's own (one copy kernel; nothing wanted: nothing copied)
                 logits = torch.empty((n_want, V), dtype=torch.float32, device=self.device)

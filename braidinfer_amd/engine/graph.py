@@ -37,21 +37,29 @@ class DecodeGraph:
     may be another graph's capture, where destroying a graph or freeing device memory is
     not permitted)."""
 
-    def __init__(self, model, cache, device, batch: int):
+    def __init__(self, model, cache, device, batch: int, position_numbers: int = 0):
+        """`position_numbers` k > 0: the step's position encodings read k numbers per token that the
+        caller brings with every step (`StepEntry.position_ids`), kept in the same refreshed array;
+        0: they read the tokens' places in their sequences."""
         self.B = B = batch
+        self.k = k = int(position_numbers)
         dev = device
         self.ws = Workspace(dev)            # its buffers belong to the recorded graph for good
-        # one int32 array: tokens | positions | slots | ctx   (refreshed per step)
-        self.ints = torch.zeros(4 * B, dtype=torch.int32, device=dev)
+        # one int32 array: tokens | positions | slots | ctx | the caller's position numbers   (refreshed per step)
+        self.ints = torch.zeros((4 + k) * B, dtype=torch.int32, device=dev)
         self.ints[2 * B:3 * B] = -1
         ar = torch.arange(B + 1, dtype=torch.int32, device=dev)
         self.want_rows = ar[:B].contiguous()
+        pid = None
+        if k:
+            pid = self.ints[4 * B:(4 + k) * B]
+            pid = pid if k == 1 else pid.view(B, k)
         self.step = StepBatch(
             n_tokens=B, n_seqs=B, tokens=self.ints[0:B], positions=self.ints[B:2 * B],
             seq_of_token=self.want_rows, cu_seqlens=ar, slots=self.ints[2 * B:3 * B],
             ctx_lens=self.ints[3 * B:4 * B], host_slots=[-1] * B, host_new=[1] * B, host_start=[0] * B,
             is_decode=True, max_new=1, max_ctx=cache.max_seq_len,
-            max_ctx_bound=cache.max_seq_len, ws=self.ws)
+            max_ctx_bound=cache.max_seq_len, ws=self.ws, position_ids=pid)
         # once eagerly with padding only: loads the kernels, sizes the workspace, stores nothing
         self.logits = torch.empty((B, model.spec.vocab_size), dtype=torch.float32, device=dev)
         model.forward(self.step, cache, self.want_rows, B, self.logits)
@@ -71,22 +79,22 @@ class DecodeGraph:
         self.model, self.cache, self.device = model, cache, dev
         # the step's arrays on the host, pinned, so that the copy to the device does not wait
         # (two, used in turn: a buffer is written again only when its last copy has been made)
-        self.host_ints = [torch.zeros(4 * B, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.host_ints = [torch.zeros((4 + k) * B, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self.host_copied = [None, None]
         self.host_turn = 0
         self.greedy_graph = None
         self.next_tokens = torch.zeros(B, dtype=torch.int32, device=dev)
         self.owner = None                # the chain whose sequences the device arrays describe, if any
 
-    def load(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int]) -> None:
+    def load(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int], position_ids=None) -> None:
         """Write the step's arrays: tokens, positions, slots and lengths of the n live rows,
-        padding rows behind them."""
+        padding rows behind them; `position_ids` [n, k] for a graph recorded with k position numbers."""
         B, n = self.B, len(slots)
-        k = self.host_turn
+        turn = self.host_turn
         self.host_turn ^= 1
-        if self.host_copied[k] is not None:
-            self.host_copied[k].synchronize()
-        h = self.host_ints[k].numpy()
+        if self.host_copied[turn] is not None:
+            self.host_copied[turn].synchronize()
+        h = self.host_ints[turn].numpy()
         h[0:n] = tokens
         h[B:B + n] = starts
         h[2 * B:2 * B + n] = slots
@@ -97,14 +105,18 @@ class DecodeGraph:
             h[B + n:2 * B] = 0
             h[2 * B + n:3 * B] = -1
             h[3 * B + n:4 * B] = 0
-        self.ints.copy_(self.host_ints[k], non_blocking=True)
-        if self.host_copied[k] is None:
-            self.host_copied[k] = torch.cuda.Event()
-        self.host_copied[k].record()
+        if self.k:
+            pid = h[4 * B:].reshape(B, self.k)
+            pid[:n] = position_ids
+            pid[n:] = 0
+        self.ints.copy_(self.host_ints[turn], non_blocking=True)
+        if self.host_copied[turn] is None:
+            self.host_copied[turn] = torch.cuda.Event()
+        self.host_copied[turn].record()
 
-    def run(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int]) -> torch.Tensor:
+    def run(self, slots: Sequence[int], tokens: Sequence[int], starts: Sequence[int], position_ids=None) -> torch.Tensor:
         self.owner = None
-        self.load(slots, tokens, starts)
+        self.load(slots, tokens, starts, position_ids)
         self.graph.replay()
         return self.logits[:len(slots)]
 
@@ -144,10 +156,16 @@ class DecodeGraphs:
     def __init__(self, model, cache, device, max_batch: int = 256):
         self.model, self.cache, self.device = model, cache, device
         self.max_batch = max_batch
-        self.graphs: Dict[int, DecodeGraph] = {}
+        self.graphs: Dict[int, DecodeGraph] = {}          # plain steps, by bucket
+        self.with_ids: Dict[tuple, DecodeGraph] = {}      # steps that bring k position numbers, by (bucket, k)
 
-    def of(self, n: int) -> DecodeGraph:
+    def of(self, n: int, position_numbers: int = 0) -> DecodeGraph:
         b = bucket_of(n)
+        if position_numbers:
+            g = self.with_ids.get((b, position_numbers))
+            if g is None:
+                g = self.with_ids[(b, position_numbers)] = DecodeGraph(self.model, self.cache, self.device, b, position_numbers)
+            return g
         g = self.graphs.get(b)
         if g is None:
             g = self.graphs[b] = DecodeGraph(self.model, self.cache, self.device, b)

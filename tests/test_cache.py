@@ -181,3 +181,26 @@ def test_random_walk_never_loses_or_doubles_a_page():
     for s in list(live):
         c.free_slot(s)
     assert all(g.pool.held_count == 0 for g in c.groups)
+
+
+def test_a_need_with_a_rule_of_its_own_gives_back_what_the_rule_says():
+    """`CacheNeed.live_from`: here chunks of 128 tokens, of which only the running one stays visible (the rule
+    of a mixer that attends within chunks): when a sequence enters a new chunk, the pages of the chunk before
+    go back; a group with the window's rule beside it is untouched by that."""
+    chunk = lambda n: (n // 128) * 128
+    needs = {0: CacheNeed(2, 16, live_from=chunk), 1: CacheNeed(2, 16, live_from=chunk), 2: CacheNeed(2, 16, 100)}
+    c = SequenceCache(needs, {}, max_tokens=64 * 12, dtype=None)
+    assert len(c.groups) == 2 and c.groups[0].unit_ids == [0, 1]
+    assert needs[0].first_live(127) == 0 and needs[0].first_live(128) == 128 and needs[0].first_live(300) == 256
+    assert CacheNeed(2, 16, 100).first_live(150) == 51 and CacheNeed(2, 16).first_live(150) == 0
+    gc, gw = c.groups
+    s = c.alloc_slot()
+    for n in (100, 27, 1, 127, 130):                                          # lengths 100, 127, 128, 255, 385
+        c.reserve([s], [n]); c.commit([s], [n])
+        first = chunk(c.lengths[s]) // 64
+        assert gc.pool.held_count == len(gc.pages[s]) - first and gc.first_page[s] == first
+        assert all(p == -1 for p in gc.pages[s][:first]) and all(p >= 0 for p in gc.pages[s][first:])
+        assert (gc.table_cpu[s, :first] == -1).all()
+    assert gw.pool.held_count == 3                                            # 385 tokens, the last 100: pages 4 to 6
+    c.free_slot(s)
+    assert gc.pool.held_count == 0 and gw.pool.held_count == 0

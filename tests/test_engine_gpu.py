@@ -274,6 +274,43 @@ def test_graph_replays_equal_eager_steps(tiny_folders, dtype):
             break
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_with_the_callers_position_numbers_replay_from_graphs_too(tiny_folders, dtype):
+    """Single-token steps whose entries bring position numbers of their own (here each token's place plus
+    1,000: rotary attention sees distances only, so the plain forward at shifted positions is the reference
+    and equals the unshifted one) run from recorded steps of their own, next to the plain ones, with the
+    results of eager steps."""
+    folder, cfg, w = tiny_folders["a"]
+    g = B.Engine.from_folder(folder, dtype=dtype, max_tokens=2048)
+    e = B.Engine.from_folder(folder, dtype=dtype, max_tokens=2048, use_graphs=False)
+    seqs = [tokens(cfg, 40, 70 + i) for i in range(3)]
+    refs = [P.forward(cfg, w, q, positions=np.arange(len(q)) + 1000) for q in seqs]
+    assert all(np.abs(r - P.forward(cfg, w, q)).max() < 1e-4 * np.abs(r).max() for r, q in zip(refs, seqs))
+    got = {}
+    for eng in (g, e):
+        slots = [eng.alloc_slot() for _ in seqs]
+        n0 = [5, 17, 30]
+        eng.step([StepEntry(sl, q[:n], [], position_ids=[1000 + t for t in range(n)]) for sl, q, n in zip(slots, seqs, n0)])
+        rows = [[] for _ in seqs]
+        for k in range(10):
+            live = [i for i in range(3) if n0[i] + k < 40]
+            out = eng.step([StepEntry(slots[i], [seqs[i][n0[i] + k]], [0], position_ids=[1000 + n0[i] + k]) for i in live])
+            # a plain step of another request in between: its recorded step is another one
+            other = eng.alloc_slot()
+            eng.step([StepEntry(other, [3], [0])])
+            eng.free_slot(other)
+            for r, i in enumerate(live):
+                rows[i].append(out[r:r + 1].cpu().numpy())
+        for sl in slots:
+            eng.free_slot(sl)
+        got[eng.use_graphs] = [np.concatenate(r) for r in rows]
+    assert g._graphs is not None and (4, 1) in g._graphs.with_ids and 1 in g._graphs.graphs and e._graphs is None
+    for i in range(3):
+        ref = refs[i][[5, 17, 30][i]:[5, 17, 30][i] + 10]
+        close(got[True][i], ref, dtype, f"request {i} with shifted positions, from a graph")
+        assert np.abs(got[True][i] - got[False][i]).max() <= CUT_TOL[dtype] * np.abs(ref).max()
+
+
 @pytest.mark.parametrize("which", ["all", "some"])
 def test_tensors_stored_in_32_bit_stay_so_in_the_bfloat16_engine(tmp_path, which):
     """A matrix stored as F32 is multiplied in 32-bit even when the engine runs in bfloat16

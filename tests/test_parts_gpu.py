@@ -709,6 +709,9 @@ class LatentMixer(Mixer):
     def cache_need(self):
         return B.cache.CacheNeed(kv_heads=1, head_dim=24, window=self.window, value_dim=8)
 
+    def first_visible(self, pos):
+        return max(0, pos - self.window + 1)
+
     def forward(self, h, x, step, ctx):
         hf = h.float()
         q, k, v = hf @ self.q.T, hf @ self.k.T, hf @ self.v.T
@@ -721,12 +724,28 @@ class LatentMixer(Mixer):
                 pg = int(table[slot, pos // 64])
                 ctx.keys[pg, 0].view(64, 24)[pos % 64] = k[o + i].to(ctx.keys.dtype)
                 ctx.values[pg, 0].view(64, 8)[pos % 64] = v[o + i].to(ctx.values.dtype)
-                lo = max(0, pos - self.window + 1)
+                lo = self.first_visible(pos)
                 ks = torch.stack([ctx.keys[int(table[slot, j // 64]), 0].view(64, 24)[j % 64] for j in range(lo, pos + 1)]).float()
                 vs = torch.stack([ctx.values[int(table[slot, j // 64]), 0].view(64, 8)[j % 64] for j in range(lo, pos + 1)]).float()
                 p = torch.softmax(ks @ q[o + i] / 24 ** 0.5, 0)
                 x[o + i] += (p @ vs) @ self.o.T
             o += n
+
+
+def _chunk_start(length):
+    return (length // 70) * 70
+
+
+class ChunkedLatentMixer(LatentMixer):
+    """The same mixer with another rule of what stays visible: a token sees the tokens of its own chunk of 70
+    (`window` is the chunk's length here).  The cache learns the rule through `CacheNeed.live_from` and gives
+    back the pages of finished chunks."""
+
+    def cache_need(self):
+        return B.cache.CacheNeed(kv_heads=1, head_dim=24, value_dim=8, live_from=_chunk_start)
+
+    def first_visible(self, pos):
+        return _chunk_start(pos)
 
 
 @dataclass(frozen=True)
@@ -741,10 +760,10 @@ class LatentConfig:
         return {"architectures": [self.architecture]}
 
 
-def latent_spec(cfg):
+def latent_spec(cfg, mixer="latent"):
     H = 40
     norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
-    layers = [prenorm_layer(f"l.layers.{i}.", PartSpec("latent", {"hidden_size": H, "window": 70}), None, norm, None, **NAMES)
+    layers = [prenorm_layer(f"l.layers.{i}.", PartSpec(mixer, {"hidden_size": H, "window": 70}), None, norm, None, **NAMES)
               for i in range(2)]
     return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=50,
                      embedding=PartSpec("embedding", {"vocab_size": 50, "hidden_size": H}), layers=layers,
@@ -755,9 +774,12 @@ def latent_spec(cfg):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_mixer_whose_keys_and_values_differ_in_width_uses_the_paged_cache(tmp_path, dtype):
-    register_part("mixer", "latent", LatentMixer)
+@pytest.mark.parametrize("rule", ["window", "chunks"])
+def test_a_mixer_whose_keys_and_values_differ_in_width_uses_the_paged_cache(tmp_path, dtype, rule):
+    """With the window's rule of what stays in the cache, and with a rule of the mixer's own (chunks)."""
+    register_part("mixer", "latent", LatentMixer if rule == "window" else ChunkedLatentMixer)
     register_architecture("ToyLatentForCausalLM", LatentConfig, latent_spec)
+    first_visible = (lambda t: max(0, t - 70 + 1)) if rule == "window" else _chunk_start
     try:
         folder = B.Engine.write_random_folder(str(tmp_path / "l"), LatentConfig(), seed=12, std=0.2)
         eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=512)
@@ -775,7 +797,7 @@ def test_a_mixer_whose_keys_and_values_differ_in_width_uses_the_paged_cache(tmp_
                 n = rd(P.rms_norm(x, w[f"l.layers.{l}.input_layernorm.weight"], 1e-5))
                 q, k, v = n @ w[p + "q.weight"].T, rd(n @ w[p + "k.weight"].T), rd(n @ w[p + "v.weight"].T)
                 for t in range(T):
-                    lo = max(0, t - 70 + 1)
+                    lo = first_visible(t)
                     sc = k[lo:t + 1] @ q[t] / np.sqrt(24.0)
                     pr = np.exp(sc - sc.max()); pr /= pr.sum()
                     x[t] = x[t] + (pr @ v[lo:t + 1]) @ w[p + "o.weight"].T
