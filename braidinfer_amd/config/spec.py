@@ -49,6 +49,11 @@ class LayerSpec:
     norms: Dict[str, PartSpec] = field(default_factory=dict)
     block: str = "prenorm_residual"
     names: Dict[str, str] = field(default_factory=dict)
+    # further mixers of the layer by a role of the architecture's choosing (mixers side by side, say attention
+    # and a recurrent one over the same input): built, loaded and given a cache unit and state like `mixer`;
+    # the block arrangement the layer names is what runs them (`mixer_ctx.others[role]`).  Their tensor-name
+    # pieces are `names["mixer.<role>"]`, their cache units `ScheduleEntry.more_caches[role]`.
+    more_mixers: Dict[str, PartSpec] = field(default_factory=dict)
 
     def name_of(self, what: str) -> str:
         if what not in self.names:
@@ -87,6 +92,8 @@ class ScheduleEntry:
     layer: int
     cache: Optional[int] = None
     writes_cache: bool = True
+    # cache units of the layer's further mixers, by their role in `LayerSpec.more_mixers`
+    more_caches: Dict[str, int] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

@@ -28,6 +28,8 @@ class Layer:
     def __init__(self, spec):
         self.spec = spec
         self.mixer = build_part("mixer", spec.mixer) if spec.mixer else None
+        # further mixers by role (run by the layer's arrangement, each with a context of its own)
+        self.more_mixers: Dict[str, object] = {role: build_part("mixer", ms) for role, ms in spec.more_mixers.items()}
         self.feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward else None
         self.norms: Dict[str, object] = {role: build_part("norm", ns) for role, ns in spec.norms.items()}
         arrangement = block_arrangement(spec.block)
@@ -61,13 +63,17 @@ class Layer:
                 part = self.feed_forward
             elif what.startswith("norm."):
                 part = self.norms.get(what[5:])
+            elif what.startswith("mixer."):
+                part = self.more_mixers.get(what[6:])
             else:
-                raise ConfigError(f"layer {s.prefix!r}: names has {what!r}; known: mixer, feed_forward, norm.<role>")
+                raise ConfigError(f"layer {s.prefix!r}: names has {what!r}; known: mixer, mixer.<role>, feed_forward, "
+                                  "norm.<role>")
             if part is not None:
                 yield part, s.name_of(what)
         named = set(s.names)
         missing = [w for w, p in [("mixer", self.mixer), ("feed_forward", self.feed_forward)]
-                   + [("norm." + r, n) for r, n in self.norms.items()] if p is not None and w not in named]
+                   + [("norm." + r, n) for r, n in self.norms.items()]
+                   + [("mixer." + r, m) for r, m in self.more_mixers.items()] if p is not None and w not in named]
         if missing:
             raise ConfigError(f"layer {s.prefix!r}: no tensor-name piece for {missing}")
 
@@ -91,10 +97,31 @@ class DecoderModel:
                     written.add(e.cache)
                 elif e.cache not in written:
                     raise ConfigError(f"schedule entry reads cache {e.cache} before any entry writes it")
+        for e in self.schedule:
+            unknown = sorted(set(e.more_caches) - set(self.layers[e.layer].more_mixers))
+            if unknown:
+                raise ConfigError(f"schedule entry of layer {e.layer} names cache units for mixers the layer has not: {unknown}")
         for layer in self.layers:
-            if layer.mixer is not None:
-                layer.mixer.check_positions(self.positions)
+            for m in self._mixers_of(layer).values():
+                m.check_positions(self.positions)
         self.rt: Optional[Runtime] = None
+
+    @staticmethod
+    def _mixers_of(layer: Layer) -> Dict[Optional[str], object]:
+        """The layer's mixers by role; the role of `Layer.mixer` is None."""
+        out: Dict[Optional[str], object] = {}
+        if layer.mixer is not None:
+            out[None] = layer.mixer
+        out.update(layer.more_mixers)
+        return out
+
+    @staticmethod
+    def _unit_of(e, role: Optional[str]) -> Optional[int]:
+        return e.cache if role is None else e.more_caches.get(role)
+
+    @staticmethod
+    def _state_key(i: int, role: Optional[str]):
+        return ("entry", i) if role is None else ("entry", i, role)
 
     # ---- weights -------------------------------------------------------------------
     def _named_parts(self):
@@ -140,28 +167,39 @@ class DecoderModel:
     def cache_needs(self) -> Dict[int, CacheNeed]:
         needs: Dict[int, CacheNeed] = {}
         for e in self.schedule:
-            m = self.layers[e.layer].mixer
-            if m is None or e.cache is None:
-                continue
-            n = m.cache_need()
-            if n is None:
-                continue
-            if e.cache in needs and needs[e.cache] != n:
-                raise ConfigError(f"cache unit {e.cache} is shared by mixers with different needs: "
-                                  f"{needs[e.cache]} and {n}")
-            needs[e.cache] = n
+            for role, m in self._mixers_of(self.layers[e.layer]).items():
+                unit = self._unit_of(e, role)
+                if unit is None:
+                    continue
+                n = m.cache_need()
+                if n is None:
+                    continue
+                if unit in needs and needs[unit] != n:
+                    raise ConfigError(f"cache unit {unit} is shared by mixers with different needs: "
+                                      f"{needs[unit]} and {n}")
+                needs[unit] = n
         return needs
 
     def state_needs(self) -> Dict[object, StateNeed]:
         out: Dict[object, StateNeed] = {}
         for i, e in enumerate(self.schedule):
-            m = self.layers[e.layer].mixer
-            if m is None:
-                continue
-            n = m.state_need()
-            if n is not None:
-                out[("entry", i)] = n
+            for role, m in self._mixers_of(self.layers[e.layer]).items():
+                n = m.state_need()
+                if n is not None:
+                    out[self._state_key(i, role)] = n
         return out
+
+    def _mixer_context(self, cache: SequenceCache, e, i: int, role: Optional[str]) -> MixerContext:
+        """What entry i of the run order hands one of its layer's mixers: its cache unit's storage and
+        table, and its slice of the state area."""
+        unit = self._unit_of(e, role)
+        ctx = MixerContext(unit=unit, writes_cache=e.writes_cache)
+        if unit is not None and unit in cache.group_of_unit:
+            g = cache.unit_group(unit)
+            ctx.storage, ctx.block_table, ctx.page_tokens = g.storage_view(unit), g.table_dev, g.page_tokens
+            ctx.keys, ctx.values = g.keys(unit), g.values(unit)
+        ctx.state = cache.state(self._state_key(i, role))
+        return ctx
 
     # ---- one step ----------------------------------------------------------------------
     def forward(self, step: StepBatch, cache: SequenceCache, want_rows: torch.Tensor, n_want: int,
@@ -197,13 +235,10 @@ class DecoderModel:
             step.norm_after_layer = None
             if i + 1 < len(self.schedule):
                 step.norm_after_layer = self.layers[self.schedule[i + 1].layer].first_norm()
-            ctx = MixerContext(unit=e.cache, writes_cache=e.writes_cache)
-            if layer.mixer is not None:
-                if e.cache is not None and e.cache in cache.group_of_unit:
-                    g = cache.unit_group(e.cache)
-                    ctx.storage, ctx.block_table, ctx.page_tokens = g.storage_view(e.cache), g.table_dev, g.page_tokens
-                    ctx.keys, ctx.values = g.keys(e.cache), g.values(e.cache)
-                ctx.state = cache.state(("entry", i))
+            ctx = (self._mixer_context(cache, e, i, None) if layer.mixer is not None
+                   else MixerContext(unit=e.cache, writes_cache=e.writes_cache))
+            for role in layer.more_mixers:
+                ctx.others[role] = self._mixer_context(cache, e, i, role)
             layer.run(layer, x, step, ctx)
         if logits_out is None:
             logits = torch.empty((n_want, self.spec.vocab_size), dtype=torch.float32, device=rt.device)

@@ -198,6 +198,8 @@ class MixerContext:
     page_tokens: int = 0
     writes_cache: bool = True
     state: Optional[torch.Tensor] = None          # [slots, *StateNeed.shape]
+    # the contexts of the layer's further mixers (`LayerSpec.more_mixers`), by role
+    others: Dict[str, "MixerContext"] = field(default_factory=dict)
 
 
 class FeedForward(Part):

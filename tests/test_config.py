@@ -159,3 +159,30 @@ def test_scaled_rotary_frequencies_are_refused_not_ignored():
     B.MistralConfig.from_dict(dict(TINY["a"], rope_scaling={"rope_type": "default"}))
     with pytest.raises(B.ConfigError, match="rope_scaling"):
         B.MistralConfig.from_dict(dict(TINY["a"], rope_scaling={"rope_type": "yarn", "factor": 4.0}))
+
+
+def test_a_layer_spec_with_further_mixers_names_their_tensors_and_cache_units():
+    from braidinfer_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from braidinfer_amd.engine import DecoderModel
+    H = 32
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = lambda w: PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                                "window": w, "position": "rope"})
+    names = {"mixer": "a.", "mixer.local": "b.", "norm.mixer": "n."}
+
+    def spec(schedule, names=names):
+        layer = LayerSpec("l.0.", attn(None), None, {"mixer": norm}, "prenorm_residual", names, more_mixers={"local": attn(4)})
+        return ModelSpec(architecture="X", hidden_size=H, vocab_size=10, embedding=PartSpec("embedding", {"vocab_size": 10, "hidden_size": H}),
+                         layers=[layer], schedule=schedule, final_norm=norm,
+                         lm_head=PartSpec("lm_head", {"vocab_size": 10, "hidden_size": H, "tied_to": None}),
+                         positions={"rope": PartSpec("rope", {"rotary_dim": 16, "theta": 1e4, "pairing": "half"})},
+                         max_position_embeddings=64, embedding_prefix="e.", final_norm_prefix="f.", lm_head_prefix="h.")
+    m = DecoderModel(spec([ScheduleEntry(0, 0, more_caches={"local": 1})]))
+    got = [t.name for t in m.weight_specs()]
+    assert "l.0.a.q_proj.weight" in got and "l.0.b.q_proj.weight" in got and got.index("l.0.a.o_proj.weight") < got.index("l.0.b.q_proj.weight")
+    needs = m.cache_needs()
+    assert sorted(needs) == [0, 1] and needs[0].window is None and needs[1].window == 4
+    with pytest.raises(B.ConfigError, match="mixers the layer has not"):
+        DecoderModel(spec([ScheduleEntry(0, 0, more_caches={"far": 1})]))
+    with pytest.raises(B.ConfigError, match="no tensor-name piece"):
+        DecoderModel(spec([ScheduleEntry(0, 0)], names={"mixer": "a.", "norm.mixer": "n."})).weight_specs()

@@ -254,6 +254,112 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(toy_registered, tm
             assert np.abs(g - refs[i]).max() < tol * np.abs(refs[i]).max(), (round_, i)
 
 
+# ------------------------------------------------------------- mixers side by side ----
+@dataclass(frozen=True)
+class SideConfig:
+    architecture = "ToySideBySideForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls()
+
+    def to_dict(self):
+        return {"architectures": [self.architecture]}
+
+
+def side_by_side(layer, x, step, mixer_ctx):
+    """x += mixer(n) + every further mixer(n), n = norm(x): all read the same normed rows; then the
+    feed-forward half as usual."""
+    h = step.ws.get("side_h", tuple(x.shape), layer.rt.dtype)
+    layer.norms["mixer"].forward(x, h)
+    layer.mixer.forward(h, x, step, mixer_ctx)
+    for role, m in layer.more_mixers.items():
+        m.forward(h, x, step, mixer_ctx.others[role])
+    h2 = step.ws.get("side_h2", tuple(x.shape), layer.rt.dtype)
+    layer.norms["feed_forward"].forward(x, h2)
+    layer.feed_forward.forward(h2, x, step)
+
+
+def side_spec(cfg):
+    H = 48
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    attn = lambda window: PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 1, "head_dim": 16,
+                                                     "window": window, "position": "rope"})
+    ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 56})
+    names = {"mixer": "self_attn.", "feed_forward": "mlp.", "norm.mixer": "input_layernorm.",
+             "norm.feed_forward": "post_attention_layernorm."}
+    layers = [
+        # attention beside a mixer with state of its own
+        LayerSpec("s.layers.0.", attn(None), ffn, {"mixer": norm, "feed_forward": norm}, "side_by_side",
+                  dict(names, **{"mixer.recurrent": "rec."}), more_mixers={"recurrent": PartSpec("running_sum", {"hidden_size": H})}),
+        # attention over everything beside attention over the last 5 tokens, each with a cache unit of its own
+        LayerSpec("s.layers.1.", attn(None), ffn, {"mixer": norm, "feed_forward": norm}, "side_by_side",
+                  dict(names, **{"mixer.local": "local_attn."}), more_mixers={"local": attn(5)}),
+    ]
+    return ModelSpec(architecture=cfg.architecture, hidden_size=H, vocab_size=70,
+                     embedding=PartSpec("embedding", {"vocab_size": 70, "hidden_size": H}), layers=layers,
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1, more_caches={"local": 2})], final_norm=norm,
+                     lm_head=PartSpec("lm_head", {"vocab_size": 70, "hidden_size": H, "tied_to": None}),
+                     positions={"rope": PartSpec("rope", {"rotary_dim": 16, "theta": 1e4, "pairing": "half"})},
+                     max_position_embeddings=512, embedding_prefix="s.embed.", final_norm_prefix="s.norm.",
+                     lm_head_prefix="s.head.")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_with_mixers_side_by_side(tmp_path, dtype):
+    """A layer may hold further mixers by role (`LayerSpec.more_mixers`), each with a cache unit
+    (`ScheduleEntry.more_caches`) and state of its own; an arrangement registered here runs them beside the
+    layer's mixer.  Whole prompts, single tokens and a batch, twice over so that slots and state are used again."""
+    register_part("mixer", "running_sum", RunningSumMixer)
+    register_part("block", "side_by_side", lambda: side_by_side)
+    register_architecture("ToySideBySideForCausalLM", SideConfig, side_spec)
+    try:
+        folder = B.Engine.write_random_folder(str(tmp_path / "s"), SideConfig(), seed=6, std=0.12)
+        eng = B.Engine.from_folder(folder, dtype=dtype, max_tokens=512)
+        assert len(eng.cache.groups) == 2 and sorted(len(g.unit_ids) for g in eng.cache.groups) == [1, 2]
+        assert eng.cache.state_bytes_per_slot == 48 * 4 and not eng.use_graphs        # the toy mixer is not graph safe
+        _, w = P.read_folder(folder)
+        assert "s.layers.0.rec.mix.weight" in w and "s.layers.1.local_attn.q_proj.weight" in w
+        sz = dict(nq=3, nkv=1, hd=16, theta=1e4, eps=1e-5, pairing="half")
+
+        def plain(toks):
+            pos = np.arange(len(toks))
+            x = P.embedding(w["s.embed.weight"], toks)
+            n = P.rms_norm(x, w["s.layers.0.input_layernorm.weight"], 1e-5)
+            x = P.attention_block(x, pos, w, "s.layers.0.", sz, None) + np.cumsum(n, axis=0) @ w["s.layers.0.rec.mix.weight"].T
+            x = P.ffn_block(x, w, "s.layers.0.", sz)
+            local = {k.replace("local_attn.", "self_attn."): v for k, v in w.items()
+                     if k.startswith("s.layers.1.local_attn.") or k == "s.layers.1.input_layernorm.weight"}
+            x = P.attention_block(x, pos, w, "s.layers.1.", sz, None) + (P.attention_block(x, pos, local, "s.layers.1.", sz, 5) - x)
+            x = P.ffn_block(x, w, "s.layers.1.", sz)
+            return P.linear(P.rms_norm(x, w["s.norm.weight"], 1e-5), w["s.head.weight"])
+
+        rng = np.random.default_rng(3)
+        seqs = [[int(t) for t in rng.integers(0, 70, n)] for n in (40, 11, 23)]
+        refs = [plain(q) for q in seqs]
+        tol = 1e-4 if dtype == "float32" else 4e-2
+        for round_ in range(2):
+            slots = [eng.alloc_slot() for _ in seqs]
+            cut = [30, 3, 22]
+            out = eng.step([StepEntry(sl, q[:c], list(range(c))) for sl, q, c in zip(slots, seqs, cut)]).cpu().numpy()
+            got = [[out[sum(cut[:i]):sum(cut[:i + 1])]] for i in range(3)]
+            pos, live = list(cut), [0, 1, 2]
+            while live:
+                out = eng.step([StepEntry(slots[i], [seqs[i][pos[i]]], [0]) for i in live]).cpu().numpy()
+                for r, i in enumerate(live):
+                    got[i].append(out[r:r + 1]); pos[i] += 1
+                for i in [i for i in live if pos[i] == len(seqs[i])]:
+                    eng.free_slot(slots[i]); live.remove(i)
+            assert all(g.pool.held_count == 0 for g in eng.cache.groups)
+            for i in range(3):
+                g = np.concatenate(got[i])
+                assert np.abs(g - refs[i]).max() < tol * np.abs(refs[i]).max(), (round_, i)
+    finally:
+        unregister_architecture("ToySideBySideForCausalLM")
+        unregister_part("block", "side_by_side")
+        unregister_part("mixer", "running_sum")
+
+
 # ------------------------------------------------------- the run order is data too ----
 @dataclass(frozen=True)
 class LoopConfig:
