@@ -442,7 +442,335 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
     tile_epilogue<TM, TN, MODE>(acc, C, M, N, ldc, m0 + wm, n0 + wn, lane);
 }
 
+// ------------------------------------------------------------ gemm_tile_quad -------
+// A BM x BN tile by four waves (2 x 2), one to a SIMD, each summing a quarter of it in the matrix-core
+// registers (256x256: 16 blocks of 32x32, all 256 of them), with the operands of one k-step of 16 in
+// vector registers, twice (the set in use and the set being read from LDS).  Per matrix instruction
+// half the LDS operand bytes of the 64x64 wave tiles above.  With one wave per SIMD nothing fills a gap
+// in that wave's instruction stream, so the order is written out: matrix instructions, LDS reads,
+// direct loads and waits are inline assembly in program order.  The compiler keeps volatile statements
+// in order, but it neither knows their latencies nor that they are matrix instructions: every wait is
+// placed by hand, and so are the idle states that the hardware wants between a register's write and
+// a matrix instruction's read of it (and the reverse).
+// NS stages of 64 k (the layout and swizzle of gemm_tile_dma).  One barrier per k-tile, before its
+// last k-step of 16: by then every wave has read the stage, which is then asked for the k-tile NS on.
+// The blocks hold the product transposed (weight rows are the instruction's first operand), which
+// gives every lane four neighbouring columns of one output row: 16-byte accesses in the epilogue, and
+// the up value of a gate column in the same lane.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+template <int I, int N_, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N_) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N_>(f);
+    }
+}
+template <int OFF>
+__device__ __forceinline__ void quad_read(i32x4& d, unsigned addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d) : "v"(addr), "n"(OFF));
+}
+template <int IMM>
+__device__ __forceinline__ void quad_load(unsigned lds_base, unsigned voff, unsigned long long sbase) {
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                 ::"s"(lds_base), "n"(IMM), "v"(voff), "s"(sbase)
+                 : "m0", "scc", "memory");
+}
+__device__ __forceinline__ void quad_mfma(f32x16& acc, const i32x4& a, const i32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void quad_touch(f32x16& acc) { asm volatile("s_nop 1" : "+a"(acc)); }
+template <int N_>
+__device__ __forceinline__ void quad_wait_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_) : "memory");
+}
+
+// acc[i][j][r]: weight row (output column) n1 + 32 i + 8 (r / 4) + 4 (lane / 32) + r % 4, activation
+// row m1 + 32 j + lane % 32.  Needs ldc % 4 == 0 and C aligned to 16 bytes.
+template <int TI, int TJ, int MODE>
+__device__ __forceinline__ void quad_epilogue(f32x16 (&acc)[TI][TJ], void* __restrict__ C, int M, int N, size_t ldc,
+                                              int m1, int n1, int lane) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const int m = m1 + j * 32 + (lane & 31);
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            const int nb = n1 + i * 32 + 4 * (lane >> 5);
+            if (MODE == OUT_SWIGLU) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int n = nb + 16 * h;                      // gate columns n .. n + 3, N a multiple of 16
+                    if (n >= N) continue;
+                    bf16x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = (bf16)silu_mul(acc[i][j][8 * h + e], acc[i][j][8 * h + 4 + e]);
+                    *(bf16x4*)((bf16*)C + (size_t)m * ldc + (n >> 4) * 8 + (n & 7)) = v;
+                }
+                continue;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nb + 8 * q;
+                const size_t at = (size_t)m * ldc + n;
+                if (n + 3 < N) {
+                    if (MODE == OUT_BF16) {
+                        bf16x4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (bf16)acc[i][j][4 * q + e];
+                        *(bf16x4*)((bf16*)C + at) = v;
+                    } else {
+                        f32x4 v;
+                        if (MODE == OUT_F32_ACC) v = *(const f32x4*)((float*)C + at);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (MODE == OUT_F32_ACC ? v[e] : 0.f) + acc[i][j][4 * q + e];
+                        *(f32x4*)((float*)C + at) = v;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) store_out<MODE>(C, at + e, acc[i][j][4 * q + e]);
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int NS, int MODE>
+__global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                              void* __restrict__ C_, int M, int N, int K, size_t lda,
+                                                              size_t ldc, int tiles_m, int tiles_n, int kt_per_part,
+                                                              size_t part_stride, int wl) {
+    constexpr int STAGE = (BM + BN) * 128;               // bytes
+    constexpr int TI = BN / 64, TJ = BM / 64;            // blocks of a wave: weight rows, activation rows
+    constexpr int NM = TI * TJ;                          // matrix instructions per k-step of 16
+    constexpr int L = (BM + BN) / 32, LA = BM / 32;      // wave-loads per wave and stage; the first LA are A's
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && NS * STAGE <= 160 * 1024 && NS >= 2, "tile");
+    static_assert(TI + TJ <= NM, "schedule: one LDS read behind each of the first matrix instructions");
+    __shared__ __attribute__((aligned(1024))) unsigned char st[NS * STAGE];
+    // blockIdx.y: which run of k-tiles this workgroup sums (one run, or the parts of a split product, each
+    // into a float matrix of its own `part_stride` elements on; runs start at an even k-tile)
+    void* C = MODE == OUT_F32 ? (void*)((float*)C_ + blockIdx.y * part_stride) : C_;
+    const int kt0 = (int)blockIdx.y * kt_per_part;
+    const int total = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = total / 8, xcd = pid % 8, idx = pid / 8;
+        if (pid < per * 8) pid = xcd * per + idx;
+    }
+    const int grp = pid / (8 * tiles_m), in = pid - grp * 8 * tiles_m;
+    int gn = tiles_n - grp * 8;
+    if (gn > 8) gn = 8;
+    const int tile_n = grp * 8 + in % gn, tile_m = in / gn;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+    const int lrow = lane & 31, g = lane >> 5;
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // wave-load q of this wave: rows (4 q + wave) 8 .. + 8 of the stacked tile [A rows | W rows], reached by a
+    // 32-bit byte offset from the matrix's first element (the launcher checks that this suffices)
+    unsigned off[L];
+#pragma unroll
+    for (int q = 0; q < L; ++q) {
+        const int R = (q * 4 + wave) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ ((R >> 1) & 7);
+        if (q < LA) {
+            int r = m0 + R;
+            if (r > M - 1) r = M - 1;
+            off[q] = (unsigned)((size_t)r * lda * 2 + c * 16);
+        } else {
+            int r = n0 + R - BM;
+            if (r > N - 1) r = N - 1;
+            off[q] = (unsigned)(w_row_base(r, K, wl) * 2 + c * 16);
+        }
+    }
+    // at the next k-tile to ask for
+    unsigned long long baseA = (unsigned long long)A + (size_t)kt0 * 128;
+    unsigned long long baseW = (unsigned long long)W + (wl ? (size_t)(kt0 >> 1) * (WL_BLOCK_ELEMS * 2) : (size_t)kt0 * 128);
+    int knext = kt0;
+    const unsigned hopW = wl ? WL_BLOCK_ELEMS * 2 - 128 : 128;                        // bytes from an odd k-tile on
+    const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)st);
+    unsigned ldsw = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);    // where this wave's loads land, stage in use
+    int cur = 0;                                                           // the stage in use
+    // LDS addresses of this lane's operand pieces in the stage in use, per k-step of 16
+    unsigned ra[4], rb[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        const int col = ((kk * 2 + g) ^ ((lrow >> 1) & 7)) * 16;
+        ra[kk] = lds0 + (wm + lrow) * 128 + col;
+        rb[kk] = lds0 + (BM + wn + lrow) * 128 + col;
+    }
+    i32x4 fa[2][TJ], fb[2][TI];
+
+    auto load = [&](auto q_) {
+        constexpr int q = decltype(q_)::value;
+        quad_load<q * 4096>(ldsw, off[q], q < LA ? baseA : baseW);
+    };
+    auto next_tile = [&]() {                                          // the pointers go on to the k-tile after
+        baseA += 128;
+        baseW += (knext & 1) ? hopW : 128;
+        ++knext;
+    };
+    // One k-step of 16 from operand set `use`: NM matrix instructions, and between them the LDS reads
+    // of set `use ^ 1` (k-step rk of the stage that ra/rb point into) and, with LD, the L direct loads.
+    auto substep = [&](auto use_, auto rd_, auto rk_, auto ld_) {
+        constexpr int use = decltype(use_)::value, rk = decltype(rk_)::value;
+        constexpr bool RD = decltype(rd_)::value, LD = decltype(ld_)::value;
+        static_for<0, NM>([&](auto n_) {
+            constexpr int n = decltype(n_)::value;
+            // block (i, j): weight rows i (the instruction's first operand, so the result's rows), activation rows j
+            constexpr int i = n / TJ, j = (i & 1) ? TJ - 1 - n % TJ : n % TJ;
+            quad_mfma(acc[i][j], fb[use][i], fa[use][j]);
+            if constexpr (RD && n < TJ) quad_read<n * 4096>(fa[use ^ 1][n], ra[rk]);
+            if constexpr (RD && n >= TJ && n < TJ + TI) quad_read<(n - TJ) * 4096>(fb[use ^ 1][n - TJ], rb[rk]);
+            if constexpr (LD) static_for<n * L / NM, (n + 1) * L / NM>(load);
+        });
+        if constexpr (RD) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    // One k-tile from the stage in use.  Not LAST: before its last k-step every wave waits for its own
+    // loads of the next k-tile (those of the NS - 2 after that may be on their way) and for the others at
+    // a barrier, which also says that all have read this stage; then it asks for the k-tile NS on into
+    // this stage (LOADS) while it reads the next one's first operands from the next stage.
+    auto step = [&](auto loads_, auto last_) {
+        constexpr bool LOADS = decltype(loads_)::value, LAST = decltype(last_)::value;
+        substep(I0{}, T{}, I1{}, F{});
+        substep(I1{}, T{}, I2{}, F{});
+        substep(I0{}, T{}, I3{}, F{});
+        if constexpr (LAST) {
+            substep(I1{}, F{}, I0{}, F{});
+        } else {
+            quad_wait_loads<LOADS ? (NS - 2) * L : 0>();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            const unsigned delta = cur == NS - 1 ? (unsigned)(-(NS - 1) * STAGE) : (unsigned)STAGE;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {                           // reads: the next stage; loads: this one
+                ra[kk] += delta;
+                rb[kk] += delta;
+            }
+            substep(I1{}, T{}, I0{}, std::integral_constant<bool, LOADS>{});
+            ldsw += delta;
+            cur = cur == NS - 1 ? 0 : cur + 1;
+            if constexpr (LOADS) next_tile();
+        }
+    };
+
+    int nk = K / DMA_BK - kt0;                                         // k-tiles of this run
+    if (nk > kt_per_part) nk = kt_per_part;
+    static_for<0, NS>([&](auto s_) {                                   // the first NS k-tiles, one to a stage
+        constexpr int sg = decltype(s_)::value;
+        if (sg < nk) {
+            static_for<0, L>([&](auto q_) {
+                constexpr int q = decltype(q_)::value;
+                quad_load<sg * STAGE + q * 4096>(ldsw, off[q], q < LA ? baseA : baseW);
+            });
+            next_tile();
+        }
+    });
+    if (nk >= NS) quad_wait_loads<(NS - 1) * L>();
+    else quad_wait_loads<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    static_for<0, TJ>([&](auto n_) { quad_read<decltype(n_)::value * 4096>(fa[0][decltype(n_)::value], ra[0]); });
+    static_for<0, TI>([&](auto n_) { quad_read<decltype(n_)::value * 4096>(fb[0][decltype(n_)::value], rb[0]); });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // Statements that name the accumulators: what the compiler wrote into one (the zeroes) is written before
+    // its statement, and a matrix instruction must not read a register in the states right after its write.
+    static_for<0, NM>([&](auto n_) { quad_touch(acc[decltype(n_)::value / TJ][decltype(n_)::value % TJ]); });
+    int t = 0;
+    for (; t + NS < nk; ++t) step(T{}, F{});
+    for (; t + 1 < nk; ++t) step(F{}, F{});
+    step(F{}, T{});
+    // the last matrix instructions' results are not in their registers yet; the epilogue's reads of an
+    // accumulator stay behind the statement that names it
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    static_for<0, NM>([&](auto n_) { quad_touch(acc[decltype(n_)::value / TJ][decltype(n_)::value % TJ]); });
+    quad_epilogue<TI, TJ, MODE>(acc, C, M, N, ldc, m0 + wm, n0 + wn, lane);
+}
+
 static int launch_split_sum(const float* scratch, int parts, void* C, int M, int N, size_t ldc, int mode, hipStream_t s);
+
+// What the quad tiles ask of a product beyond K % 64 == 0 and aligned rows: the loads reach a row by a
+// 32-bit byte offset from the matrix's first element, and the epilogue stores 16 bytes at a time.
+static bool quad_takes(const void* C, int M, int N, int K, size_t lda, size_t ldc) {
+    return (unsigned long long)M * lda * 2 < (1ull << 32) && ((unsigned long long)N + 16) * K * 2 < (1ull << 32) &&
+           ldc % 4 == 0 && (uintptr_t)C % 16 == 0;
+}
+
+// parts > 1: the k-tiles are cut into runs of an even number of k-tiles, every (tile, run) workgroup writes
+// its float sums to a matrix of its own in `scratch`, and gemm_split_sum_kernel adds the runs in run order
+// and applies the epilogue.
+template <int BM, int BN, int NS>
+static int launch_tile_quad(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
+                            int mode, hipStream_t s, int wl, int parts = 1, float* scratch = nullptr) {
+    const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    const long long total = (long long)tm * tn;
+    if (total > 0x7fffffffLL || !quad_takes(C, M, N, K, lda, ldc)) return BR_BAD_ARG;
+    const int nk = K / DMA_BK;
+    if (parts > 1) {
+        if (N % 4 != 0 || (uintptr_t)scratch % 16 != 0) return BR_BAD_ARG;
+        int kpp = (nk + parts - 1) / parts;
+        kpp += kpp & 1;
+        parts = (nk + kpp - 1) / kpp;                                 // no empty run
+        dim3 grid((unsigned)total, (unsigned)parts);
+        gemm_tile_quad_kernel<BM, BN, NS, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp,
+                                                                        (size_t)M * N, wl);
+        int rc = br_check_launch();
+        if (rc != BR_OK) return rc;
+        return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
+    }
+    if (mode == OUT_BF16)
+        gemm_tile_quad_kernel<BM, BN, NS, OUT_BF16><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+    else if (mode == OUT_F32)
+        gemm_tile_quad_kernel<BM, BN, NS, OUT_F32><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+    else if (mode == OUT_F32_ACC)
+        gemm_tile_quad_kernel<BM, BN, NS, OUT_F32_ACC><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+    else
+        gemm_tile_quad_kernel<BM, BN, NS, OUT_SWIGLU><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+    return br_check_launch();
+}
+
+// Which quad tile (12: 256x256, 13: 128x256 with three stages, 14: 256x192) and how many runs of k-tiles: the
+// least time by a count in microseconds: rounds of workgroups over the chip times k-tiles times what a k-tile
+// takes (measured: 1.62, 0.93 and 1.30 us with every compute unit at work, 1.30, 0.83 and 1.12 with few),
+// plus what a launch costs besides and, when split, the second launch and the traffic of the partial sums.
+static void choose_quad(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* kernel, int* parts) {
+    const int nk = K / DMA_BK;
+    static const int bm[3] = {256, 128, 256}, bn[3] = {256, 256, 192};
+    static const double full[3] = {1.62, 0.93, 1.30}, few[3] = {1.30, 0.83, 1.12};
+    double best = 1e30;
+    *kernel = 13;
+    *parts = 1;
+    for (int k = 0; k < 3; ++k) {
+        const long long tiles = (long long)((M + bm[k] - 1) / bm[k]) * ((N + bn[k] - 1) / bn[k]);
+        for (int p = 1; p <= 16; p *= 2) {
+            if (p > 1 && (p * 4 > nk || N % 4 != 0 || (size_t)p * M * N * sizeof(float) > scratch_bytes)) break;
+            int kpp = (nk + p - 1) / p;
+            kpp += kpp & 1;
+            const long long units = tiles * p, rounds = (units + cus - 1) / cus;
+            const double per = units >= cus ? full[k] : few[k] + (full[k] - few[k]) * (double)units / cus;
+            double t = (double)rounds * kpp * per + (mode == OUT_BF16 ? 8.0 : 12.0);
+            if (p > 1) t += 5.0 + (double)p * M * N * 8.0 / 4e6;
+            if (t < best - 1e-9) { best = t; *kernel = 12 + k; *parts = p; }
+        }
+    }
+}
+
 
 // parts > 1: the k-tiles are cut into `parts` runs, every (tile, run) workgroup writes its
 // float sums to a matrix of its own in `scratch`, and gemm_split_sum_kernel adds the runs in
@@ -1455,7 +1783,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
     const bool wide_ok = aligned && M > 16 && M <= 64 && K % 128 == 0 && K >= 256 &&
                          (!scratch || (uintptr_t)scratch % 16 == 0);
-    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 11 || kernel < 0 || (kernel >= 10 && !dma_ok) ||
+    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 14 || kernel < 0 || (kernel >= 10 && !dma_ok) ||
         (kernel == 11 && mode != OUT_SWIGLU) ||
         (kernel == 9 && (!dma_ok || M > 64)))
         return BR_BAD_ARG;
@@ -1479,6 +1807,13 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel == 7) return M <= 8 ? launch_stream<8, 0>(A, W, C, M, N, K, lda, ldc, mode, s, StreamNorm{}, wl)
                                    : launch_stream<16, 0>(A, W, C, M, N, K, lda, ldc, mode, s, StreamNorm{}, wl);
     int parts = 1;
+    if (chosen && M > 128 && (kernel == 5 || kernel == 6) && quad_takes(C, M, N, K, lda, ldc)) {
+        // More than 128 rows, K in steps of 64: the tiles of one wave per SIMD, where the product's addresses
+        // allow.  (Up to 128 rows the tiles of eight waves below stream the weights faster: 7B shapes at 128
+        // rows, gate/up 59 against 69 us, the 32,768-row head 71 against 85, down 39 against 45.)
+        const int cus = br_device_cus();
+        if (cus > 0) choose_quad(M, N, K, mode, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
+    }
     if (chosen && (kernel == 5 || kernel == 6)) {
         const int cus = br_device_cus();
         if (cus > 0) choose_tile(M, N, K, mode, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
@@ -1508,6 +1843,15 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
             }
         }
     }
+    if (kernel >= 12 && forced_parts > 1) {
+        if (!scratch || (uintptr_t)scratch % 16 || (size_t)forced_parts * M * N * sizeof(float) > scratch_bytes ||
+            forced_parts * 2 > K / DMA_BK)
+            return BR_BAD_ARG;
+        parts = forced_parts;
+    }
+    if (kernel == 12) return launch_tile_quad<256, 256, 2>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
+    if (kernel == 13) return launch_tile_quad<128, 256, 3>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
+    if (kernel == 14) return launch_tile_quad<256, 192, 2>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
     if (kernel == 10) return launch_tile_dma<256, 192, 4, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
     if (kernel == 11) {
         gemm_tile_dma_kernel<256, 256, 2, 4, 2, OUT_SWIGLU><<<(unsigned)(((M + 255) / 256) * ((N + 255) / 256)), 512, 0, s>>>(

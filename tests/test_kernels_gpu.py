@@ -72,7 +72,7 @@ SHAPES = [(1, 64, 64), (5, 100, 96), (17, 192, 320), (64, 301, 100), (33, 1000, 
           (17, 100, 256), (64, 16500, 384), (33, 301, 1152), (48, 4100, 1024)]
 
 
-def _skip_unless_kernel_takes(kernel, M, Kd):
+def _skip_unless_kernel_takes(kernel, M, Kd, N=None):
     if kernel == 3 and (Kd % 8 or M > 64):
         pytest.skip("the skinny kernels take M <= 64 and K in steps of 8")
     if (4 <= kernel <= 6 or kernel in (10, 11)) and Kd % 64:
@@ -81,6 +81,8 @@ def _skip_unless_kernel_takes(kernel, M, Kd):
         pytest.skip("the streaming kernel takes M <= 16 and K in steps of 128 from 1024")
     if kernel == 8 and (M <= 16 or M > 64 or Kd % 128 or Kd < 256):
         pytest.skip("the wide streaming kernel takes 16 < M <= 64 and K in steps of 128 from 256")
+    if 12 <= kernel <= 14 and (Kd % 64 or N is None or N % 4):
+        pytest.skip("the tiles of one wave per SIMD take K in steps of 64 and output rows in steps of 16 bytes")
 
 
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
@@ -105,10 +107,10 @@ def test_gemm_f32_rows_do_not_depend_on_the_batch():
     assert torch.equal(one[0], full[33])
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 13, 14])
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
 def test_gemm_bf16(M, N, Kd, kernel):
-    _skip_unless_kernel_takes(kernel, M, Kd)
+    _skip_unless_kernel_takes(kernel, M, Kd, N)
     a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
     want = a.double() @ w.double().T
     o32 = torch.empty(M, N, device=DEV)
@@ -315,6 +317,60 @@ def test_gemm_with_blocked_weights(M, N, Kd, kernel):
         K.gemm(a, w, torch.empty(M, N + 64, device=DEV))             # a width the blocks do not have
     with pytest.raises(KernelError):
         K.block_weight(rnd(64, 960, dtype=torch.bfloat16))           # K in steps of 128 from 1024
+
+
+@pytest.mark.parametrize("blocked", [False, True])
+@pytest.mark.parametrize("parts", [1, 2, 4])
+@pytest.mark.parametrize("kernel", [12, 13, 14])
+@pytest.mark.parametrize("M,N,Kd", [(130, 516, 1024), (300, 700, 2048), (513, 264, 1152), (65, 1032, 1280), (260, 1500, 1024)])
+def test_gemm_tiles_of_one_wave_per_simd(M, N, Kd, kernel, parts, blocked):
+    """The 256x256, 128x256 and 256x192 tiles of four waves (written-out instruction order, products kept
+    transposed in the matrix-core registers): every epilogue, one run or several along k, either weight
+    layout, tiles that hang over every edge; a strided output whose width is no multiple of four (the
+    elements that no 16-byte store takes); and what they refuse."""
+    code = kernel + (16 * parts if parts > 1 else 0)
+    w_rows = rnd(N, Kd, seed=2, scale=0.5, dtype=torch.bfloat16)
+    a, w = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16), (K.block_weight(w_rows) if blocked else w_rows)
+    want = a.double() @ w_rows.double().T
+    scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
+    o32 = torch.empty(M, N, device=DEV)
+    K.gemm(a, w, o32, kernel=code, scratch=scratch)
+    assert (o32.double() - want).abs().max() < 1e-4 * want.abs().max()
+    again = torch.full((M, N), float("nan"), device=DEV)
+    K.gemm(a, w, again, kernel=code, scratch=scratch)
+    assert torch.equal(again, o32)
+    o16 = torch.empty(M, N + 8, device=DEV, dtype=torch.bfloat16)[:, 8:8 + N]
+    K.gemm(a, w, o16, kernel=code, scratch=scratch)
+    assert (o16.double() - want).abs().max() < 1e-2 * want.abs().max()
+    base = rnd(M, N + 12, seed=3)
+    acc = base.clone()
+    K.gemm(a, w, acc[:, 4:4 + N], accumulate=True, kernel=code, scratch=scratch)
+    assert (acc[:, 4:4 + N].double() - (base[:, 4:4 + N].double() + want)).abs().max() < 1e-4 * want.abs().max()
+    assert torch.equal(acc[:, :4], base[:, :4]) and torch.equal(acc[:, 4 + N:], base[:, 4 + N:])
+    I = (N // 2) // 8 * 8
+    wg, wu = rnd(I, Kd, seed=4, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=5, scale=0.3, dtype=torch.bfloat16)
+    wgu = K.interleave_gate_up(wg, wu)
+    out = torch.empty(M, I, device=DEV, dtype=torch.bfloat16)
+    K.gemm_swiglu(a, K.block_weight(wgu) if blocked else wgu, out, kernel=code, scratch=scratch)
+    g, u = a.double() @ wg.double().T, a.double() @ wu.double().T
+    sw = g / (1 + torch.exp(-g)) * u
+    assert (out.double() - sw).abs().max() < 1e-2 * sw.abs().max()
+    if parts == 1 and not blocked:
+        # a width of N - 2 inside rows of N floats: the last columns go out one by one, the neighbours stay
+        wide = torch.full((M, N), 7.0, device=DEV)
+        K.gemm(a, w_rows[:N - 2], wide[:, :N - 2], kernel=code)
+        assert torch.equal(wide[:, :N - 2], o32[:, :N - 2]) and bool((wide[:, N - 2:] == 7.0).all())
+    with pytest.raises(KernelError):                     # rows that no 16-byte store can take
+        K.gemm(a, w, torch.empty(M, N + 6, device=DEV)[:, 3:3 + N], kernel=code, scratch=scratch)
+    with pytest.raises(KernelError):
+        K.gemm(a, w, torch.empty(M, N + 1, device=DEV)[:, :N], kernel=code, scratch=scratch)
+    if parts > 1:
+        with pytest.raises(KernelError):                 # forced runs need their room
+            K.gemm(a, w, again, scratch=torch.empty(16, device=DEV), kernel=code)
+    # chosen by shape: the same sums where these tiles are taken, and a right result where they are not
+    chosen = torch.empty(M, N + 6, device=DEV)[:, 3:3 + N]
+    K.gemm(a, w, chosen, scratch=scratch)
+    assert (chosen.double() - want).abs().max() < 1e-4 * want.abs().max()
 
 
 def test_gemm_reference_vectors():
@@ -717,12 +773,12 @@ def test_attention_kernels_refuse_what_they_do_not_take():
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("M,I,Kd", [(40, 8264, 256), (64, 328, 1152), (1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
                                     (300, 512, 1024), (129, 200, 192), (1, 2056, 1024), (8, 328, 1152), (13, 4400, 1280),
                                     (100, 264, 4096), (260, 520, 2048)])
 def test_gemm_with_swiglu_epilogue(M, I, Kd, kernel):
-    _skip_unless_kernel_takes(kernel, M, Kd)
+    _skip_unless_kernel_takes(kernel, M, Kd, I)
     a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
     wg, wu = rnd(I, Kd, seed=2, scale=0.3, dtype=torch.bfloat16), rnd(I, Kd, seed=3, scale=0.3, dtype=torch.bfloat16)
     out = torch.empty(M, I, device=DEV, dtype=torch.bfloat16)
