@@ -537,18 +537,24 @@ __device__ __forceinline__ void quad_epilogue(f32x16 (&acc)[TI][TJ], void* __res
     }
 }
 
-template <int BM, int BN, int NS, int MODE>
+template <int BM, int BN, int NSA, int NSB, int MODE>
 __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                               void* __restrict__ C_, int M, int N, int K, size_t lda,
                                                               size_t ldc, int tiles_m, int tiles_n, int kt_per_part,
                                                               size_t part_stride, int wl) {
-    constexpr int STAGE = (BM + BN) * 128;               // bytes
+    constexpr int SA = BM * 128, SB = BN * 128;          // bytes of a stage of activation rows, of weight rows
     constexpr int TI = BN / 64, TJ = BM / 64;            // blocks of a wave: weight rows, activation rows
     constexpr int NM = TI * TJ;                          // matrix instructions per k-step of 16
-    constexpr int L = (BM + BN) / 32, LA = BM / 32;      // wave-loads per wave and stage; the first LA are A's
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && NS * STAGE <= 160 * 1024 && NS >= 2, "tile");
-    static_assert(TI + TJ <= NM, "schedule: one LDS read behind each of the first matrix instructions");
-    __shared__ __attribute__((aligned(1024))) unsigned char st[NS * STAGE];
+    constexpr int LA = BM / 32, LB = BN / 32;            // wave-loads per wave and stage
+    // An operand with three stages is asked for during the first three k-steps of 16 of a k-tile, into the
+    // stage that the barrier before freed, and has a whole k-tile more to arrive; one with two stages after
+    // the barrier, into the stage just read.  Either way k-tile t asks for k-tile t + 2.
+    constexpr bool EARLY_A = NSA == 3, EARLY_B = NSB == 3;
+    constexpr int NEARLY = (EARLY_A ? LA : 0) + (EARLY_B ? LB : 0), NLATE = LA + LB - NEARLY;
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && NSA * SA + NSB * SB <= 160 * 1024, "tile");
+    static_assert((NSA == 2 || NSA == 3) && (NSB == 2 || NSB == 3), "two or three stages an operand");
+    static_assert(TI + TJ <= NM && NLATE <= 2 * NM, "schedule");
+    __shared__ __attribute__((aligned(1024))) unsigned char st[NSA * SA + NSB * SB];
     // blockIdx.y: which run of k-tiles this workgroup sums (one run, or the parts of a split product, each
     // into a float matrix of its own `part_stride` elements on; runs start at an even k-tile)
     void* C = MODE == OUT_F32 ? (void*)((float*)C_ + blockIdx.y * part_stride) : C_;
@@ -576,21 +582,22 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // wave-load q of this wave: rows (4 q + wave) 8 .. + 8 of the stacked tile [A rows | W rows], reached by a
-    // 32-bit byte offset from the matrix's first element (the launcher checks that this suffices)
-    unsigned off[L];
+    // wave-load q of this wave: rows (4 q + wave) 8 .. + 8 of the operand's tile, reached by a 32-bit byte
+    // offset from the matrix's first element (the launcher checks that this suffices)
+    unsigned offA[LA], offB[LB];
 #pragma unroll
-    for (int q = 0; q < L; ++q) {
+    for (int q = 0; q < (LA > LB ? LA : LB); ++q) {
         const int R = (q * 4 + wave) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((R >> 1) & 7);
         if (q < LA) {
             int r = m0 + R;
             if (r > M - 1) r = M - 1;
-            off[q] = (unsigned)((size_t)r * lda * 2 + c * 16);
-        } else {
-            int r = n0 + R - BM;
+            offA[q] = (unsigned)((size_t)r * lda * 2 + c * 16);
+        }
+        if (q < LB) {
+            int r = n0 + R;
             if (r > N - 1) r = N - 1;
-            off[q] = (unsigned)(w_row_base(r, K, wl) * 2 + c * 16);
+            offB[q] = (unsigned)(w_row_base(r, K, wl) * 2 + c * 16);
         }
     }
     // at the next k-tile to ask for
@@ -599,32 +606,56 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
     int knext = kt0;
     const unsigned hopW = wl ? WL_BLOCK_ELEMS * 2 - 128 : 128;                        // bytes from an odd k-tile on
     const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)st);
-    unsigned ldsw = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);    // where this wave's loads land, stage in use
-    int cur = 0;                                                           // the stage in use
-    // LDS addresses of this lane's operand pieces in the stage in use, per k-step of 16
+    // where this wave's loads of the next k-tile to ask for land, and which stage that is
+    unsigned ldsA = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+    unsigned ldsB = __builtin_amdgcn_readfirstlane(lds0 + NSA * SA + wave * 1024);
+    int slotA = 0, slotB = 0;
+    // LDS addresses of this lane's operand pieces in the stage in use, per k-step of 16, and which stage that is
     unsigned ra[4], rb[4];
+    int curA = 0, curB = 0;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
         const int col = ((kk * 2 + g) ^ ((lrow >> 1) & 7)) * 16;
         ra[kk] = lds0 + (wm + lrow) * 128 + col;
-        rb[kk] = lds0 + (BM + wn + lrow) * 128 + col;
+        rb[kk] = lds0 + NSA * SA + (wn + lrow) * 128 + col;
     }
     i32x4 fa[2][TJ], fb[2][TI];
 
-    auto load = [&](auto q_) {
+    auto loadA = [&](auto q_) {
         constexpr int q = decltype(q_)::value;
-        quad_load<q * 4096>(ldsw, off[q], q < LA ? baseA : baseW);
+        quad_load<q * 4096>(ldsA, offA[q], baseA);
     };
-    auto next_tile = [&]() {                                          // the pointers go on to the k-tile after
+    auto loadB = [&](auto q_) {
+        constexpr int q = decltype(q_)::value;
+        quad_load<q * 4096>(ldsB, offB[q], baseW);
+    };
+    // the x-th early load (A's first where both operands are early), the x-th late load
+    auto early = [&](auto x_) {
+        constexpr int x = decltype(x_)::value;
+        if constexpr (EARLY_A && x < LA) loadA(x_);
+        else loadB(std::integral_constant<int, x - (EARLY_A ? LA : 0)>{});
+    };
+    auto late = [&](auto x_) {
+        constexpr int x = decltype(x_)::value;
+        if constexpr (!EARLY_A && x < LA) loadA(x_);
+        else loadB(std::integral_constant<int, x - (!EARLY_A ? LA : 0)>{});
+    };
+    auto next_tile = [&]() {                       // the pointers and the stages to load go on by a k-tile
         baseA += 128;
         baseW += (knext & 1) ? hopW : 128;
         ++knext;
+        ldsA += slotA == NSA - 1 ? (unsigned)(-(NSA - 1) * SA) : (unsigned)SA;
+        slotA = slotA == NSA - 1 ? 0 : slotA + 1;
+        ldsB += slotB == NSB - 1 ? (unsigned)(-(NSB - 1) * SB) : (unsigned)SB;
+        slotB = slotB == NSB - 1 ? 0 : slotB + 1;
     };
-    // One k-step of 16 from operand set `use`: NM matrix instructions, and between them the LDS reads
-    // of set `use ^ 1` (k-step rk of the stage that ra/rb point into) and, with LD, the L direct loads.
-    auto substep = [&](auto use_, auto rd_, auto rk_, auto ld_) {
+    // One k-step of 16 from operand set `use`: NM matrix instructions, and between them the LDS reads of set
+    // `use ^ 1` (k-step rk of the stage that ra/rb point into) and the direct loads [E0, E1) of the early
+    // ones or [L0, L1) of the late ones, evenly.
+    auto substep = [&](auto use_, auto rd_, auto rk_, auto e0_, auto e1_, auto l0_, auto l1_) {
         constexpr int use = decltype(use_)::value, rk = decltype(rk_)::value;
-        constexpr bool RD = decltype(rd_)::value, LD = decltype(ld_)::value;
+        constexpr bool RD = decltype(rd_)::value;
+        constexpr int E0 = decltype(e0_)::value, E1 = decltype(e1_)::value, L0 = decltype(l0_)::value, L1 = decltype(l1_)::value;
         static_for<0, NM>([&](auto n_) {
             constexpr int n = decltype(n_)::value;
             // block (i, j): weight rows i (the instruction's first operand, so the result's rows), activation rows j
@@ -632,7 +663,8 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
             quad_mfma(acc[i][j], fb[use][i], fa[use][j]);
             if constexpr (RD && n < TJ) quad_read<n * 4096>(fa[use ^ 1][n], ra[rk]);
             if constexpr (RD && n >= TJ && n < TJ + TI) quad_read<(n - TJ) * 4096>(fb[use ^ 1][n - TJ], rb[rk]);
-            if constexpr (LD) static_for<n * L / NM, (n + 1) * L / NM>(load);
+            static_for<E0 + n * (E1 - E0) / NM, E0 + (n + 1) * (E1 - E0) / NM>(early);
+            static_for<L0 + n * (L1 - L0) / NM, L0 + (n + 1) * (L1 - L0) / NM>(late);
         });
         if constexpr (RD) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
@@ -642,48 +674,50 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
-    // One k-tile from the stage in use.  Not LAST: before its last k-step every wave waits for its own
-    // loads of the next k-tile (those of the NS - 2 after that may be on their way) and for the others at
-    // a barrier, which also says that all have read this stage; then it asks for the k-tile NS on into
-    // this stage (LOADS) while it reads the next one's first operands from the next stage.
+    // One k-tile from the stages in use.  Not LAST: before its last k-step every wave waits for its own
+    // loads of the next k-tile (the early ones of the one after may be on their way) and for the others at
+    // a barrier, which also says that all have read these stages; then it reads the next k-tile's first
+    // operands.  LOADS: it asks for the k-tile two on, the early loads before the barrier, the late ones after.
     auto step = [&](auto loads_, auto last_) {
         constexpr bool LOADS = decltype(loads_)::value, LAST = decltype(last_)::value;
-        substep(I0{}, T{}, I1{}, F{});
-        substep(I1{}, T{}, I2{}, F{});
-        substep(I0{}, T{}, I3{}, F{});
+        constexpr int NE = LOADS ? NEARLY : 0, NL = LOADS ? NLATE : 0;
+        using Z = std::integral_constant<int, 0>;
+        substep(I0{}, T{}, I1{}, Z{}, std::integral_constant<int, NE / 3>{}, Z{}, Z{});
+        substep(I1{}, T{}, I2{}, std::integral_constant<int, NE / 3>{}, std::integral_constant<int, 2 * NE / 3>{}, Z{}, Z{});
+        substep(I0{}, T{}, I3{}, std::integral_constant<int, 2 * NE / 3>{}, std::integral_constant<int, NE>{}, Z{}, Z{});
         if constexpr (LAST) {
-            substep(I1{}, F{}, I0{}, F{});
+            substep(I1{}, F{}, I0{}, Z{}, Z{}, Z{}, Z{});
         } else {
-            quad_wait_loads<LOADS ? (NS - 2) * L : 0>();
+            quad_wait_loads<NE>();
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            const unsigned delta = cur == NS - 1 ? (unsigned)(-(NS - 1) * STAGE) : (unsigned)STAGE;
+            const unsigned da = curA == NSA - 1 ? (unsigned)(-(NSA - 1) * SA) : (unsigned)SA;
+            const unsigned db = curB == NSB - 1 ? (unsigned)(-(NSB - 1) * SB) : (unsigned)SB;
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {                           // reads: the next stage; loads: this one
-                ra[kk] += delta;
-                rb[kk] += delta;
+            for (int kk = 0; kk < 4; ++kk) {                           // reads: the next stages
+                ra[kk] += da;
+                rb[kk] += db;
             }
-            substep(I1{}, T{}, I0{}, std::integral_constant<bool, LOADS>{});
-            ldsw += delta;
-            cur = cur == NS - 1 ? 0 : cur + 1;
+            curA = curA == NSA - 1 ? 0 : curA + 1;
+            curB = curB == NSB - 1 ? 0 : curB + 1;
+            substep(I1{}, T{}, I0{}, Z{}, Z{}, Z{}, std::integral_constant<int, NL>{});
             if constexpr (LOADS) next_tile();
         }
     };
 
     int nk = K / DMA_BK - kt0;                                         // k-tiles of this run
     if (nk > kt_per_part) nk = kt_per_part;
-    static_for<0, NS>([&](auto s_) {                                   // the first NS k-tiles, one to a stage
-        constexpr int sg = decltype(s_)::value;
-        if (sg < nk) {
-            static_for<0, L>([&](auto q_) {
-                constexpr int q = decltype(q_)::value;
-                quad_load<sg * STAGE + q * 4096>(ldsw, off[q], q < LA ? baseA : baseW);
-            });
-            next_tile();
-        }
-    });
-    if (nk >= NS) quad_wait_loads<(NS - 1) * L>();
-    else quad_wait_loads<0>();
+    static_for<0, LA>(loadA);                                          // the first two k-tiles
+    static_for<0, LB>(loadB);
+    next_tile();
+    if (nk > 1) {
+        static_for<0, LA>(loadA);
+        static_for<0, LB>(loadB);
+        next_tile();
+        quad_wait_loads<LA + LB>();
+    } else {
+        quad_wait_loads<0>();
+    }
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     static_for<0, TJ>([&](auto n_) { quad_read<decltype(n_)::value * 4096>(fa[0][decltype(n_)::value], ra[0]); });
@@ -693,7 +727,7 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
     // its statement, and a matrix instruction must not read a register in the states right after its write.
     static_for<0, NM>([&](auto n_) { quad_touch(acc[decltype(n_)::value / TJ][decltype(n_)::value % TJ]); });
     int t = 0;
-    for (; t + NS < nk; ++t) step(T{}, F{});
+    for (; t + 2 < nk; ++t) step(T{}, F{});
     for (; t + 1 < nk; ++t) step(F{}, F{});
     step(F{}, T{});
     // the last matrix instructions' results are not in their registers yet; the epilogue's reads of an
@@ -715,7 +749,16 @@ static bool quad_takes(const void* C, int M, int N, int K, size_t lda, size_t ld
 // parts > 1: the k-tiles are cut into runs of an even number of k-tiles, every (tile, run) workgroup writes
 // its float sums to a matrix of its own in `scratch`, and gemm_split_sum_kernel adds the runs in run order
 // and applies the epilogue.
-template <int BM, int BN, int NS>
+#ifndef QUAD12
+#define QUAD12 2, 3
+#endif
+#ifndef QUAD13
+#define QUAD13 3, 3
+#endif
+#ifndef QUAD14
+#define QUAD14 2, 3
+#endif
+template <int BM, int BN, int NSA, int NSB>
 static int launch_tile_quad(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                             int mode, hipStream_t s, int wl, int parts = 1, float* scratch = nullptr) {
     const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
@@ -728,31 +771,34 @@ static int launch_tile_quad(const bf16* A, const bf16* W, void* C, int M, int N,
         kpp += kpp & 1;
         parts = (nk + kpp - 1) / kpp;                                 // no empty run
         dim3 grid((unsigned)total, (unsigned)parts);
-        gemm_tile_quad_kernel<BM, BN, NS, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp,
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp,
                                                                         (size_t)M * N, wl);
         int rc = br_check_launch();
         if (rc != BR_OK) return rc;
         return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
     }
     if (mode == OUT_BF16)
-        gemm_tile_quad_kernel<BM, BN, NS, OUT_BF16><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_BF16><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else if (mode == OUT_F32)
-        gemm_tile_quad_kernel<BM, BN, NS, OUT_F32><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_F32><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else if (mode == OUT_F32_ACC)
-        gemm_tile_quad_kernel<BM, BN, NS, OUT_F32_ACC><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_F32_ACC><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else
-        gemm_tile_quad_kernel<BM, BN, NS, OUT_SWIGLU><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_SWIGLU><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     return br_check_launch();
 }
 
-// Which quad tile (12: 256x256, 13: 128x256 with three stages, 14: 256x192) and how many runs of k-tiles: the
-// least time by a count in microseconds: rounds of workgroups over the chip times k-tiles times what a k-tile
-// takes (measured: 1.62, 0.93 and 1.30 us with every compute unit at work, 1.30, 0.83 and 1.12 with few),
-// plus what a launch costs besides and, when split, the second launch and the traffic of the partial sums.
-static void choose_quad(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* kernel, int* parts) {
+// Which quad tile (12: 256x256, 13: 128x256, 14: 256x192) and how many runs of k-tiles: the least time by a
+// count in microseconds.  A k-tile takes 1.50, 0.85 and 1.20 us with every compute unit at work and 1.08,
+// 0.80 and 0.92 us with few (measured; in between, the cube of the share at work fits: at half the chip
+// the tiles hardly feel each other yet); whole rounds of workgroups over the chip, then the rest of them,
+// which after whole rounds take nearly what a whole round takes (2,048 x 28,672 by 896 tiles of 256x256,
+// three and a half rounds: 390 us, the half round 1.41 us a k-tile); plus what a launch costs besides and, when split along k, the second launch and the traffic of the partial
+// sums.  Returns the count.
+static const double QUAD_FULL[3] = {1.50, 0.85, 1.20}, QUAD_FEW[3] = {1.08, 0.80, 0.92};
+static double choose_quad(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* kernel, int* parts) {
     const int nk = K / DMA_BK;
     static const int bm[3] = {256, 128, 256}, bn[3] = {256, 256, 192};
-    static const double full[3] = {1.62, 0.93, 1.30}, few[3] = {1.30, 0.83, 1.12};
     double best = 1e30;
     *kernel = 13;
     *parts = 1;
@@ -762,15 +808,40 @@ static void choose_quad(int M, int N, int K, int mode, int cus, size_t scratch_b
             if (p > 1 && (p * 4 > nk || N % 4 != 0 || (size_t)p * M * N * sizeof(float) > scratch_bytes)) break;
             int kpp = (nk + p - 1) / p;
             kpp += kpp & 1;
-            const long long units = tiles * p, rounds = (units + cus - 1) / cus;
-            const double per = units >= cus ? full[k] : few[k] + (full[k] - few[k]) * (double)units / cus;
-            double t = (double)rounds * kpp * per + (mode == OUT_BF16 ? 8.0 : 12.0);
+            const long long units = tiles * p, whole = units / cus;
+            const double share = (double)(units % cus) / cus;
+            const double rest = units % cus == 0 ? 0.0
+                                : whole        ? QUAD_FULL[k] * (0.9 + 0.1 * share)
+                                               : QUAD_FEW[k] + (QUAD_FULL[k] - QUAD_FEW[k]) * share * share * share;
+            double t = kpp * ((double)whole * QUAD_FULL[k] + rest) + (mode == OUT_BF16 ? 8.0 : 12.0);
             if (p > 1) t += 5.0 + (double)p * M * N * 8.0 / 4e6;
             if (t < best - 1e-9) { best = t; *kernel = 12 + k; *parts = p; }
         }
     }
+    return best;
 }
 
+// Weight rows that the 256x256 tile covers in whole rounds of workgroups over the chip, where the count says that
+// these rounds and the best tile for the rest (`kernel`, `parts`, chosen over N - n1 weight rows) take less than
+// the best single tile over all rows (`single`); 0 where not.  n1 is a multiple of 256.
+static int quad_whole_rounds(int M, int N, int K, int mode, int cus, size_t scratch_bytes, double single, int* kernel,
+                             int* parts) {
+    const int tm = (M + 255) / 256, nk = K / DMA_BK;
+    const int cols = cus / tm;                                        // tile columns of one round
+    if (cols < 1) return 0;
+    const long long rounds = (long long)(N / 256) / cols, n1 = rounds * cols * 256;
+    if (rounds < 1 || n1 >= N || (mode == OUT_SWIGLU && (N - n1) % 16 != 0)) return 0;
+    const long long used = (long long)tm * cols;                      // workgroups of such a round
+    const double share = (double)used / cus;
+    const double per = used == cus ? QUAD_FULL[0] : QUAD_FEW[0] + (QUAD_FULL[0] - QUAD_FEW[0]) * share * share * share;
+    int k2, p2;
+    const double t = (double)rounds * nk * per + (mode == OUT_BF16 ? 8.0 : 12.0) +
+                     choose_quad(M, (int)(N - n1), K, mode, cus, scratch_bytes, &k2, &p2);
+    if (t >= 0.97 * single) return 0;
+    *kernel = k2;
+    *parts = p2;
+    return (int)n1;
+}
 
 // parts > 1: the k-tiles are cut into `parts` runs, every (tile, run) workgroup writes its
 // float sums to a matrix of its own in `scratch`, and gemm_split_sum_kernel adds the runs in
@@ -1812,7 +1883,25 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
         // allow.  (Up to 128 rows the tiles of eight waves below stream the weights faster: 7B shapes at 128
         // rows, gate/up 59 against 69 us, the 32,768-row head 71 against 85, down 39 against 45.)
         const int cus = br_device_cus();
-        if (cus > 0) choose_quad(M, N, K, mode, cus, (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0, &kernel, &parts);
+        const size_t room = (scratch && (uintptr_t)scratch % 16 == 0) ? scratch_bytes : 0;
+        if (cus > 0) {
+            const double single = choose_quad(M, N, K, mode, cus, room, &kernel, &parts);
+            int k2, p2;
+            const int n1 = quad_whole_rounds(M, N, K, mode, cus, room, single, &k2, &p2);
+            if (n1 > 0) {
+                // whole rounds of the 256x256 tile over the first n1 weight rows, then the rest; n1 rows on
+                // is the same number of elements in either weight layout (n1 is a multiple of 16)
+                int rc = launch_tile_quad<256, 256, QUAD12>(A, W, C, M, n1, K, lda, ldc, mode, s, wl);
+                if (rc != BR_OK) return rc;
+                const bf16* W2 = W + (size_t)n1 * K;
+                void* C2 = mode == OUT_SWIGLU ? (void*)((bf16*)C + n1 / 2)
+                           : mode == OUT_BF16 ? (void*)((bf16*)C + n1) : (void*)((float*)C + n1);
+                const int N2 = N - n1;
+                if (k2 == 12) return launch_tile_quad<256, 256, QUAD12>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
+                if (k2 == 13) return launch_tile_quad<128, 256, QUAD13>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
+                return launch_tile_quad<256, 192, QUAD14>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
+            }
+        }
     }
     if (chosen && (kernel == 5 || kernel == 6)) {
         const int cus = br_device_cus();
@@ -1849,9 +1938,9 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
             return BR_BAD_ARG;
         parts = forced_parts;
     }
-    if (kernel == 12) return launch_tile_quad<256, 256, 2>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
-    if (kernel == 13) return launch_tile_quad<128, 256, 3>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
-    if (kernel == 14) return launch_tile_quad<256, 192, 2>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
+    if (kernel == 12) return launch_tile_quad<256, 256, QUAD12>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
+    if (kernel == 13) return launch_tile_quad<128, 256, QUAD13>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
+    if (kernel == 14) return launch_tile_quad<256, 192, QUAD14>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
     if (kernel == 10) return launch_tile_dma<256, 192, 4, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
     if (kernel == 11) {
         gemm_tile_dma_kernel<256, 256, 2, 4, 2, OUT_SWIGLU><<<(unsigned)(((M + 255) / 256) * ((N + 255) / 256)), 512, 0, s>>>(
@@ -1892,11 +1981,26 @@ extern "C" int br_gemm_bf16(const void* A, const void* W, void* C, int M, int N,
     return br_gemm_bf16_ex(A, W, C, M, N, K, lda, ldc, mode, 0, nullptr, 0, WL_ROWS, s);
 }
 
-// what br_gemm_bf16_ex would pick for more than 64 rows (tests and benchmarks print it)
-extern "C" int br_gemm_bf16_tile_choice(int M, int N, int K, size_t scratch_bytes, int* kernel, int* parts) {
+// What br_gemm_bf16_ex picks for a product of more than 64 rows with K in steps of 64, aligned rows and a
+// contiguous, aligned output (tests and benchmarks ask): the kernel and its runs along k; and, where the product is
+// cut along its weight rows, `n1` > 0 rows by the 256x256 tile first and `kernel`, `parts` for the rest.
+extern "C" int br_gemm_bf16_tile_choice(int M, int N, int K, int mode, size_t scratch_bytes, int* kernel, int* parts,
+                                        int* n1) {
     const int cus = br_device_cus();
     if (!cus) return BR_LAUNCH_FAILED;
-    choose_tile(M, N, K, OUT_BF16, cus, scratch_bytes, kernel, parts);
+    *n1 = 0;
+    if (M > 128 && quad_takes(nullptr, M, N, K, (size_t)K, (size_t)(mode == OUT_SWIGLU ? N / 2 : N))) {
+        const double single = choose_quad(M, N, K, mode, cus, scratch_bytes, kernel, parts);
+        int k2, p2;
+        const int rows = quad_whole_rounds(M, N, K, mode, cus, scratch_bytes, single, &k2, &p2);
+        if (rows > 0) {
+            *n1 = rows;
+            *kernel = k2;
+            *parts = p2;
+        }
+        return BR_OK;
+    }
+    choose_tile(M, N, K, mode, cus, scratch_bytes, kernel, parts);
     return BR_OK;
 }
 

@@ -353,6 +353,17 @@ def gemm_stream_takes(M: int, K: int) -> bool:
     return (0 < M <= 16 and K % 128 == 0 and K >= 1024) or (16 < M <= 64 and K % 128 == 0 and K >= 256)
 
 
+def gemm_tile_choice(M: int, N: int, K: int, mode: int = 0, scratch_floats: int = 0):
+    """What a bf16 product of more than 64 rows runs on when its K is a multiple of 64 and its rows and output
+    are aligned: (kernel, runs along k, n1).  n1 > 0: the first n1 weight rows go to the 256x256 tile of one
+    wave per SIMD in whole rounds over the chip, the rest to `kernel`.  mode: 0 bf16 out, 1 float out,
+    2 float out added to, 3 SwiGLU."""
+    f = _fn("gemm_bf16", "br_gemm_bf16_tile_choice", [c_int, c_int, c_int, c_int, c_size_t, _P, _P, _P])
+    k, p, n1 = c_int(0), c_int(0), c_int(0)
+    _check(f(M, N, K, mode, scratch_floats * 4, ctypes.byref(k), ctypes.byref(p), ctypes.byref(n1)), "gemm_tile_choice")
+    return k.value, p.value, n1.value
+
+
 def gemm_wide_parts(M: int, N: int, K: int, scratch_floats: int, accumulate: bool = True) -> int:
     """Into how many runs along k a bf16 product of 17 to 64 rows is cut when it is given that
     much scratch (0: the wide streaming product does not take it)."""

@@ -373,6 +373,41 @@ def test_gemm_tiles_of_one_wave_per_simd(M, N, Kd, kernel, parts, blocked):
     assert (chosen.double() - want).abs().max() < 1e-4 * want.abs().max()
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_gemm_cut_along_weight_rows_into_whole_rounds_and_a_rest(mode):
+    """2,048 x 28,672 x 4,096 is three and a half rounds of 256x256 tiles over the chip: the product goes as
+    three whole rounds over the first weight rows and another tile over the rest.  Every output mode: the
+    same sums as the one tile over all rows, and right against double sums at sampled rows."""
+    M, N, Kd = 2048, 28672, 4096
+    kernel, parts, n1 = K.gemm_tile_choice(M, N, Kd, mode, K.GEMM_SCRATCH_FLOATS)
+    assert 0 < n1 < N and n1 % 256 == 0 and kernel in (12, 13, 14), (kernel, parts, n1)
+    a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
+    w = rnd(N, Kd, seed=2, scale=0.05, dtype=torch.bfloat16)
+    scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
+    rows = torch.tensor([0, 1, 255, 256, 1023, 1500, 2047], device=DEV)
+    want = a[rows].double() @ w.double().T
+    def run(kern):
+        if mode == 3:
+            out = torch.empty(M, N // 2, device=DEV, dtype=torch.bfloat16)
+            K.gemm_swiglu(a, w, out, kernel=kern, scratch=scratch)
+        elif mode == 0:
+            out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+            K.gemm(a, w, out, kernel=kern, scratch=scratch)
+        else:
+            out = torch.full((M, N), 0.25, device=DEV)
+            K.gemm(a, w, out, accumulate=(mode == 2), kernel=kern, scratch=scratch)
+        return out
+    chosen, one = run(0), run(12)
+    assert torch.equal(chosen, one)
+    if mode == 3:
+        g = want.view(len(rows), N // 16, 2, 8)
+        want = (g[:, :, 0] / (1 + torch.exp(-g[:, :, 0])) * g[:, :, 1]).reshape(len(rows), N // 2)
+    elif mode == 2:
+        want = want + 0.25
+    tol = 1e-4 if mode in (1, 2) else 1e-2
+    assert (chosen[rows].double() - want).abs().max() < tol * want.abs().max()
+
+
 def test_gemm_reference_vectors():
     # tests/wmma_gemm_test.rs:27-69,72-114: sin/cos ramps times 0.5 / 0.3, tol 1e-3
     for M, N, Kd in ((32, 32, 64), (256, 256, 1024)):
