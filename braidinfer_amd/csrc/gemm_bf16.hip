@@ -452,8 +452,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
 // in order, but it neither knows their latencies nor that they are matrix instructions: every wait is
 // placed by hand, and so are the idle states that the hardware wants between a register's write and
 // a matrix instruction's read of it (and the reverse).
-// NS stages of 64 k (the layout and swizzle of gemm_tile_dma).  One barrier per k-tile, before its
-// last k-step of 16: by then every wave has read the stage, which is then asked for the k-tile NS on.
+// Each operand has a ring of two or three stages of 64 k (the layout and swizzle of gemm_tile_dma).  One
+// barrier per k-tile, before its last k-step of 16: by then every wave has read the stages in use.  An
+// operand with two stages is asked for after that barrier, into the stage just read; one with three
+// during the k-steps before it, into the stage that the barrier before freed: a compute unit's path into
+// LDS takes one 1 KB load per 16 cycles, so a k-tile's loads are spread over it, not bunched (bunched,
+// the waves wait at their load instructions with the matrix cores idle behind them).
 // The blocks hold the product transposed (weight rows are the instruction's first operand), which
 // gives every lane four neighbouring columns of one output row: 16-byte accesses in the epilogue, and
 // the up value of a gate column in the same lane.
@@ -1830,9 +1834,11 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
 // rows), 8 = stream wide (16 < M <= 64, K a multiple of 128), 9 = direct-to-LDS tile 64x128
-// (M <= 64), 10 = direct-to-LDS tile 256x192, 11 = the same 256x256 (SwiGLU epilogue only); tests force one.  (A 256x256 tile of 8 waves was tried: it runs out of registers in
-// three of the four epilogues and was no faster in the fourth.)
-// `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 9).
+// (M <= 64), 10 = direct-to-LDS tile 256x192, 11 = the same 256x256 (SwiGLU epilogue only), 12..14 = the tiles of
+// four waves, one to a SIMD: 256x256, 128x256, 256x192 (K a multiple of 64, aligned rows, output rows in steps
+// of 16 bytes; plus 16 p: with p runs along k); tests force one.  (A 256x256 tile of 8 waves for every epilogue
+// was tried: it runs out of registers in three of the four and was no faster in the fourth.)
+// `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 14).
 // `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
 // weight rows be split along k (see gemm_split_sum_kernel); BR_GEMM_SCRATCH_BYTES always suffices.
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
