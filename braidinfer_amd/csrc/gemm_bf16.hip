@@ -443,7 +443,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
 }
 
 // ------------------------------------------------------------ gemm_tile_quad -------
-// A BM x BN tile by four waves (2 x 2), one to a SIMD, each summing a quarter of it in the matrix-core
+// A BM x BN tile by four waves (2 x 2, or 4 x 1 for the 256x224 tile), one to a SIMD, each summing a quarter of it in the matrix-core
 // registers (256x256: 16 blocks of 32x32, all 256 of them), with the operands of one k-step of 16 in
 // vector registers, twice (the set in use and the set being read from LDS).  Per matrix instruction
 // half the LDS operand bytes of the 64x64 wave tiles above.  With one wave per SIMD nothing fills a gap
@@ -541,13 +541,14 @@ __device__ __forceinline__ void quad_epilogue(f32x16 (&acc)[TI][TJ], void* __res
     }
 }
 
-template <int BM, int BN, int NSA, int NSB, int MODE>
+template <int BM, int BN, int NSA, int NSB, int WVM, int MODE>
 __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                               void* __restrict__ C_, int M, int N, int K, size_t lda,
                                                               size_t ldc, int tiles_m, int tiles_n, int kt_per_part,
                                                               size_t part_stride, int wl) {
     constexpr int SA = BM * 128, SB = BN * 128;          // bytes of a stage of activation rows, of weight rows
-    constexpr int TI = BN / 64, TJ = BM / 64;            // blocks of a wave: weight rows, activation rows
+    constexpr int WVN = 4 / WVM;                         // the four waves: WVM along the activation rows x WVN
+    constexpr int TI = BN / WVN / 32, TJ = BM / WVM / 32; // blocks of a wave: weight rows, activation rows
     constexpr int NM = TI * TJ;                          // matrix instructions per k-step of 16
     constexpr int LA = BM / 32, LB = BN / 32;            // wave-loads per wave and stage
     // An operand with three stages is asked for during the first three k-steps of 16 of a k-tile, into the
@@ -555,7 +556,8 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
     // the barrier, into the stage just read.  Either way k-tile t asks for k-tile t + 2.
     constexpr bool EARLY_A = NSA == 3, EARLY_B = NSB == 3;
     constexpr int NEARLY = (EARLY_A ? LA : 0) + (EARLY_B ? LB : 0), NLATE = LA + LB - NEARLY;
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && NSA * SA + NSB * SB <= 160 * 1024, "tile");
+    static_assert((WVM == 2 || WVM == 4) && BM % (32 * WVM) == 0 && BN % (32 * WVN) == 0 && BM % 32 == 0 && BN % 32 == 0 &&
+                      NSA * SA + NSB * SB <= 160 * 1024 && TI * TJ * 16 <= 256, "tile");
     static_assert((NSA == 2 || NSA == 3) && (NSB == 2 || NSB == 3), "two or three stages an operand");
     static_assert(TI + TJ <= NM && NLATE <= 2 * NM, "schedule");
     __shared__ __attribute__((aligned(1024))) unsigned char st[NSA * SA + NSB * SB];
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(256) void gemm_tile_quad_kernel(const bf16* __restr
     const int tile_n = grp * 8 + in % gn, tile_m = in / gn;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+    const int wm = (wave / WVN) * (BM / WVM), wn = (wave % WVN) * (BN / WVN);
     const int lrow = lane & 31, g = lane >> 5;
 
     f32x16 acc[TI][TJ];
@@ -762,7 +764,7 @@ static bool quad_takes(const void* C, int M, int N, int K, size_t lda, size_t ld
 #ifndef QUAD14
 #define QUAD14 2, 3
 #endif
-template <int BM, int BN, int NSA, int NSB>
+template <int BM, int BN, int NSA, int NSB, int WVM = 2>
 static int launch_tile_quad(const bf16* A, const bf16* W, void* C, int M, int N, int K, size_t lda, size_t ldc,
                             int mode, hipStream_t s, int wl, int parts = 1, float* scratch = nullptr) {
     const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
@@ -775,38 +777,39 @@ static int launch_tile_quad(const bf16* A, const bf16* W, void* C, int M, int N,
         kpp += kpp & 1;
         parts = (nk + kpp - 1) / kpp;                                 // no empty run
         dim3 grid((unsigned)total, (unsigned)parts);
-        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp,
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, WVM, OUT_F32><<<grid, 256, 0, s>>>(A, W, scratch, M, N, K, lda, (size_t)N, tm, tn, kpp,
                                                                         (size_t)M * N, wl);
         int rc = br_check_launch();
         if (rc != BR_OK) return rc;
         return launch_split_sum(scratch, parts, C, M, N, ldc, mode, s);
     }
     if (mode == OUT_BF16)
-        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_BF16><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, WVM, OUT_BF16><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else if (mode == OUT_F32)
-        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_F32><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, WVM, OUT_F32><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else if (mode == OUT_F32_ACC)
-        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_F32_ACC><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, WVM, OUT_F32_ACC><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     else
-        gemm_tile_quad_kernel<BM, BN, NSA, NSB, OUT_SWIGLU><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
+        gemm_tile_quad_kernel<BM, BN, NSA, NSB, WVM, OUT_SWIGLU><<<(unsigned)total, 256, 0, s>>>(A, W, C, M, N, K, lda, ldc, tm, tn, nk, 0, wl);
     return br_check_launch();
 }
 
-// Which quad tile (12: 256x256, 13: 128x256, 14: 256x192) and how many runs of k-tiles: the least time by a
-// count in microseconds.  A k-tile takes 1.50, 0.85 and 1.20 us with every compute unit at work and 1.08,
-// 0.80 and 0.92 us with few (measured; in between, the cube of the share at work fits: at half the chip
+// Which quad tile (12: 256x256, 13: 128x256, 14: 256x192, 15: 256x224, whose 128 tile columns over 28,672
+// weight rows make whole rounds where 112 of 256 do not) and how many runs of k-tiles: the least time by a
+// count in microseconds.  A k-tile takes 1.50, 0.85, 1.20 and 1.39 us with every compute unit at work and 1.08,
+// 0.80, 0.92 and 1.00 us with few (measured; in between, the cube of the share at work fits: at half the chip
 // the tiles hardly feel each other yet); whole rounds of workgroups over the chip, then the rest of them,
 // which after whole rounds take nearly what a whole round takes (2,048 x 28,672 by 896 tiles of 256x256,
 // three and a half rounds: 390 us, the half round 1.41 us a k-tile); plus what a launch costs besides and, when split along k, the second launch and the traffic of the partial
 // sums.  Returns the count.
-static const double QUAD_FULL[3] = {1.50, 0.85, 1.20}, QUAD_FEW[3] = {1.08, 0.80, 0.92};
+static const double QUAD_FULL[4] = {1.50, 0.85, 1.20, 1.39}, QUAD_FEW[4] = {1.08, 0.80, 0.92, 1.00};
 static double choose_quad(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* kernel, int* parts) {
     const int nk = K / DMA_BK;
-    static const int bm[3] = {256, 128, 256}, bn[3] = {256, 256, 192};
+    static const int bm[4] = {256, 128, 256, 256}, bn[4] = {256, 256, 192, 224};
     double best = 1e30;
     *kernel = 13;
     *parts = 1;
-    for (int k = 0; k < 3; ++k) {
+    for (int k = 0; k < 4; ++k) {
         const long long tiles = (long long)((M + bm[k] - 1) / bm[k]) * ((N + bn[k] - 1) / bn[k]);
         for (int p = 1; p <= 16; p *= 2) {
             if (p > 1 && (p * 4 > nk || N % 4 != 0 || (size_t)p * M * N * sizeof(float) > scratch_bytes)) break;
@@ -1834,11 +1837,11 @@ static int launch_stream_wide(const bf16* A, const bf16* W, void* C, int M, int 
 // 3 = skinny (M <= 64), 4..6 = direct-to-LDS tiles 256x128, 128x256, 128x128 (K a multiple
 // of 64, aligned rows), 7 = stream (M <= 16, K a multiple of 128 and at least 1024, aligned
 // rows), 8 = stream wide (16 < M <= 64, K a multiple of 128), 9 = direct-to-LDS tile 64x128
-// (M <= 64), 10 = direct-to-LDS tile 256x192, 11 = the same 256x256 (SwiGLU epilogue only), 12..14 = the tiles of
-// four waves, one to a SIMD: 256x256, 128x256, 256x192 (K a multiple of 64, aligned rows, output rows in steps
+// (M <= 64), 10 = direct-to-LDS tile 256x192, 11 = the same 256x256 (SwiGLU epilogue only), 12..15 = the tiles of
+// four waves, one to a SIMD: 256x256, 128x256, 256x192, 256x224 (K a multiple of 64, aligned rows, output rows in steps
 // of 16 bytes; plus 16 p: with p runs along k); tests force one.  (A 256x256 tile of 8 waves for every epilogue
 // was tried: it runs out of registers in three of the four and was no faster in the fourth.)
-// `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 14).
+// `wl`: the layout of W (see WL_BLOCKED; K in steps of 128 then, kernels 4 to 15).
 // `scratch` (float, `scratch_bytes`; may be null) lets a product of 16 < M <= 64 rows with few
 // weight rows be split along k (see gemm_split_sum_kernel); BR_GEMM_SCRATCH_BYTES always suffices.
 extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, int N, int K, size_t lda,
@@ -1860,7 +1863,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel >= 4 && kernel <= 6 && !dma_ok) return BR_BAD_ARG;
     const bool wide_ok = aligned && M > 16 && M <= 64 && K % 128 == 0 && K >= 256 &&
                          (!scratch || (uintptr_t)scratch % 16 == 0);
-    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 14 || kernel < 0 || (kernel >= 10 && !dma_ok) ||
+    if ((kernel == 7 && !stream_ok) || (kernel == 8 && !wide_ok) || kernel > 15 || kernel < 0 || (kernel >= 10 && !dma_ok) ||
         (kernel == 11 && mode != OUT_SWIGLU) ||
         (kernel == 9 && (!dma_ok || M > 64)))
         return BR_BAD_ARG;
@@ -1905,6 +1908,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
                 const int N2 = N - n1;
                 if (k2 == 12) return launch_tile_quad<256, 256, QUAD12>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
                 if (k2 == 13) return launch_tile_quad<128, 256, QUAD13>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
+                if (k2 == 15) return launch_tile_quad<256, 224, 2, 3, 4>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
                 return launch_tile_quad<256, 192, QUAD14>(A, W2, C2, M, N2, K, lda, ldc, mode, s, wl, p2, (float*)scratch);
             }
         }
@@ -1947,6 +1951,7 @@ extern "C" int br_gemm_bf16_ex(const void* A_, const void* W_, void* C, int M, i
     if (kernel == 12) return launch_tile_quad<256, 256, QUAD12>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
     if (kernel == 13) return launch_tile_quad<128, 256, QUAD13>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
     if (kernel == 14) return launch_tile_quad<256, 192, QUAD14>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
+    if (kernel == 15) return launch_tile_quad<256, 224, 2, 3, 4>(A, W, C, M, N, K, lda, ldc, mode, s, wl, parts, (float*)scratch);
     if (kernel == 10) return launch_tile_dma<256, 192, 4, 2, 2>(A, W, C, M, N, K, lda, ldc, mode, s, 1, nullptr, wl);
     if (kernel == 11) {
         gemm_tile_dma_kernel<256, 256, 2, 4, 2, OUT_SWIGLU><<<(unsigned)(((M + 255) / 256) * ((N + 255) / 256)), 512, 0, s>>>(

@@ -287,9 +287,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     loaded straight into LDS, K in steps of 64; 7: streaming by workgroups that stay, M <= 16
     and K in steps of 128 from 1024; 8: the same for 17 to 64 rows, K in steps of 128; 5 or 6 plus
     16 p: that tile with p runs along k, for measurements; 9: a 64x128 tile loaded straight into
-    LDS, M <= 64; 10: a 256x192 tile loaded straight into LDS; 12, 13, 14: 256x256, 128x256 and 256x192
-    tiles of four waves, one to a SIMD, K in steps of 64 and output rows in steps of 16 bytes, plus 16 p
-    for p runs along k); 0 chooses by shape.  A weight from `block_weight` is taken by kernels 4 to 14.
+    LDS, M <= 64; 10: a 256x192 tile loaded straight into LDS; 12 to 15: 256x256, 128x256, 256x192 and
+    256x224 tiles of four waves, one to a SIMD, K in steps of 64 and output rows in steps of 16 bytes, plus
+    16 p for p runs along k); 0 chooses by shape.  A weight from `block_weight` is taken by kernels 4 to 15.
     `scratch` (float32, on the device): with it, a bf16 product of more than 16 rows with too
     few tiles to fill the chip is cut along k into runs that a second kernel sums in a fixed order.
     """

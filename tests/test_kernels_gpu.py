@@ -81,7 +81,7 @@ def _skip_unless_kernel_takes(kernel, M, Kd, N=None):
         pytest.skip("the streaming kernel takes M <= 16 and K in steps of 128 from 1024")
     if kernel == 8 and (M <= 16 or M > 64 or Kd % 128 or Kd < 256):
         pytest.skip("the wide streaming kernel takes 16 < M <= 64 and K in steps of 128 from 256")
-    if 12 <= kernel <= 14 and (Kd % 64 or N is None or N % 4):
+    if 12 <= kernel <= 15 and (Kd % 64 or N is None or N % 4):
         pytest.skip("the tiles of one wave per SIMD take K in steps of 64 and output rows in steps of 16 bytes")
 
 
@@ -107,7 +107,7 @@ def test_gemm_f32_rows_do_not_depend_on_the_batch():
     assert torch.equal(one[0], full[33])
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 13, 14])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 13, 14, 15])
 @pytest.mark.parametrize("M,N,Kd", SHAPES)
 def test_gemm_bf16(M, N, Kd, kernel):
     _skip_unless_kernel_takes(kernel, M, Kd, N)
@@ -321,10 +321,10 @@ def test_gemm_with_blocked_weights(M, N, Kd, kernel):
 
 @pytest.mark.parametrize("blocked", [False, True])
 @pytest.mark.parametrize("parts", [1, 2, 4])
-@pytest.mark.parametrize("kernel", [12, 13, 14])
+@pytest.mark.parametrize("kernel", [12, 13, 14, 15])
 @pytest.mark.parametrize("M,N,Kd", [(130, 516, 1024), (300, 700, 2048), (513, 264, 1152), (65, 1032, 1280), (260, 1500, 1024)])
 def test_gemm_tiles_of_one_wave_per_simd(M, N, Kd, kernel, parts, blocked):
-    """The 256x256, 128x256 and 256x192 tiles of four waves (written-out instruction order, products kept
+    """The 256x256, 128x256, 256x192 and 256x224 tiles of four waves (written-out instruction order, products kept
     transposed in the matrix-core registers): every epilogue, one run or several along k, either weight
     layout, tiles that hang over every edge; a strided output whose width is no multiple of four (the
     elements that no 16-byte store takes); and what they refuse."""
@@ -375,16 +375,16 @@ def test_gemm_tiles_of_one_wave_per_simd(M, N, Kd, kernel, parts, blocked):
 
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_gemm_cut_along_weight_rows_into_whole_rounds_and_a_rest(mode):
-    """2,048 x 28,672 x 4,096 is three and a half rounds of 256x256 tiles over the chip: the product goes as
-    three whole rounds over the first weight rows and another tile over the rest.  Every output mode: the
+    """1,024 x 17,408 x 4,096 is one round of 256x256 tiles over the chip and a sixteenth: the product goes as
+    one whole round over the first 16,384 weight rows and another tile over the rest.  Every output mode: the
     same sums as the one tile over all rows, and right against double sums at sampled rows."""
-    M, N, Kd = 2048, 28672, 4096
+    M, N, Kd = 1024, 17408, 4096
     kernel, parts, n1 = K.gemm_tile_choice(M, N, Kd, mode, K.GEMM_SCRATCH_FLOATS)
-    assert 0 < n1 < N and n1 % 256 == 0 and kernel in (12, 13, 14), (kernel, parts, n1)
+    assert 0 < n1 < N and n1 % 256 == 0 and kernel in (12, 13, 14, 15), (kernel, parts, n1)
     a = rnd(M, Kd, seed=1, scale=0.5, dtype=torch.bfloat16)
     w = rnd(N, Kd, seed=2, scale=0.05, dtype=torch.bfloat16)
     scratch = torch.full((K.GEMM_SCRATCH_FLOATS,), float("nan"), device=DEV)
-    rows = torch.tensor([0, 1, 255, 256, 1023, 1500, 2047], device=DEV)
+    rows = torch.tensor([0, 1, 255, 256, 700, 1023], device=DEV)
     want = a[rows].double() @ w.double().T
     def run(kern):
         if mode == 3:
@@ -398,7 +398,11 @@ def test_gemm_cut_along_weight_rows_into_whole_rounds_and_a_rest(mode):
             K.gemm(a, w, out, accumulate=(mode == 2), kernel=kern, scratch=scratch)
         return out
     chosen, one = run(0), run(12)
-    assert torch.equal(chosen, one)
+    c1 = n1 // 2 if mode == 3 else n1                    # output columns of the first n1 weight rows
+    assert torch.equal(chosen[:, :c1], one[:, :c1])      # the same tile, the same sums
+    # the rest may be cut along k as well: float sums in another order, then the same rounding
+    step = 1e-5 if mode in (1, 2) else 2.0 ** -7
+    assert (chosen[:, c1:].float() - one[:, c1:].float()).abs().max() <= step * one.float().abs().max()
     if mode == 3:
         g = want.view(len(rows), N // 16, 2, 8)
         want = (g[:, :, 0] / (1 + torch.exp(-g[:, :, 0])) * g[:, :, 1]).reshape(len(rows), N // 2)
@@ -808,7 +812,7 @@ def test_attention_kernels_refuse_what_they_do_not_take():
         K.attention_prefill_bf16(q, 48, out, i32([0, 4]), i32([0]), i32([4]), i32([[0]]), cache, 1, 4, 2, 1, 24, 64, None, 1.0)
 
 
-@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("M,I,Kd", [(40, 8264, 256), (64, 328, 1152), (1, 64, 64), (8, 192, 96), (17, 320, 64), (64, 1024, 264), (130, 328, 100), (300, 512, 1032),
                                     (300, 512, 1024), (129, 200, 192), (1, 2056, 1024), (8, 328, 1152), (13, 4400, 1280),
                                     (100, 264, 4096), (260, 520, 2048)])
