@@ -917,7 +917,7 @@ __global__ __launch_bounds__(256) void attn_decode_lds_kernel(
                 gp_ = pg_ + v_off + (size_t)row_ * PAGE + (((lane & 7) ^ ((row_ >> 1) & 7)) * 8);            \
             }                                                                                                \
             const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + ((I) % S) * STAGE + in_ * 1024); \
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_), "v"(gp_) : "m0"); \
         }                                                                                                    \
     } while (0)
 

@@ -286,8 +286,12 @@ __device__ __forceinline__ size_t w_row_base(int n, int K, int wl) {
         _Pragma("unroll") for (int q = 0; q < INSTR; ++q) {                                                    \
             const unsigned lds_ = __builtin_amdgcn_readfirstlane(                                              \
                 (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)(ST)) + dst[q]);          \
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q]) \
-                         : "m0");                                                                              \
+            if (once[q])                                   /* weights that no other row of tiles reads */      \
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_), "v"(src[q]) \
+                             : "m0");                                                                          \
+            else                                                                                               \
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q]) \
+                             : "m0");                                                                          \
             src[q] += (knext & 1) ? hop[q] : DMA_BK;       /* k-tiles are issued in order, (kt) is the next */ \
         }                                                                                                      \
         if (++knext == kwrap) {                            /* on to the run's first k-tile */                  \
@@ -364,6 +368,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
     const bf16* src[INSTR];
     int dst[INSTR];
     int hop[INSTR];                                      // elements from an odd k-tile to the next (even) one
+    bool once[INSTR];                                    // a load of weight rows that are read this once (non-temporal)
     const int kt0 = (int)blockIdx.y * kt_per_part;       // the run's first k-tile
     int nk_run = K / DMA_BK - kt0;                       // k-tiles of this run
     if (nk_run > kt_per_part) nk_run = kt_per_part;
@@ -394,6 +399,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_dma_kernel(
             hop[q] = wl ? WL_BLOCK_ELEMS - DMA_BK : DMA_BK;
         }
         hop[q] = __builtin_amdgcn_readfirstlane(hop[q]);             // the same for the 8 rows of a wave-load
+        once[q] = __builtin_amdgcn_readfirstlane((int)((q * NW + wave) * 8 >= BM && tiles_m == 1)) != 0;
         dst[q] = (q * NW + wave) * 1024;
     }
     const int nk = nk_run;
@@ -1350,7 +1356,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_stream_kernel(const bf16* __rest
                 gp_ = A + (size_t)m_ * lda + (size_t)chunk_ * KC + ((dcol ^ (row_ & 7)) * 8);            \
             }                                                                                            \
             const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + (J) * STAGE + q_ * 1024);    \
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
+            if (q_ < WDMA)                              /* weights pass once: non-temporal */            \
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_), "v"(gp_) : "m0"); \
+            else                                        /* activations are every workgroup's: they stay cached */ \
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(gp_) : "m0"); \
         }                                                                                                \
         if (++is_c == ncw) { is_c = 0; ++is_t; }                                                         \
     } while (0)
@@ -1605,7 +1614,10 @@ __global__ __launch_bounds__(512) void gemm_stream_wide_kernel(const bf16* __res
     do {                                                                                                      \
         _Pragma("unroll") for (int q_ = 0; q_ < NDMA; ++q_) {                                                 \
             const unsigned lds_ = __builtin_amdgcn_readfirstlane(ring_lds + is_off + WIDE_LOAD_INDEX(q_) * 1024); \
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q_]) : "m0"); \
+            if (WIDE_LOAD_INDEX(q_) * 4 < H)                /* weights pass once: non-temporal */             \
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_), "v"(src[q_]) : "m0"); \
+            else                                                                                              \
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_), "v"(src[q_]) : "m0"); \
             src[q_] += WIDE_LOAD_INDEX(q_) * 4 < H ? wstep : 128;                                             \
         }                                                                                                     \
         if (--is_wrap == 0) {                              /* on to the run's first chunk */                  \
