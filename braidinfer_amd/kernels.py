@@ -208,9 +208,9 @@ def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
 
 
 def stream_read(src: torch.Tensor, sums: torch.Tensor) -> None:
-    """Reads all of `src` once (four 16-byte loads in flight per lane) and leaves partial sums
-    of its words in `sums` (float32, at least 32 per compute unit): the read rate of a
-    kernel that only streams."""
+    """Reads all of `src` once (every workgroup a contiguous region of its own, eight non-temporal
+    16-byte loads in flight per lane) and leaves partial sums of its words in `sums` (float32, at
+    least 32 per compute unit): the read rate of a kernel that only streams."""
     _dev("stream_read", src, sums)
     n = src.numel() * src.element_size()
     _req(n % 16 == 0 and sums.dtype == torch.float32, "stream_read: a multiple of 16 bytes, float32 sums")
