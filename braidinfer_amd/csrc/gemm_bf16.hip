@@ -806,8 +806,8 @@ static int launch_tile_quad(const bf16* A, const bf16* W, void* C, int M, int N,
 // 0.80, 0.92 and 1.00 us with few (measured; in between, the cube of the share at work fits: at half the chip
 // the tiles hardly feel each other yet); whole rounds of workgroups over the chip, then the rest of them,
 // which after whole rounds take nearly what a whole round takes (2,048 x 28,672 by 896 tiles of 256x256,
-// three and a half rounds: 390 us, the half round 1.41 us a k-tile); plus what a launch costs besides and, when split along k, the second launch and the traffic of the partial
-// sums.  Returns the count.
+// three and a half rounds: 390 us, the half round 1.41 us a k-tile); plus what a launch costs besides and,
+// when split along k, the second launch and the traffic of the partial sums.  Returns the count.
 static const double QUAD_FULL[4] = {1.50, 0.85, 1.20, 1.39}, QUAD_FEW[4] = {1.08, 0.80, 0.92, 1.00};
 static double choose_quad(int M, int N, int K, int mode, int cus, size_t scratch_bytes, int* kernel, int* parts) {
     const int nk = K / DMA_BK;
