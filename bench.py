@@ -176,6 +176,7 @@ class Shape:
         V, W = self.V, self.W
         rng = np.random.default_rng(seed)
         lens = [int(n) for n in rng.integers(self.prompt_min, self.prompt_max + 1, batch)]
+        lens.sort(reverse=True)       # the generation loop's order within a batch: longest prompts first
         prompts = [[int(t) for t in rng.integers(0, V, n)] for n in lens]
         slots = [eng.alloc_slot() for _ in range(batch)]
         # prompts in chunks of at most 16k tokens a step, to bound the activations

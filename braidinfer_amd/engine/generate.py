@@ -177,6 +177,10 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]],
                 live.append(i)
         if not live:
             continue
+        # Longest prompts first: the single-token attention starts its workgroups in row order, and where
+        # they are more than the chip holds at once, long sequences that start first do not end last
+        # (128 sequences of 128 to 2,048 tokens: 99 against 107 us a layer).
+        live.sort(key=lambda i: -len(prompts[i]))
         slot = {i: engine.alloc_slot() for i in live}
         out = {i: [] for i in live}
         hist = {i: list(prompts[i]) for i in live}

@@ -95,7 +95,7 @@ def test_shorter_sequences_leave_the_batch_and_give_their_slot_back():
     assert res[0].tokens == [41, 42, 43, 44, 45] and res[1].tokens == [48, 49] and res[2].tokens == [12, 13, 14, 15, 16]
     sizes = [len(s[0]) for s in e.steps]
     assert sizes == [3, 3, 3, 2, 2]     # request 1 stops on its third token and leaves before the fourth step
-    assert e.steps[0][1] == [1, 1, 2] and not e.live
+    assert e.steps[0][1] == [2, 1, 1] and not e.live         # a batch's longest prompts come first
 
 
 def test_batches_run_one_after_another_when_the_cache_is_small():
