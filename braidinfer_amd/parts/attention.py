@@ -12,6 +12,7 @@ config.rs:416).
 from __future__ import annotations
 
 import math
+import warnings
 from typing import Dict, List, Optional
 
 import torch
@@ -63,6 +64,7 @@ class GQAAttention(Mixer):
         self.w_qkv = self.w_o = None
         self._expects_tables = False       # set by check_positions when the model is put together
         self.force_simple = False          # tests set it to run the one-wave-per-query kernel in bf16
+        self._told_slow = False            # the notice below is given once per layer
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         return [
@@ -156,6 +158,12 @@ class GQAAttention(Mixer):
                                          ctx.block_table, ctx.storage, B, step.max_new, nq, nkv, hd,
                                          ctx.page_tokens, self.window, self.scale)
             return
+        if qkv.dtype == torch.bfloat16 and not self.force_simple and not self._told_slow:
+            # right, but an order of magnitude slower than the matrix-core kernels: said once, not silently
+            self._told_slow = True
+            warnings.warn(f"attention: head size {hd} with pages of {ctx.page_tokens} tokens is outside what the "
+                          "matrix-core attention kernels take (head sizes in steps of 16 up to 256, pages of 64 "
+                          "tokens); the one-wave-per-query kernel runs instead", RuntimeWarning, stacklevel=2)
         K.attention_simple(qkv, qkv.stride(0), o, step.positions, step.seq_of_token, step.slots,
                            ctx.block_table, ctx.storage, T, self.nq, self.nkv, self.hd, ctx.page_tokens,
                            self.window, self.scale)

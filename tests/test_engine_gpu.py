@@ -584,6 +584,31 @@ def test_wide_matrices_take_the_blocked_layout_by_themselves(tmp_path):
         close(np.stack([out[i], out2[i]]), r[-2:], "bfloat16", f"wide matrices, request {i} of 24")
 
 
+def test_a_head_size_outside_the_matrix_core_kernels_is_said_and_right(tmp_path):
+    """A head size that is no multiple of 16 is allowed; in bfloat16 its attention runs by the one-wave-per-query
+    kernel, which the engine says once per layer instead of slowing down silently; the logits are right."""
+    from conftest import TINY
+    cfg_d = dict(TINY["a"], head_dim=24)
+    folder = str(tmp_path / "m")
+    B.Engine.write_random_folder(folder, B.MistralConfig.from_dict(cfg_d), seed=4, std=0.08, vector_jitter=0.2)
+    cfg, w = P.read_folder(folder)
+    toks = tokens(cfg, 40, 3)
+    ref = P.forward(cfg, w, toks)
+    eng = B.Engine.from_folder(folder, dtype="bfloat16", max_tokens=512)
+    s = eng.alloc_slot()
+    with pytest.warns(RuntimeWarning, match="head size 24") as seen:
+        first = eng.step([StepEntry(s, toks[:30], list(range(30)))]).cpu().numpy()
+        rest = [eng.step([StepEntry(s, [t], [0])]).cpu().numpy() for t in toks[30:]]
+    eng.free_slot(s)
+    assert len([x for x in seen if "head size 24" in str(x.message)]) == cfg_d["num_hidden_layers"]
+    close(np.concatenate([first] + rest), ref, "bfloat16", "head size 24")
+    eng32 = B.Engine.from_folder(folder, dtype="float32", max_tokens=512)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")                        # the 32-bit path is that kernel by design: nothing to say
+        close(whole(eng32, toks), ref, "float32", "head size 24")
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
 def test_configurations_drawn_at_random(seed, tmp_path):
     """Sizes drawn at random (head sizes in steps of 16, groups of 1 to 6 heads, widths and vocabularies
